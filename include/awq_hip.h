@@ -1,0 +1,110 @@
+/* C ABI of libawq_hip.so -- the MI355X (gfx950) AWQ W4A16 linear path.
+ *
+ * Every pointer is a DEVICE pointer on the current HIP device unless said
+ * otherwise; `stream` is a hipStream_t passed as void* (NULL = default stream).
+ * Tensors are dense row-major:
+ *   qweight int32 [K, N/8]   nibble j of a word = logical column 8i + {0,2,4,6,1,3,5,7}[j]
+ *   qzeros  int32 [K/g, N/8] same nibble order
+ *   qscales f16|bf16 [K/g, N]
+ *   x       f16|bf16 [M, K]      y  f16|bf16 [M, N]     bias f16|bf16 [N] or NULL
+ * `dtype` is AWQ_F16 or AWQ_BF16 and names the type of x, qscales, bias and y.
+ * Inputs are borrowed and never written.  Calls are asynchronous on `stream`
+ * and return an awq_status; awq_hip_last_error() gives the message of the
+ * last failing call on the calling thread.
+ *
+ * Citations name the interface of the reference (liyuan24/nanoquantization)
+ * that an entry point stands in for.
+ */
+#ifndef AWQ_HIP_H_
+#define AWQ_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    AWQ_OK = 0,
+    AWQ_ERR_INVALID_ARG = 1,  /* null pointer, bad shape, bad dtype                       */
+    AWQ_ERR_UNSUPPORTED = 2,  /* a shape/group size this build has no kernel for          */
+    AWQ_ERR_WORKSPACE = 3,    /* workspace missing or smaller than *_workspace_bytes()    */
+    AWQ_ERR_HIP = 4           /* the HIP runtime refused the launch                       */
+} awq_status;
+
+typedef enum { AWQ_F16 = 0, AWQ_BF16 = 1 } awq_dtype;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int awq_hip_version(void);
+
+/* Message of the last failing call on this thread ("" if none). Host pointer, do not free. */
+const char* awq_hip_last_error(void);
+
+/* out[k, 8i+c] = RN_dtype(float(q - z) * s), bit-exact with the reference's
+ * dequantised weight.  out: dtype [K, N].
+ * Replaces awq_dequantize(qweight, qscales, qzeros) + awq_dequantize_kernel,
+ * nanoquantization/layers/gemm.py:126-180 and :10-123. */
+int awq_dequantize(const int32_t* qweight, const void* qscales, const int32_t* qzeros, void* out,
+                   int64_t K, int64_t N, int64_t group_size, int dtype, void* stream);
+
+/* Bytes of device workspace awq_gemv / awq_gemm / awq_linear need for this
+ * problem (0 is possible).  The workspace must be zero-filled ONCE when it is
+ * allocated; every call leaves it in that state (its counters are reset by
+ * the kernel), so it can be reused by later calls on the same stream.  Calls
+ * that share a workspace must not overlap in time. */
+size_t awq_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
+size_t awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* Decode regime, 1 <= M <= 16: y = x @ dequant(W) (+ bias), fp32 accumulation,
+ * split-K with a fixed-order (run-to-run bit-stable) reduction.
+ * Replaces awq_gemm(x, qweight, qscales, qzeros, split_k_iters) for small M:
+ * nanoquantization/layers/gemm.py:329-379 (kernel :183-326, torch.zeros :361,
+ * out.sum :378). */
+int awq_gemv(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+             const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
+             int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Prefill regime, any M >= 1 (meant for M > 16): fused dequant + MFMA GEMM,
+ * y = x @ dequant(W) (+ bias), W rounded to dtype exactly as the reference
+ * does before the product, fp32 accumulation.
+ * Replaces awq_dequantize + torch.matmul, nanoquantization/layers/gemm.py:559-561,
+ * and awq_gemm for 16 < M < 256, :562-564. */
+int awq_gemm(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+             const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
+             int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The whole forward of one AWQ linear: picks the regime from M (awq_gemv for
+ * M <= 16, awq_gemm above) and applies the bias.
+ * Replaces WQLinear_GEMM.forward, nanoquantization/layers/gemm.py:552-567
+ * (the reshape of x/y to 2-D stays with the caller). */
+int awq_linear(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+               const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
+               int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* awq_gemv / awq_gemm with the launch configuration forced, for tuning and for
+ * tests that must reach every compiled variant.  `variant` indexes the
+ * kernel-shape table (see awq_gemv_variant_count / awq_gemm_variant_count),
+ * `split_k` >= 1 is the number of K-splits across workgroups.  No reference
+ * counterpart (the reference exposes block sizes as keyword arguments of
+ * awq_gemm, nanoquantization/layers/gemm.py:334-337). */
+int awq_gemv_variant_count(void);
+int awq_gemm_variant_count(void);
+const char* awq_gemv_variant_name(int variant);
+const char* awq_gemm_variant_name(int variant);
+size_t awq_gemv_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k);
+size_t awq_gemm_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k);
+int awq_gemv_ex(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                int dtype, void* workspace, size_t workspace_bytes, void* stream, int variant,
+                int split_k);
+int awq_gemm_ex(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                int dtype, void* workspace, size_t workspace_bytes, void* stream, int variant,
+                int split_k);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AWQ_HIP_H_ */

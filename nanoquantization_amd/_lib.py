@@ -1,0 +1,98 @@
+"""ctypes binding of libawq_hip.so, the C ABI declared in include/awq_hip.h.
+
+There is no fallback: if the library is missing or a call fails, an exception
+is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "libawq_hip.so")
+
+AWQ_F16, AWQ_BF16 = 0, 1
+_STATUS = {1: "invalid argument", 2: "unsupported", 3: "workspace", 4: "HIP runtime"}
+
+_lib = None
+_lock = threading.Lock()
+
+_vp, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+_LINEAR_ARGS = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]
+
+# symbol -> (restype, argtypes); every symbol of include/awq_hip.h
+SYMBOLS = {
+    "awq_hip_version": (_int, []),
+    "awq_hip_last_error": (ctypes.c_char_p, []),
+    "awq_dequantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "awq_gemv_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "awq_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "awq_linear_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "awq_gemv": (_int, _LINEAR_ARGS),
+    "awq_gemm": (_int, _LINEAR_ARGS),
+    "awq_linear": (_int, _LINEAR_ARGS),
+    "awq_gemv_variant_count": (_int, []),
+    "awq_gemm_variant_count": (_int, []),
+    "awq_gemv_variant_name": (ctypes.c_char_p, [_int]),
+    "awq_gemm_variant_name": (ctypes.c_char_p, [_int]),
+    "awq_gemv_ex_workspace_bytes": (_sz, [_i64, _i64, _i64, _int, _int]),
+    "awq_gemm_ex_workspace_bytes": (_sz, [_i64, _i64, _i64, _int, _int]),
+    "awq_gemv_ex": (_int, _LINEAR_ARGS + [_int, _int]),
+    "awq_gemm_ex": (_int, _LINEAR_ARGS + [_int, _int]),
+}
+
+
+class AwqHipError(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise AwqHipError(
+                        f"{LIB_PATH} is missing: build it with `python -m nanoquantization_amd.build` "
+                        "(there is no CPU or eager fallback for the AWQ kernels)")
+                handle = ctypes.CDLL(LIB_PATH)
+                for name, (res, args) in SYMBOLS.items():
+                    fn = getattr(handle, name)
+                    fn.restype, fn.argtypes = res, args
+                _lib = handle
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        msg = lib().awq_hip_last_error().decode("utf-8", "replace")
+        raise AwqHipError(f"libawq_hip: {_STATUS.get(status, status)}: {msg}")
+
+
+def dtype_id(dtype: torch.dtype) -> int:
+    if dtype == torch.float16:
+        return AWQ_F16
+    if dtype == torch.bfloat16:
+        return AWQ_BF16
+    raise AwqHipError(f"qscales dtype must be float16 or bfloat16, got {dtype}")
+
+
+# One zero-initialised split-K workspace per (device, stream).  The kernels leave
+# it zeroed, and calls on one stream are ordered, so it is shared by every layer.
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def workspace(device: torch.device, stream_ptr: int, nbytes: int) -> torch.Tensor | None:
+    if nbytes == 0:
+        return None
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        size = max(nbytes, 8 << 20)
+        ws = torch.zeros(size, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws

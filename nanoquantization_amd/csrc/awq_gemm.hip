@@ -1,0 +1,485 @@
+// Kernel (c): prefill-regime fused dequant + GEMM on the 32x32x16 MFMA.
+//
+// A workgroup of 4 wavefronts owns a BM x BN output tile and walks K in steps
+// of BK = 64.  Per step it stages in LDS
+//   A: x[m0.., k0..k0+63]            copied as 16-byte chunks,
+//   B: W[k0..k0+63, n0..]^T          unpacked from the int4 words in registers,
+//                                    multiplied out to RN_dtype((q - z) * s) --
+//                                    the very values the reference's dequantise
+//                                    kernel produces -- and written k-contiguous,
+// both in [k-block of 8][row][8 x 16-bit] order so that one ds_read_b128 per
+// lane is one MFMA operand.  Slots are XOR-swizzled so neither the writers
+// (which hold 8 adjacent columns / 8 k-chunks of one row) nor the readers
+// (32 adjacent rows) pile onto one LDS bank.  Global loads for step i+1 are
+// issued before the MFMAs of step i and land in the other LDS buffer.
+//
+// The packed words are transposed in registers: a lane holds one word column
+// for UR consecutive k rows and emits, per output column, UR k-consecutive
+// values.  fp16 uses the packed-half magic (1024 + q) - (1024 + z), exact, then
+// one packed multiply by the scale; bf16 converts q to fp32 and uses one fma
+// q*s - z*s whose exact result needs no more than fp32's significand, then
+// packs two rows with a single round-to-nearest-even conversion.
+//
+// Split-K: as in the GEMV, fp32 partials + an arrival counter per tile; the
+// last workgroup adds the partials in split order.
+#include "awq_common.hpp"
+
+namespace awq {
+
+constexpr int kBK = 64;
+
+template <typename T>
+struct UnpackRows;
+
+// fp16: returns, for byte-pair i (columns 2i, 2i+1) of one word, the packed
+// pair of dequantised halves.
+template <>
+struct UnpackRows<F16> {
+    uint32_t zp[4];
+    f16x2 sc[4];
+    __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            zp[i] = ((zw >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            sc[i] = __builtin_bit_cast(f16x2, sv[i]);
+        }
+    }
+    // out[c] = (W[k, c], W[k+1, c]) for the 8 columns of the word pair (w0 = row k, w1 = row k+1)
+    __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t q0 = ((w0 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            uint32_t q1 = ((w1 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            f16x2 d0 = (__builtin_bit_cast(f16x2, q0) - __builtin_bit_cast(f16x2, zp[i])) * sc[i];
+            f16x2 d1 = (__builtin_bit_cast(f16x2, q1) - __builtin_bit_cast(f16x2, zp[i])) * sc[i];
+            uint32_t u0 = __builtin_bit_cast(uint32_t, d0), u1 = __builtin_bit_cast(uint32_t, d1);
+            // columns 2i (low halves) and 2i+1 (high halves), rows k / k+1
+            out[2 * i] = __builtin_amdgcn_perm(u1, u0, 0x05040100u);
+            out[2 * i + 1] = __builtin_amdgcn_perm(u1, u0, 0x07060302u);
+        }
+    }
+};
+
+template <>
+struct UnpackRows<BF16> {
+    float sc[8], nzs[8];  // s and -(z * s), both exact in fp32
+    __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t pr = sv[c >> 1];
+            sc[c] = __builtin_bit_cast(float, (c & 1) ? (pr & 0xFFFF0000u) : (pr << 16));
+            nzs[c] = -(float)((zw >> nibble_shift(c)) & 0xFu) * sc[c];
+        }
+    }
+    __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float q0 = (float)((w0 >> nibble_shift(c)) & 0xFu);
+            const float q1 = (float)((w1 >> nibble_shift(c)) & 0xFu);
+            // q*s - z*s: the exact value (q-z)*s has <= 13 significant bits, so the
+            // fused multiply-add returns it exactly.
+            out[c] = BF16::pack2(__builtin_fmaf(q0, sc[c], nzs[c]), __builtin_fmaf(q1, sc[c], nzs[c]));
+        }
+    }
+};
+
+// LDS slot (16-byte unit) of A row `row`, k-chunk `kc` (8 k's) inside a [8][BM] buffer
+template <int BM>
+__device__ __forceinline__ int a_slot(int row, int kc) { return kc * BM + (row ^ (2 * kc)); }
+
+// LDS slot of B column n = 8*wc + c, k-block kblk inside a [8][BN] buffer
+template <int BN>
+__device__ __forceinline__ int b_slot(int wc, int c, int kblk) {
+    return kblk * BN + ((wc >> 4) << 7) + (c << 4) + ((wc & 15) ^ (2 * c));
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(256) void gemm_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
+    int* __restrict__ counters, int M, int N, int K, int g, int iters_per_split, int splits) {
+    static_assert(WM * WN == 4, "4 wavefronts per workgroup");
+    static_assert(BN == 256 || BN == 128, "BN is 128 or 256");
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    static_assert(TM >= 1 && TN >= 1, "wave tile at least 32x32");
+    constexpr int UR = BN / 32;          // k rows per lane per step: 8 (BN=256) or 4 (BN=128)
+    constexpr int WCOLS = BN / 8;        // packed word columns per tile
+    constexpr int ACH = BM / 32;         // 16-byte A chunks per thread per step
+    constexpr int A_SLOTS = 8 * BM, B_SLOTS = 8 * BN;
+
+    extern __shared__ u32x4 lds[];  // [2][A_SLOTS + B_SLOTS]
+    __shared__ int s_last;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int split = blockIdx.z;
+    const int words = N >> 3;
+    const int total_iters = K / kBK;
+    const int it_begin = split * iters_per_split;
+    const int it_end = min(it_begin + iters_per_split, total_iters);
+
+    // B loader coordinates
+    const int wc = tid % WCOLS, rb = tid / WCOLS;  // word column, row block (UR rows)
+    const int gwc = (n0 >> 3) + wc;
+    const bool wc_ok = gwc < words;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+
+    u32x4 areg[ACH];
+    uint32_t wreg[UR];
+    uint32_t zreg;
+    u32x4 sreg;
+
+    auto load_global = [&](int it) {
+        const int k0 = it * kBK;
+#pragma unroll
+        for (int i = 0; i < ACH; ++i) {
+            const int id = tid + 256 * i;
+            const int row = id >> 3, kc = id & 7;
+            if (m0 + row < M)
+                areg[i] = *reinterpret_cast<const u32x4*>(x + (size_t)(m0 + row) * K + k0 + kc * 8);
+            else
+                areg[i] = u32x4{0u, 0u, 0u, 0u};
+        }
+        const int krow = k0 + rb * UR;
+        if (wc_ok) {
+#pragma unroll
+            for (int r = 0; r < UR; ++r) wreg[r] = qweight[(size_t)(krow + r) * words + gwc];
+            const int gi = krow / g;
+            zreg = qzeros[(size_t)gi * words + gwc];
+            sreg = *reinterpret_cast<const u32x4*>(scales + (size_t)gi * N + (size_t)gwc * 8);
+        } else {
+#pragma unroll
+            for (int r = 0; r < UR; ++r) wreg[r] = 0u;
+            zreg = 0u;
+            sreg = u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+
+    auto store_lds = [&](int buf) {
+        u32x4* abase = lds + buf * (A_SLOTS + B_SLOTS);
+        u32x4* bbase = abase + A_SLOTS;
+#pragma unroll
+        for (int i = 0; i < ACH; ++i) {
+            const int id = tid + 256 * i;
+            abase[a_slot<BM>(id >> 3, id & 7)] = areg[i];
+        }
+        UnpackRows<T> up;
+        up.set_group(zreg, sreg);
+        uint32_t cols[8][UR / 2];
+#pragma unroll
+        for (int rp = 0; rp < UR / 2; ++rp) {
+            uint32_t o[8];
+            up.pair(wreg[2 * rp], wreg[2 * rp + 1], o);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) cols[c][rp] = o[c];
+        }
+        if constexpr (UR == 8) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                bbase[b_slot<BN>(wc, c, rb)] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
+        } else {  // UR == 4: two lanes share a 16-byte slot, 8 bytes each
+            u32x2* b2 = reinterpret_cast<u32x2*>(bbase);
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                b2[b_slot<BN>(wc, c, rb >> 1) * 2 + (rb & 1)] = u32x2{cols[c][0], cols[c][1]};
+        }
+    };
+
+    const int li = lane & 31, kb2 = lane >> 5;
+    auto compute = [&](int buf) {
+        const u32x4* abase = lds + buf * (A_SLOTS + B_SLOTS);
+        const u32x4* bbase = abase + A_SLOTS;
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            const int kblk = ks * 2 + kb2;
+            u32x4 af[TM], bf[TN];
+#pragma unroll
+            for (int a = 0; a < TM; ++a) af[a] = abase[a_slot<BM>(wm0 + a * 32 + li, kblk)];
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                const int n = wn0 + b * 32 + li;
+                bf[b] = bbase[b_slot<BN>(n >> 3, n & 7, kblk)];
+            }
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b) acc[a][b] = T::mfma32(af[a], bf[b], acc[a][b]);
+        }
+    };
+
+    if (it_begin < it_end) {
+        load_global(it_begin);
+        store_lds(0);
+        __syncthreads();
+        for (int it = it_begin; it < it_end; ++it) {
+            const int buf = (it - it_begin) & 1;
+            const bool more = it + 1 < it_end;
+            if (more) load_global(it + 1);
+            compute(buf);
+            if (more) store_lds(buf ^ 1);
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue -----------------------------------------------------------
+    // acc[a][b][v]: row (v/4)*8 + kb2*4 + v%4, column li of the 32x32 tile
+    const bool direct = splits == 1;
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b) {
+            const int n = n0 + wn0 + b * 32 + li;
+            if (n >= N) continue;
+            float bv = 0.f;
+            if (direct && bias) bv = T::to_f32(bias[n]);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm0 + a * 32 + (v >> 2) * 8 + kb2 * 4 + (v & 3);
+                if (m >= M) continue;
+                if (direct)
+                    y[(size_t)m * N + n] = T::from_f32(acc[a][b][v] + bv);
+                else
+                    partials[((size_t)split * M + m) * N + n] = acc[a][b][v];
+            }
+        }
+    if (direct) return;
+
+    __threadfence();
+    __syncthreads();
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    if (tid == 0) {
+        const int prev = __hip_atomic_fetch_add(&counters[tile], 1, __ATOMIC_ACQ_REL,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == splits - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    const int rows = min(BM, M - m0);
+    const int wcount = min(WCOLS, words - (n0 >> 3));
+    for (int idx = tid; idx < rows * wcount; idx += 256) {
+        const int m = m0 + idx / wcount;
+        const size_t nn = (size_t)n0 + (size_t)(idx % wcount) * 8;
+        float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < splits; ++s) {
+            const float* p = partials + ((size_t)s * M + m) * N + nn;
+            const f32x4 u = *reinterpret_cast<const f32x4*>(p);
+            const f32x4 w = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                out[c] += u[c];
+                out[4 + c] += w[c];
+            }
+        }
+        if (bias) {
+            const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
+        }
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+        *reinterpret_cast<u32x4*>(y + (size_t)m * N + nn) = o;
+    }
+    if (tid == 0) counters[tile] = 0;
+}
+
+// ---- host side -------------------------------------------------------------
+struct GemmVariant {
+    const char* name;
+    int BM, BN;
+};
+static const GemmVariant kGemmVariants[] = {
+    {"256x256", 256, 256}, {"128x256", 128, 256}, {"128x128", 128, 128},
+    {"64x256", 64, 256},   {"32x256", 32, 256},   {"64x128", 64, 128},
+};
+constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
+
+template <typename T, int BM, int BN, int WM, int WN>
+static hipError_t launch_gemm(const void* x, const int32_t* qweight, const void* qscales,
+                              const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
+                              int g, void* workspace, int split_k, hipStream_t stream) {
+    const int tiles_m = (int)cdiv(M, BM), tiles_n = (int)cdiv(N, BN);
+    const int total_iters = K / kBK;
+    const int ips = (int)cdiv(total_iters, split_k);
+    const int splits = (int)cdiv(total_iters, ips);
+    int* counters = reinterpret_cast<int*>(workspace);
+    float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
+                                                            counter_bytes((int64_t)tiles_m * tiles_n))
+                                : nullptr;
+    const size_t lds = (size_t)2 * 8 * (BM + BN) * 16;
+    auto kern = gemm_kernel<T, BM, BN, WM, WN>;
+    if (lds > 64 * 1024) {
+        static bool raised = false;  // once per process and instantiation
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return e;
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(tiles_n, tiles_m, splits), dim3(256), lds, stream,
+                       reinterpret_cast<const uint16_t*>(x),
+                       reinterpret_cast<const uint32_t*>(qweight),
+                       reinterpret_cast<const uint16_t*>(qscales),
+                       reinterpret_cast<const uint32_t*>(qzeros),
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
+                       partials, counters, M, N, K, g, ips, splits);
+    return hipGetLastError();
+}
+
+static int gemm_effective_splits(int64_t K, int split_k) {
+    const int total = (int)(K / kBK);
+    const int ips = (int)cdiv(total, split_k);
+    return (int)cdiv(total, ips);
+}
+
+static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k) {
+    const GemmVariant& gv = kGemmVariants[variant];
+    const int splits = gemm_effective_splits(K, split_k);
+    if (splits <= 1) return 0;
+    return counter_bytes(cdiv(M, gv.BM) * cdiv(N, gv.BN)) + (size_t)splits * M * N * sizeof(float);
+}
+
+// Tile shape and split for the default entry point: the largest tile that still
+// yields at least one workgroup per CU, then split K until the chip is covered.
+static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
+    const int kCUs = 256;
+    int v;
+    if (M <= 32) v = 4;
+    else if (M <= 64) v = 3;
+    else {
+        v = 0;
+        if (cdiv(M, 256) * cdiv(N, 256) < kCUs) v = 1;
+        if (cdiv(M, 128) * cdiv(N, 256) < kCUs) v = 2;
+    }
+    const GemmVariant& gv = kGemmVariants[v];
+    const int64_t tiles = cdiv(M, gv.BM) * cdiv(N, gv.BN);
+    int64_t s = 1;
+    if (tiles < kCUs) s = kCUs / tiles;
+    const int64_t max_s = K / kBK / 4 > 0 ? K / kBK / 4 : 1;  // at least 4 K-steps per split
+    if (s > max_s) s = max_s;
+    if (s > 32) s = 32;
+    if (s < 1) s = 1;
+    *variant = v;
+    *split_k = (int)s;
+}
+
+static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, const void* qscales,
+                         const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
+                         int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
+                         void* stream, int variant, int split_k) {
+    int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
+    if (rc != AWQ_OK) return rc;
+    if (K % kBK != 0 || g % 8 != 0) {
+        set_error("%s: needs K %% 64 == 0 and group_size %% 8 == 0 (K=%lld, g=%lld)", fn,
+                  (long long)K, (long long)g);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    if (bias && (reinterpret_cast<uintptr_t>(bias) & 15u)) {
+        set_error("%s: bias must be 16-byte aligned", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    if (variant < 0 || variant >= kNumGemmVariants || split_k < 1) {
+        set_error("%s: bad variant %d / split_k %d", fn, variant, split_k);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    const GemmVariant& gv = kGemmVariants[variant];
+    if (cdiv(M, gv.BM) > 65535) {
+        set_error("%s: M=%lld exceeds the launch grid for tile %s", fn, (long long)M, gv.name);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    const size_t need = gemm_ws_bytes(M, N, K, variant, split_k);
+    if (need > 0 && (!workspace || workspace_bytes < need)) {
+        set_error("%s: workspace of %zu bytes needed, %zu given", fn, need, workspace ? workspace_bytes : (size_t)0);
+        return AWQ_ERR_WORKSPACE;
+    }
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    hipError_t e = hipErrorInvalidValue;
+#define AWQ_GEMM_CASE(IDX, BM_, BN_, WM_, WN_)                                                    \
+    case IDX:                                                                                     \
+        e = dtype == AWQ_F16                                                                      \
+                ? launch_gemm<F16, BM_, BN_, WM_, WN_>(x, qweight, qscales, qzeros, bias, y,      \
+                                                       (int)M, (int)N, (int)K, (int)g, workspace, \
+                                                       split_k, s)                                \
+                : launch_gemm<BF16, BM_, BN_, WM_, WN_>(x, qweight, qscales, qzeros, bias, y,     \
+                                                        (int)M, (int)N, (int)K, (int)g,           \
+                                                        workspace, split_k, s);                   \
+        break;
+    switch (variant) {
+        AWQ_GEMM_CASE(0, 256, 256, 2, 2)
+        AWQ_GEMM_CASE(1, 128, 256, 2, 2)
+        AWQ_GEMM_CASE(2, 128, 128, 2, 2)
+        AWQ_GEMM_CASE(3, 64, 256, 1, 4)
+        AWQ_GEMM_CASE(4, 32, 256, 1, 4)
+        AWQ_GEMM_CASE(5, 64, 128, 1, 4)
+    }
+#undef AWQ_GEMM_CASE
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+}  // namespace awq
+
+extern "C" int awq_gemm_variant_count(void) { return awq::kNumGemmVariants; }
+
+extern "C" const char* awq_gemm_variant_name(int variant) {
+    return (variant >= 0 && variant < awq::kNumGemmVariants) ? awq::kGemmVariants[variant].name : "";
+}
+
+extern "C" size_t awq_gemm_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant,
+                                              int split_k) {
+    if (variant < 0 || variant >= awq::kNumGemmVariants || split_k < 1 || K < awq::kBK || N < 8 || M < 1)
+        return 0;
+    return awq::gemm_ws_bytes(M, N, K, variant, split_k);
+}
+
+extern "C" size_t awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (K < awq::kBK || N < 8 || M < 1) return 0;
+    int v, s;
+    awq::pick_gemm(M, N, K, &v, &s);
+    return awq::gemm_ws_bytes(M, N, K, v, s);
+}
+
+extern "C" int awq_gemm_ex(const void* x, const int32_t* qweight, const void* qscales,
+                           const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
+                           int64_t K, int64_t group_size, int dtype, void* workspace,
+                           size_t workspace_bytes, void* stream, int variant, int split_k) {
+    return awq::gemm_dispatch("awq_gemm_ex", x, qweight, qscales, qzeros, bias, y, M, N, K,
+                              group_size, dtype, workspace, workspace_bytes, stream, variant,
+                              split_k);
+}
+
+extern "C" int awq_gemm(const void* x, const int32_t* qweight, const void* qscales,
+                        const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
+                        int64_t K, int64_t group_size, int dtype, void* workspace,
+                        size_t workspace_bytes, void* stream) {
+    int v = 0, s = 1;
+    if (K >= awq::kBK && N >= 8 && M >= 1) awq::pick_gemm(M, N, K, &v, &s);
+    return awq::gemm_dispatch("awq_gemm", x, qweight, qscales, qzeros, bias, y, M, N, K, group_size,
+                              dtype, workspace, workspace_bytes, stream, v, s);
+}
+
+extern "C" size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    return M <= 16 ? awq_gemv_workspace_bytes(M, N, K) : awq_gemm_workspace_bytes(M, N, K);
+}
+
+extern "C" int awq_linear(const void* x, const int32_t* qweight, const void* qscales,
+                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
+                          int64_t K, int64_t group_size, int dtype, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+    if (M >= 1 && M <= 16 && group_size % 32 == 0)
+        return awq_gemv(x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, workspace,
+                        workspace_bytes, stream);
+    return awq_gemm(x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, workspace,
+                    workspace_bytes, stream);
+}

@@ -1,0 +1,98 @@
+"""Kernel (c): fused dequant + MFMA GEMM through the C ABI against the fp32-accumulation oracle."""
+import numpy as np
+import pytest
+import torch
+
+import nanoquantization_amd as nq
+from nanoquantization_amd import _lib
+from nanoquantization_amd.layers.gemm import awq_gemm_variant
+from conftest import make_case, make_x, random_packed, to_bits, to_dev
+from oracle import awq_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+TIGHT = {"f16": 1.5e-3, "bf16": 6e-3}
+
+
+def _check(y, xb, p, dtype, bias=None):
+    ref = o.linear_fp32(xb, p["qweight"], p["qzeros"], p["qscales"], dtype, bias)
+    err = o.max_rel_err(o.from_bits16(to_bits(y), dtype), ref)
+    assert err <= TOL, f"max rel err {err}"
+    assert err <= TIGHT[dtype], f"max rel err {err}"
+    return err
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_every_variant_and_split(dtype):
+    L = _lib.lib()
+    K, N = 512, 520            # N not a multiple of any tile: exercises the column masks
+    p = random_packed(K, N, 128, dtype, seed=60)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    for M in (17, 128, 300):
+        xb = make_x(M, K, dtype, seed=61 + M)
+        xd = to_dev(xb, dtype)
+        for v in range(L.awq_gemm_variant_count()):
+            for split in (1, 3):
+                print(f"gemm variant {L.awq_gemm_variant_name(v).decode()} split={split} M={M} {dtype}", flush=True)
+                y = awq_gemm_variant(xd, *dev, v, split)
+                torch.cuda.synchronize()
+                _check(y, xb, p, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,K,N,g", [(32, 1024, 3072, 128), (64, 3072, 1024, 128), (256, 1024, 2048, 32),
+                                      (512, 4096, 1024, 128), (130, 256, 8, 64), (1000, 2048, 264, 128)])
+def test_gemm_default_dispatch(dtype, M, K, N, g):
+    print(f"gemm default {dtype} M={M} K={K} N={N} g={g}", flush=True)
+    p = make_case(K, N, g, dtype, seed=M + K)
+    xb = make_x(M, K, dtype, seed=M)
+    y = nq.awq_gemm(to_dev(xb, dtype), to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"]), 8)
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (M, N)
+    _check(y, xb, p, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_equals_dequant_then_matmul(dtype):
+    # the reference's M >= 256 branch: awq_dequantize + torch.matmul (layers/gemm.py:559-561); the fused
+    # kernel multiplies the very same rounded weights, so it must agree with that path to fp32-sum accuracy
+    print(f"gemm vs dequant+matmul {dtype}", flush=True)
+    M, K, N = 384, 1024, 1024
+    p = make_case(K, N, 128, dtype, seed=70)
+    xb = make_x(M, K, dtype, seed=71)
+    qw, qs, qz = to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])
+    xd = to_dev(xb, dtype)
+    w = nq.awq_dequantize(qw, qs, qz)
+    y_unfused = torch.matmul(xd.float(), w.float())
+    y = nq.awq_gemm(xd, qw, qs, qz, 8)
+    err = (y.float() - y_unfused).abs().max().item() / y_unfused.abs().max().item()
+    assert err <= (1e-3 if dtype == "f16" else 5e-3), err
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_bias_and_determinism(dtype):
+    print(f"gemm bias {dtype}", flush=True)
+    M, K, N = 200, 1024, 512
+    p = make_case(K, N, 128, dtype, seed=80)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    xb = make_x(M, K, dtype, seed=81)
+    xd = to_dev(xb, dtype)
+    bias = np.linspace(-2, 2, N).astype(np.float32)
+    for split in (1, 4):
+        y = awq_gemm_variant(xd, *dev, 2, split, bias=to_dev(o.to_bits16(bias, dtype), dtype))
+        _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
+    y1 = awq_gemm_variant(xd, *dev, 2, 4)
+    y2 = awq_gemm_variant(xd, *dev, 2, 4)
+    assert torch.equal(y1, y2)
+    assert torch.count_nonzero(awq_gemm_variant(torch.zeros_like(xd), *dev, 2, 4)) == 0
+
+
+def test_gemm_prefill_full_size_bf16():
+    # Qwen3-8B MLP gate/up at M=512, its real size (oracle: numpy float64 matmul, a few seconds)
+    print("gemm full size M=512 4096x12288 bf16", flush=True)
+    M, K, N = 512, 4096, 12288
+    p = random_packed(K, N, 128, "bf16", seed=90)
+    xb = make_x(M, K, "bf16", seed=91)
+    y = nq.awq_gemm(to_dev(xb, "bf16"), to_dev(p["qweight"]), to_dev(p["qscales"], "bf16"), to_dev(p["qzeros"]), 8)
+    _check(y, xb, p, "bf16")

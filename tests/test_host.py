@@ -1,0 +1,132 @@
+"""CPU-side checks of the product: the host mirror of the reference interface against the oracle, the
+module contract, and that the C-ABI library loads and exports every declared symbol (no compute)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import nanoquantization_amd as nq
+from nanoquantization_amd import _lib
+from nanoquantization_amd.layers.gemm import pack_awq
+from oracle import awq_oracle as o
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _ensure_built():
+    if not os.path.exists(_lib.LIB_PATH):
+        from nanoquantization_amd.build import build
+        build(verbose=False)
+
+
+def test_library_exports_every_declared_symbol():
+    _ensure_built()
+    header = open(os.path.join(ROOT, "include", "awq_hip.h")).read()
+    declared = set(re.findall(r"\b(awq_[a-z0-9_]+)\s*\(", header))
+    declared -= {"awq_status", "awq_dtype"}
+    assert declared, "no declarations parsed"
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in sorted(declared):
+        assert hasattr(handle, name), f"{name} declared in include/awq_hip.h but not exported"
+    assert declared == set(_lib.SYMBOLS), "ctypes table and header disagree"
+    L = _lib.lib()
+    assert L.awq_hip_version() >= 100
+    assert L.awq_gemv_variant_count() >= 1 and L.awq_gemm_variant_count() >= 1
+    assert L.awq_gemv_variant_name(0)
+    # argument validation happens before anything touches a device
+    rc = L.awq_gemv(None, None, None, None, None, None, 1, 8, 128, 128, 0, None, 0, None)
+    assert rc == 1 and b"null pointer" in L.awq_hip_last_error()
+    # the published packed-weight workspace rule: 0 bytes when there is nothing to split
+    assert L.awq_gemv_ex_workspace_bytes(1, 1024, 1024, 0, 1) == 0
+    assert L.awq_gemv_ex_workspace_bytes(4, 1024, 1024, 0, 4) == 256 + 4 * 4 * 1024 * 4
+
+
+def test_pseudo_quantize_matches_oracle_bitwise():
+    torch.manual_seed(0)
+    w = torch.randn(96, 512) * 0.02
+    dq, s, z = nq.pseudo_quantize(w, 128, 4, True)
+    odq, os_, oz = o.quantize_minmax(w.numpy(), 128)
+    assert (dq.numpy() == odq).all() and (s.numpy() == os_).all() and (z.numpy() == oz).all()
+    assert dq.shape == w.shape and s.shape == (96, 4) and z.shape == (96, 4)
+    dq, s, z = nq.pseudo_quantize(w, 64, 4, False)
+    odq, os_, oz = o.quantize_minmax(w.numpy(), 64, 4, False)
+    assert z is None and oz is None and (dq.numpy() == odq).all() and (s.numpy() == os_).all()
+    wh = w.half()
+    dq, s, z = nq.pseudo_quantize(wh, 32, 4, True)
+    odq, os_, oz = o.quantize_minmax(wh.numpy(), 32)
+    assert dq.dtype == torch.float16 and (dq.numpy() == odq).all() and (z.numpy() == oz).all()
+
+
+def test_pseudo_quantize_rejects_nan_and_bad_group():
+    w = torch.randn(4, 128)
+    w[0, 0] = float("nan")
+    with pytest.raises(AssertionError):
+        nq.pseudo_quantize(w, 128, 4, True)
+    with pytest.raises(AssertionError):
+        nq.pseudo_quantize(torch.randn(4, 100), 128, 4, True)
+
+
+@pytest.mark.parametrize("dt,tdt", [("f16", torch.float16), ("bf16", torch.bfloat16)])
+@pytest.mark.parametrize("g", [32, 128])
+def test_from_linear_matches_oracle_words(dt, tdt, g):
+    torch.manual_seed(1)
+    N, K = 72, 256
+    w = torch.randn(N, K) * 0.02
+    dq, s, z = nq.pseudo_quantize(w, g, 4, True)
+    lin = torch.nn.Linear(K, N, bias=True)
+    lin.weight.data = dq
+    m = nq.WQLinear_GEMM.from_linear(lin, 4, g, s.t().contiguous(), z.t().contiguous(), tdt)
+    p = o.make_packed(w.numpy(), g, dt)
+    assert m.qweight.dtype == torch.int32 and tuple(m.qweight.shape) == (K, N // 8)
+    assert (m.qweight.numpy() == p["qweight"]).all()
+    assert (m.qzeros.numpy() == p["qzeros"]).all()
+    assert m.qscales.dtype == tdt
+    assert (m.qscales.view(torch.int16).numpy().view(np.uint16) == p["qscales"]).all()
+    assert m.bias is not None and m.bias.dtype == tdt and m.bias.shape == (N,)
+
+
+def test_pack_known_words_and_sign():
+    v = torch.tensor([[0, 1, 2, 3, 4, 5, 6, 7], [8, 9, 10, 11, 12, 13, 14, 15], [15] * 8, [0, 1, 0, 0, 0, 0, 0, 0]])
+    assert pack_awq(v).flatten().tolist() == [1966171168, -38146904, -1, 0x00010000]
+    assert pack_awq(v).dtype == torch.int32
+
+
+def test_module_contract():
+    m = nq.WQLinear_GEMM(4, 128, 1024, 3072)
+    assert m.qweight.shape == (1024, 384) and m.qweight.dtype == torch.int32
+    assert m.qscales.shape == (8, 3072) and m.qscales.dtype == torch.bfloat16
+    assert m.qzeros.shape == (8, 384) and m.qzeros.dtype == torch.int32
+    assert m.bias is None
+    assert set(dict(m.named_buffers())) == {"qweight", "qscales", "qzeros"}
+    assert (m.w_bits, m.group_size, m.in_features, m.out_features) == (4, 128, 1024, 3072)
+    mb = nq.WQLinear_GEMM(4, 128, 256, 64, bias=True, output_dtype=torch.float16)
+    assert mb.bias.dtype == torch.bfloat16 and mb.qscales.dtype == torch.float16
+    assert "bias" in dict(mb.named_buffers())
+    with pytest.raises(ValueError):
+        nq.WQLinear_GEMM(8, 128, 256, 64)
+    with pytest.raises(AssertionError):
+        nq.WQLinear_GEMM(4, 128, 200, 64)
+    with pytest.raises(AssertionError):
+        nq.WQLinear_GEMM(4, 128, 256, 60)
+    # state_dict keys are the checkpoint contract
+    assert list(m.state_dict()) == ["qweight", "qscales", "qzeros"]
+
+
+def test_no_cpu_fallback():
+    m = nq.WQLinear_GEMM(4, 128, 256, 64, output_dtype=torch.float16)
+    with pytest.raises(_lib.AwqHipError):
+        m(torch.randn(2, 256, dtype=torch.float16))
+    with pytest.raises(_lib.AwqHipError):
+        nq.awq_dequantize(m.qweight, m.qscales, m.qzeros)
+
+
+def test_product_does_not_import_oracle():
+    pkg = os.path.join(ROOT, "nanoquantization_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"

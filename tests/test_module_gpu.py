@@ -1,0 +1,56 @@
+"""WQLinear_GEMM.forward on the GPU: shapes, dtype, bias, regime switch, state_dict round trip."""
+import numpy as np
+import pytest
+import torch
+
+import nanoquantization_amd as nq
+from conftest import to_bits
+from oracle import awq_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def _module(K, N, g, tdt, bias, seed=0):
+    torch.manual_seed(seed)
+    w = torch.randn(N, K) * 0.02
+    dq, s, z = nq.pseudo_quantize(w, g, 4, True)
+    lin = torch.nn.Linear(K, N, bias=bias)
+    lin.weight.data = dq
+    return nq.WQLinear_GEMM.from_linear(lin, 4, g, s.t().contiguous(), z.t().contiguous(), tdt).to("cuda")
+
+
+@pytest.mark.parametrize("tdt,dt", [(torch.float16, "f16"), (torch.bfloat16, "bf16")])
+@pytest.mark.parametrize("bias", [False, True])
+def test_forward_matches_oracle_all_regimes(tdt, dt, bias):
+    K, N, g = 1024, 3072, 128
+    m = _module(K, N, g, tdt, bias)
+    qw, qz = m.qweight.cpu().numpy(), m.qzeros.cpu().numpy()
+    qs = to_bits(m.qscales)
+    b = m.bias.float().cpu().numpy() if bias else None
+    for shape in [(16, K), (1, K), (2, 3, K), (4, 40, K), (300, K)]:   # cfg1 is the first
+        print(f"forward {dt} bias={bias} x{shape}", flush=True)
+        torch.manual_seed(sum(shape))
+        x = torch.randn(*shape).to(tdt).cuda()
+        y = m(x)
+        assert y.shape == x.shape[:-1] + (N,) and y.dtype == tdt
+        ref = o.linear_fp32(to_bits(x.reshape(-1, K)), qw, qz, qs, dt, b)
+        err = o.max_rel_err(y.float().cpu().numpy().reshape(-1, N), ref)
+        assert err <= 1e-2 and err <= (1.5e-3 if dt == "f16" else 6e-3), err
+
+
+def test_forward_casts_x_to_scale_dtype():
+    # the reference's test runs fp16 activations through bf16 scales: x is cast on load (layers/gemm.py:259)
+    m = _module(512, 256, 128, torch.bfloat16, False)
+    x = torch.randn(8, 512, dtype=torch.float16, device="cuda")
+    y = m(x)
+    assert y.dtype == torch.bfloat16
+    assert torch.equal(y, m(x.to(torch.bfloat16)))
+
+
+def test_state_dict_roundtrip_keeps_outputs():
+    m = _module(512, 256, 128, torch.float16, True)
+    m2 = nq.WQLinear_GEMM(4, 128, 512, 256, bias=True, output_dtype=torch.float16)
+    m2.load_state_dict({k: v.cpu() for k, v in m.state_dict().items()})
+    m2 = m2.to("cuda")
+    x = torch.randn(5, 512, dtype=torch.float16, device="cuda")
+    assert torch.equal(m(x), m2(x))
