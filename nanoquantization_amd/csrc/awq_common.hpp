@@ -19,6 +19,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kWave = 64;
 
+// Reinterpret one 32-bit register as a pair of halves.  Takes the word BY VALUE:
+// __builtin_bit_cast applied directly to a vector element (v[i]) reads element 0.
+__device__ __forceinline__ f16x2 as_f16x2(uint32_t w) { return __builtin_bit_cast(f16x2, w); }
+__device__ __forceinline__ uint32_t as_u32(f16x2 h) { return __builtin_bit_cast(uint32_t, h); }
+
 // Bit position of logical column c inside a packed word: the packer stores
 // column {0,2,4,6,1,3,5,7}[j] in nibble j, so column c sits at nibble
 // 4*(c&1) + (c>>1).
@@ -76,6 +81,31 @@ struct BF16 {
     }
 };
 
+// ---- split-K exchange between workgroups ----------------------------------
+// Partials cross workgroups (and XCDs, each with its own L2) as agent-scope
+// relaxed atomic stores/loads: they are written through to, and read from, the
+// agent's point of coherence, so no cache write-back or invalidate -- which
+// costs every wave of the grid a serialised L2 operation -- is needed.
+__device__ __forceinline__ void publish_f32(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float fetch_f32(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// All of this workgroup's publish_f32 stores have been acknowledged (vmcnt = 0
+// in every wave, then the barrier) before one thread bumps the tile's arrival
+// counter; returns true in the workgroup that arrived last.
+__device__ __forceinline__ bool arrive_last(int* counter, int splits, int* s_flag) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int prev = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_flag = (prev == splits - 1);
+    }
+    __syncthreads();
+    return *s_flag != 0;
+}
+
 // ---- host-side error plumbing -------------------------------------------
 void set_error(const char* fmt, ...);
 int check_linear_args(const char* fn, const void* x, const int32_t* qweight, const void* qscales,
@@ -86,9 +116,12 @@ int hip_fail(const char* fn, hipError_t e);
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Split-K bookkeeping shared by the GEMV and GEMM kernels.  The workspace is
-//   [ int32 counters, one per output tile, padded to 256 B | fp32 partials ]
-// Counters start at zero and the last workgroup to arrive at a tile resets its
-// counter, so the buffer is reusable without a memset between calls.
-static inline size_t counter_bytes(int64_t tiles) { return (size_t)cdiv(tiles * 4, 256) * 256; }
+//   [ kMaxSplitTiles int32 arrival counters | fp32 partials [splits][M][N] ]
+// The counter region has the same size for every problem, so partials of one
+// call never land on counters of the next.  Counters start at zero and the last
+// workgroup to arrive at a tile resets its counter: the buffer is reusable
+// without a memset between calls.
+constexpr int64_t kMaxSplitTiles = 4096;
+constexpr size_t kCounterBytes = (size_t)kMaxSplitTiles * sizeof(int);
 
 }  // namespace awq

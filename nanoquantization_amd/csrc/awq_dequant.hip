@@ -24,7 +24,7 @@ struct DequantWord<F16> {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             zp[i] = ((zw >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            sc[i] = __builtin_bit_cast(f16x2, sv[i]);
+            sc[i] = as_f16x2(sv[i]);
         }
     }
     __device__ __forceinline__ u32x4 apply(uint32_t w) const {
@@ -32,8 +32,8 @@ struct DequantWord<F16> {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             uint32_t qp = ((w >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            f16x2 d = __builtin_bit_cast(f16x2, qp) - __builtin_bit_cast(f16x2, zp[i]);
-            o[i] = __builtin_bit_cast(uint32_t, (f16x2)(d * sc[i]));
+            f16x2 d = as_f16x2(qp) - as_f16x2(zp[i]);
+            o[i] = as_u32(d * sc[i]);
         }
         return o;
     }
@@ -72,24 +72,22 @@ template <typename T, int ROWS>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint32_t* __restrict__ qweight,
                                                       const uint16_t* __restrict__ scales,
                                                       const uint32_t* __restrict__ qzeros,
-                                                      uint16_t* __restrict__ out, int K, int words,
-                                                      int g) {
+                                                      uint16_t* __restrict__ out, int words, int g) {
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= words) return;
     const int k0 = blockIdx.y * ROWS;
-    const int gi = k0 / g;  // host guarantees g % ROWS == 0: all ROWS rows share a group
+    // host guarantees g % ROWS == 0 (all ROWS rows share a group) and hence K % ROWS == 0
+    const int gi = k0 / g;
     const size_t N = (size_t)words * 8;
     DequantWord<T> dq;
     dq.set_group(qzeros[(size_t)gi * words + c],
                  *reinterpret_cast<const u32x4*>(scales + (size_t)gi * N + (size_t)c * 8));
     uint32_t w[ROWS];
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) w[r] = (k0 + r < K) ? qweight[(size_t)(k0 + r) * words + c] : 0u;
+    for (int r = 0; r < ROWS; ++r) w[r] = qweight[(size_t)(k0 + r) * words + c];
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        if (k0 + r < K)
-            *reinterpret_cast<u32x4*>(out + (size_t)(k0 + r) * N + (size_t)c * 8) = dq.apply(w[r]);
-    }
+    for (int r = 0; r < ROWS; ++r)
+        *reinterpret_cast<u32x4*>(out + (size_t)(k0 + r) * N + (size_t)c * 8) = dq.apply(w[r]);
 }
 
 template <typename T>
@@ -103,12 +101,10 @@ static int launch_dequant(const int32_t* qweight, const void* qscales, const int
     auto o = reinterpret_cast<uint16_t*>(out);
     if (g % 16 == 0) {
         dim3 grid((unsigned)cdiv(words, 256), (unsigned)cdiv(K, 16));
-        hipLaunchKernelGGL((dequant_kernel<T, 16>), grid, block, 0, stream, qw, sc, qz, o, (int)K,
-                           words, (int)g);
+        hipLaunchKernelGGL((dequant_kernel<T, 16>), grid, block, 0, stream, qw, sc, qz, o, words, (int)g);
     } else {
         dim3 grid((unsigned)cdiv(words, 256), (unsigned)K);
-        hipLaunchKernelGGL((dequant_kernel<T, 1>), grid, block, 0, stream, qw, sc, qz, o, (int)K,
-                           words, (int)g);
+        hipLaunchKernelGGL((dequant_kernel<T, 1>), grid, block, 0, stream, qw, sc, qz, o, words, (int)g);
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail("awq_dequantize", e);

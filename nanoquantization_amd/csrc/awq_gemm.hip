@@ -41,7 +41,7 @@ struct UnpackRows<F16> {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             zp[i] = ((zw >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            sc[i] = __builtin_bit_cast(f16x2, sv[i]);
+            sc[i] = as_f16x2(sv[i]);
         }
     }
     // out[c] = (W[k, c], W[k+1, c]) for the 8 columns of the word pair (w0 = row k, w1 = row k+1)
@@ -50,9 +50,9 @@ struct UnpackRows<F16> {
         for (int i = 0; i < 4; ++i) {
             uint32_t q0 = ((w0 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
             uint32_t q1 = ((w1 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            f16x2 d0 = (__builtin_bit_cast(f16x2, q0) - __builtin_bit_cast(f16x2, zp[i])) * sc[i];
-            f16x2 d1 = (__builtin_bit_cast(f16x2, q1) - __builtin_bit_cast(f16x2, zp[i])) * sc[i];
-            uint32_t u0 = __builtin_bit_cast(uint32_t, d0), u1 = __builtin_bit_cast(uint32_t, d1);
+            f16x2 d0 = (as_f16x2(q0) - as_f16x2(zp[i])) * sc[i];
+            f16x2 d1 = (as_f16x2(q1) - as_f16x2(zp[i])) * sc[i];
+            uint32_t u0 = as_u32(d0), u1 = as_u32(d1);
             // columns 2i (low halves) and 2i+1 (high halves), rows k / k+1
             out[2 * i] = __builtin_amdgcn_perm(u1, u0, 0x05040100u);
             out[2 * i + 1] = __builtin_amdgcn_perm(u1, u0, 0x07060302u);
@@ -248,22 +248,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(
                 if (direct)
                     y[(size_t)m * N + n] = T::from_f32(acc[a][b][v] + bv);
                 else
-                    partials[((size_t)split * M + m) * N + n] = acc[a][b][v];
+                    publish_f32(&partials[((size_t)split * M + m) * N + n], acc[a][b][v]);
             }
         }
     if (direct) return;
 
-    __threadfence();
-    __syncthreads();
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
-    if (tid == 0) {
-        const int prev = __hip_atomic_fetch_add(&counters[tile], 1, __ATOMIC_ACQ_REL,
-                                                __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == splits - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
+    if (!arrive_last(&counters[tile], splits, &s_last)) return;
     const int rows = min(BM, M - m0);
     const int wcount = min(WCOLS, words - (n0 >> 3));
     for (int idx = tid; idx < rows * wcount; idx += 256) {
@@ -272,13 +263,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         for (int s = 0; s < splits; ++s) {
             const float* p = partials + ((size_t)s * M + m) * N + nn;
-            const f32x4 u = *reinterpret_cast<const f32x4*>(p);
-            const f32x4 w = *reinterpret_cast<const f32x4*>(p + 4);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                out[c] += u[c];
-                out[4 + c] += w[c];
-            }
+            for (int c = 0; c < 8; ++c) out[c] += fetch_f32(p + c);
         }
         if (bias) {
             const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);
@@ -291,7 +277,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(
         for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
         *reinterpret_cast<u32x4*>(y + (size_t)m * N + nn) = o;
     }
-    if (tid == 0) counters[tile] = 0;
+    if (tid == 0) __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- host side -------------------------------------------------------------
@@ -315,7 +301,7 @@ static hipError_t launch_gemm(const void* x, const int32_t* qweight, const void*
     const int splits = (int)cdiv(total_iters, ips);
     int* counters = reinterpret_cast<int*>(workspace);
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
-                                                            counter_bytes((int64_t)tiles_m * tiles_n))
+                                                            kCounterBytes)
                                 : nullptr;
     const size_t lds = (size_t)2 * 8 * (BM + BN) * 16;
     auto kern = gemm_kernel<T, BM, BN, WM, WN>;
@@ -348,7 +334,7 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
     const GemmVariant& gv = kGemmVariants[variant];
     const int splits = gemm_effective_splits(K, split_k);
     if (splits <= 1) return 0;
-    return counter_bytes(cdiv(M, gv.BM) * cdiv(N, gv.BN)) + (size_t)splits * M * N * sizeof(float);
+    return kCounterBytes + (size_t)splits * M * N * sizeof(float);
 }
 
 // Tile shape and split for the default entry point: the largest tile that still
@@ -397,6 +383,11 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     const GemmVariant& gv = kGemmVariants[variant];
     if (cdiv(M, gv.BM) > 65535) {
         set_error("%s: M=%lld exceeds the launch grid for tile %s", fn, (long long)M, gv.name);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    if (gemm_effective_splits(K, split_k) > 1 && cdiv(M, gv.BM) * cdiv(N, gv.BN) > kMaxSplitTiles) {
+        set_error("%s: split-K supports at most %lld output tiles (M=%lld N=%lld tile %s)", fn,
+                  (long long)kMaxSplitTiles, (long long)M, (long long)N, gv.name);
         return AWQ_ERR_UNSUPPORTED;
     }
     const size_t need = gemm_ws_bytes(M, N, K, variant, split_k);

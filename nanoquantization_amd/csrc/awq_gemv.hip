@@ -61,137 +61,130 @@ __device__ __forceinline__ uint32_t vget(const typename WordVec<V>::type& v, int
     if constexpr (V == 1) return v; else return v[i];
 }
 
-template <int V>
-struct StepData {
-    typename WordVec<V>::type w[8];  // 8 rows x V words
-    u32x4 xa;                        // A operand: x[m = j][k0 + 8kb .. +7]
+// One chunk = CH steps of 32 rows inside one quantisation group.
+template <int V, int CH>
+struct Chunk {
+    typename WordVec<V>::type w[CH][8];  // per step: 8 rows x V words
+    u32x4 xa[CH];                        // per step: A operand x[m = j][k0 + 8kb .. +7]
+    typename WordVec<V>::type zw;        // V zero words of the group
+    u32x4 sv[V];                         // 8 scales per word
 };
 
-template <int V>
-struct GroupData {
-    typename WordVec<V>::type zw;  // V zero words
-    u32x4 sv[V];                   // 8 scales per word
-};
-
-template <typename T, int V, int WAVES>
+template <typename T, int V, int WAVES, int CH, bool PF>
 __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
-    int* __restrict__ counters, int M, int N, int K, int g, int steps_per_split, int splits) {
+    int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
+    int splits) {
     using WV = typename WordVec<V>::type;
     constexpr int NF = 8 * V;  // column fragments per lane
     extern __shared__ float red[];  // [WAVES][NF*4][64]
     __shared__ int s_last;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
+    const int wstride = words / V;  // row stride in WV units (host guarantees words % V == 0)
     const int tile = blockIdx.x, split = blockIdx.y;
-    const int c0 = (tile * 16 + j) * V;
-    const bool col_ok = c0 < words;  // words % V == 0, so all V words are in or out together
+    const int wv_col = tile * 16 + j;        // this lane's column in WV units
+    const bool col_ok = wv_col < wstride;
+    // lanes past the last column (and A rows past M) read a valid neighbour instead of
+    // branching; whatever they compute is never stored
+    const int wv_ld = col_ok ? wv_col : wstride - 1;
+    const int xrow = j < M ? j : 0;
 
-    const int total_steps = K >> 5;
-    const int s_begin = split * steps_per_split;
-    const int s_end = min(s_begin + steps_per_split, total_steps);
-    const int per_wave = (max(s_end - s_begin, 0) + WAVES - 1) / WAVES;
-    const int t0 = s_begin + wave * per_wave;
-    const int t1 = min(t0 + per_wave, s_end);
-    const int steps_per_group = g >> 5;  // host guarantees g % 32 == 0
+    const int total_chunks = K / (32 * CH);
+    const int c_begin = split * chunks_per_split;
+    const int c_end = min(c_begin + chunks_per_split, total_chunks);
+    const int per_wave = (max(c_end - c_begin, 0) + WAVES - 1) / WAVES;
+    const int c0 = c_begin + wave * per_wave;
+    const int c1 = min(c0 + per_wave, c_end);
 
-    f32x4 acc[NF], dg[NF], dones;
+    const WV* wlane = reinterpret_cast<const WV*>(qweight) + (size_t)(kb * 8) * wstride + wv_ld;
+    const WV* zlane = reinterpret_cast<const WV*>(qzeros) + wv_ld;
+    const u32x4* slane = reinterpret_cast<const u32x4*>(scales) + (size_t)wv_ld * V;
+    const uint16_t* xlane = x + (size_t)xrow * K + kb * 8;
+
+    f32x4 acc[NF];
 #pragma unroll
     for (int f = 0; f < NF; ++f) acc[f] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto load_step = [&](int t, StepData<V>& d) {
-        const int kbase = t * 32 + kb * 8;
+    auto load_chunk = [&](int c, Chunk<V, CH>& d) {
+        const int row0 = c * (32 * CH);  // wave-uniform
+        const WV* wp = wlane + (size_t)row0 * wstride;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            if (col_ok)
-                d.w[r] = *reinterpret_cast<const WV*>(qweight + (size_t)(kbase + r) * words + c0);
-            else
-                d.w[r] = WV{};
-        }
-        if (j < M)
-            d.xa = *reinterpret_cast<const u32x4*>(x + (size_t)j * K + kbase);
-        else
-            d.xa = u32x4{0u, 0u, 0u, 0u};
+        for (int s = 0; s < CH; ++s)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) d.w[s][r] = wp[(size_t)(s * 32 + r) * wstride];
+#pragma unroll
+        for (int s = 0; s < CH; ++s) d.xa[s] = *reinterpret_cast<const u32x4*>(xlane + row0 + s * 32);
+        const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
+        d.zw = zlane[(size_t)gi * wstride];
+#pragma unroll
+        for (int v = 0; v < V; ++v) d.sv[v] = slane[(size_t)gi * words + v];
     };
-    auto load_group = [&](int gi, GroupData<V>& gd) {
-        if (col_ok) {
-            gd.zw = *reinterpret_cast<const WV*>(qzeros + (size_t)gi * words + c0);
+
+    const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
+    const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto compute_chunk = [&](const Chunk<V, CH>& d) {
+        f32x4 dones = zero4;
 #pragma unroll
-            for (int v = 0; v < V; ++v)
-                gd.sv[v] = *reinterpret_cast<const u32x4*>(scales + (size_t)gi * N +
-                                                           (size_t)(c0 + v) * 8);
-        } else {
-            gd.zw = WV{};
-#pragma unroll
-            for (int v = 0; v < V; ++v) gd.sv[v] = u32x4{0u, 0u, 0u, 0u};
-        }
-    };
-    // acc += s * (dg - (16 + z) * dones), one group's worth
-    auto flush = [&](const GroupData<V>& gd) {
+        for (int s = 0; s < CH; ++s) dones = T::mfma16(d.xa[s], ones, dones);
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            const uint32_t zw = vget<V>(gd.zw, v);
+            const uint32_t zw = vget<V>(d.zw, v);
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const float zf = (float)(((zw >> nibble_shift(c)) & 0xFu) | 16u);
-                const uint32_t pair = gd.sv[v][c >> 1];
-                const float sc = T::to_f32((uint16_t)((c & 1) ? (pair >> 16) : (pair & 0xFFFFu)));
-                const int f = v * 8 + c;
+            for (int b = 0; b < 4; ++b) {
+                f32x4 dlo = zero4, dhi = zero4;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[f][r] += sc * (dg[f][r] - zf * dones[r]);
+                for (int s = 0; s < CH; ++s) {
+                    u32x4 flo, fhi;
+#pragma unroll
+                    for (int rp = 0; rp < 4; ++rp) {
+                        // byte b of row 2rp -> bits 0..7, byte b of row 2rp+1 -> bits 16..23
+                        const uint32_t p = __builtin_amdgcn_perm(
+                            vget<V>(d.w[s][2 * rp + 1], v), vget<V>(d.w[s][2 * rp], v),
+                            0x0c000c00u | (uint32_t)b | ((4u + b) << 16));
+                        flo[rp] = Embed<T>::lo(p);
+                        fhi[rp] = Embed<T>::hi(p);
+                    }
+                    dlo = T::mfma16(d.xa[s], flo, dlo);
+                    dhi = T::mfma16(d.xa[s], fhi, dhi);
+                }
+                // byte b holds column {0,4,1,5}[b] in its low and {2,6,3,7}[b] in its high nibble
+                constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int c = h ? kHiCol[b] : kLoCol[b];
+                    const f32x4 dq = h ? dhi : dlo;
+                    const float zf = (float)(((zw >> nibble_shift(c)) & 0xFu) | 16u);
+                    const uint32_t pair = d.sv[v][c >> 1];
+                    const float sc = T::to_f32((uint16_t)((c & 1) ? (pair >> 16) : (pair & 0xFFFFu)));
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[v * 8 + c][r] += sc * (dq[r] - zf * dones[r]);
+                }
             }
         }
     };
 
-    if (t0 < t1) {
-        StepData<V> cur, nxt;
-        GroupData<V> gcur, gnxt;
-        load_step(t0, cur);
-        load_group(t0 / steps_per_group, gcur);
-        bool fresh = true;  // dg/dones need zeroing before the next MFMA
-        const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
-        for (int t = t0; t < t1; ++t) {
-            const bool more = t + 1 < t1;
-            const bool next_new_group = more && ((t + 1) % steps_per_group == 0);
-            if (more) load_step(t + 1, nxt);
-            if (next_new_group) load_group((t + 1) / steps_per_group, gnxt);
-            if (fresh) {
-#pragma unroll
-                for (int f = 0; f < NF; ++f) dg[f] = f32x4{0.f, 0.f, 0.f, 0.f};
-                dones = f32x4{0.f, 0.f, 0.f, 0.f};
-                fresh = false;
+    if constexpr (PF) {
+        Chunk<V, CH> a, b;
+        if (c0 < c1) load_chunk(c0, a);
+        for (int c = c0; c < c1; c += 2) {
+            if (c + 1 < c1) load_chunk(c + 1, b);
+            compute_chunk(a);
+            if (c + 1 < c1) {
+                if (c + 2 < c1) load_chunk(c + 2, a);
+                compute_chunk(b);
             }
-#pragma unroll
-            for (int v = 0; v < V; ++v) {
-                u32x4 bfrag[8];
-#pragma unroll
-                for (int rp = 0; rp < 4; ++rp) {
-                    const uint32_t w0 = vget<V>(cur.w[2 * rp], v);
-                    const uint32_t w1 = vget<V>(cur.w[2 * rp + 1], v);
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        // byte b of row 2rp -> bits 0..7, byte b of row 2rp+1 -> bits 16..23
-                        const uint32_t p =
-                            __builtin_amdgcn_perm(w1, w0, 0x0c000c00u | (uint32_t)b | ((4u + b) << 16));
-                        constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
-                        bfrag[kLoCol[b]][rp] = Embed<T>::lo(p);
-                        bfrag[kHiCol[b]][rp] = Embed<T>::hi(p);
-                    }
-                }
-#pragma unroll
-                for (int c = 0; c < 8; ++c) dg[v * 8 + c] = T::mfma16(cur.xa, bfrag[c], dg[v * 8 + c]);
-            }
-            dones = T::mfma16(cur.xa, ones, dones);
-            if (next_new_group || !more) {
-                flush(gcur);
-                fresh = true;
-                if (next_new_group) gcur = gnxt;
-            }
-            if (more) cur = nxt;
+        }
+    } else {
+        Chunk<V, CH> a;
+        for (int c = c0; c < c1; ++c) {
+            load_chunk(c, a);
+            compute_chunk(a);
         }
     }
 
@@ -231,7 +224,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
                         for (int c = 0; c < 8; ++c) out[c] = acc[vv * 8 + c][rr];
         }
         if (m < M && col_ok) {
-            const size_t n0 = (size_t)(c0 + v) * 8;
+            const size_t n0 = ((size_t)wv_col * V + v) * 8;
             if (splits == 1) {
                 if (bias) {
                     const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
@@ -245,24 +238,15 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
                 *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
             } else {
                 float* p = partials + ((size_t)split * M + m) * N + n0;
-                *reinterpret_cast<f32x4*>(p) = f32x4{out[0], out[1], out[2], out[3]};
-                *reinterpret_cast<f32x4*>(p + 4) = f32x4{out[4], out[5], out[6], out[7]};
+#pragma unroll
+                for (int c = 0; c < 8; ++c) publish_f32(p + c, out[c]);
             }
         }
     }
     if (splits == 1) return;
 
     // ---- cross-workgroup: last arriver sums the partials in split order -----
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const int prev = __hip_atomic_fetch_add(&counters[tile], 1, __ATOMIC_ACQ_REL,
-                                                __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == splits - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
+    if (!arrive_last(&counters[tile], splits, &s_last)) return;
     const int tile_words = 16 * V;
     const int w_begin = tile * tile_words;
     const int w_count = min(tile_words, words - w_begin);
@@ -272,13 +256,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         for (int s = 0; s < splits; ++s) {
             const float* p = partials + ((size_t)s * M + m) * N + n0;
-            const f32x4 a = *reinterpret_cast<const f32x4*>(p);
-            const f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                out[c] += a[c];
-                out[4 + c] += b[c];
-            }
+            for (int c = 0; c < 8; ++c) out[c] += fetch_f32(p + c);
         }
         if (bias) {
             const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
@@ -291,35 +270,40 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
         for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
         *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
     }
-    if (threadIdx.x == 0) counters[tile] = 0;
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- host side -------------------------------------------------------------
 struct GemvVariant {
     const char* name;
     int V, waves;
+    bool prefetch;
 };
 static const GemvVariant kGemvVariants[] = {
-    {"v1w4", 1, 4}, {"v1w8", 1, 8}, {"v1w16", 1, 16}, {"v2w4", 2, 4},
-    {"v2w8", 2, 8}, {"v4w4", 4, 4}, {"v1w1", 1, 1},  {"v2w1", 2, 1},
+    {"v1w4p", 1, 4, true},  {"v1w8p", 1, 8, true},  {"v2w4", 2, 4, false}, {"v2w8", 2, 8, false},
+    {"v2w4p", 2, 4, true},  {"v1w16", 1, 16, false}, {"v1w1p", 1, 1, true}, {"v2w1", 2, 1, false},
+    {"v1w4", 1, 4, false},  {"v1w8", 1, 8, false},
 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 
-template <typename T, int V, int WAVES>
+// rows per chunk: 128 when the group size allows it, else 32
+static inline int chunk_steps(int64_t g) { return g % 128 == 0 ? 4 : 1; }
+
+template <typename T, int V, int WAVES, int CH, bool PF>
 static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void* qscales,
                               const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                               int g, void* workspace, int split_k, hipStream_t stream) {
     const int words = N / 8;
     const int tiles = (int)cdiv(words, 16 * V);
-    const int total_steps = K / 32;
-    const int steps_per_split = (int)cdiv(total_steps, split_k);
-    const int splits = (int)cdiv(total_steps, steps_per_split);
+    const int total_chunks = K / (32 * CH);
+    const int cps = (int)cdiv(total_chunks, split_k);
+    const int splits = (int)cdiv(total_chunks, cps);
     int* counters = reinterpret_cast<int*>(workspace);
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
-                                                            counter_bytes(tiles))
+                                                            kCounterBytes)
                                 : nullptr;
     const size_t lds = WAVES > 1 ? (size_t)WAVES * 8 * V * 4 * 64 * sizeof(float) : 0;
-    auto kern = gemv_kernel<T, V, WAVES>;
+    auto kern = gemv_kernel<T, V, WAVES, CH, PF>;
     if (lds > 64 * 1024) {
         // once per process and instantiation; a racing second call only repeats it
         static bool raised = false;
@@ -336,36 +320,29 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
                        reinterpret_cast<const uint16_t*>(qscales),
                        reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
-                       partials, counters, M, N, K, g, steps_per_split, splits);
+                       partials, counters, M, N, K, g / (32 * CH), cps, splits);
     return hipGetLastError();
 }
 
-static int effective_splits(int64_t K, int split_k) {
-    const int total_steps = (int)(K / 32);
-    const int sps = (int)cdiv(total_steps, split_k);
-    return (int)cdiv(total_steps, sps);
-}
-
+// Upper bound that does not depend on the group size: the kernel never uses
+// more K-splits than asked for.
 static size_t gemv_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k) {
-    const GemvVariant& gv = kGemvVariants[variant];
-    const int splits = effective_splits(K, split_k);
-    if (splits <= 1) return 0;
-    const int64_t tiles = cdiv(N / 8, 16 * gv.V);
-    return counter_bytes(tiles) + (size_t)splits * M * N * sizeof(float);
+    (void)variant;
+    if (split_k <= 1 || K < 64) return 0;
+    return kCounterBytes + (size_t)split_k * M * N * sizeof(float);
 }
 
-// Launch shape for the default entry point: enough waves to cover the chip a
-// few times over, K-runs per wave as long as that allows.
+// Launch shape for the default entry point.
 static void pick_gemv(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     (void)M;
-    const int64_t steps = K / 32;
-    int v = (N % 16 == 0 && N * K >= (int64_t)4096 * 4096) ? 3 /* v2w4 */ : 0 /* v1w4 */;
+    const int64_t chunks = K / 128 > 0 ? K / 128 : 1;
+    const bool wide = (N % 16 == 0) && N >= 4096;
+    const int v = wide ? 2 /* v2w4 */ : 0 /* v1w4p */;
     const GemvVariant& gv = kGemvVariants[v];
     const int64_t tiles = cdiv(N / 8, 16 * gv.V);
-    // target ~4 waves per SIMD: 256 CUs * 4 SIMDs * 4
-    const int64_t want_wgs = (256 * 16) / gv.waves;
-    int64_t s = cdiv(want_wgs, tiles);
-    const int64_t max_s = steps / gv.waves > 0 ? steps / gv.waves : 1;  // >= 1 step per wave
+    // aim at ~2 workgroups of 4 waves per CU, but never less than one chunk per wave
+    int64_t s = cdiv(512, tiles);
+    const int64_t max_s = chunks / gv.waves > 0 ? chunks / gv.waves : 1;
     if (s > max_s) s = max_s;
     if (s < 1) s = 1;
     if (s > 64) s = 64;
@@ -400,32 +377,46 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         set_error("%s: variant %s needs N %% %d == 0 (N=%lld)", fn, gv.name, 8 * gv.V, (long long)N);
         return AWQ_ERR_UNSUPPORTED;
     }
+    if (split_k > 1 && cdiv(N / 8, 16 * gv.V) > kMaxSplitTiles) {
+        set_error("%s: split-K supports at most %lld column tiles (N=%lld)", fn,
+                  (long long)kMaxSplitTiles, (long long)N);
+        return AWQ_ERR_UNSUPPORTED;
+    }
     const size_t need = gemv_ws_bytes(M, N, K, variant, split_k);
     if (need > 0 && (!workspace || workspace_bytes < need)) {
         set_error("%s: workspace of %zu bytes needed, %zu given", fn, need, workspace ? workspace_bytes : (size_t)0);
         return AWQ_ERR_WORKSPACE;
     }
+    if (need == 0) split_k = 1;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
-#define AWQ_GEMV_CASE(IDX, VV, WW)                                                                \
-    case IDX:                                                                                     \
-        e = dtype == AWQ_F16                                                                      \
-                ? launch_gemv<F16, VV, WW>(x, qweight, qscales, qzeros, bias, y, (int)M, (int)N,  \
-                                           (int)K, (int)g, workspace, split_k, s)                 \
-                : launch_gemv<BF16, VV, WW>(x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, \
-                                            (int)K, (int)g, workspace, split_k, s);               \
+    const bool big_chunk = chunk_steps(g) == 4;
+#define AWQ_GEMV_LAUNCH(TT, VV, WW, CC, PP)                                                        \
+    launch_gemv<TT, VV, WW, CC, PP>(x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, \
+                                    (int)g, workspace, split_k, s)
+#define AWQ_GEMV_CASE(IDX, VV, WW, PP)                                                     \
+    case IDX:                                                                              \
+        if (big_chunk)                                                                     \
+            e = dtype == AWQ_F16 ? AWQ_GEMV_LAUNCH(F16, VV, WW, 4, PP)                     \
+                                 : AWQ_GEMV_LAUNCH(BF16, VV, WW, 4, PP);                   \
+        else /* group sizes 32/64/96...: one 32-row step per chunk, no prefetch variant */ \
+            e = dtype == AWQ_F16 ? AWQ_GEMV_LAUNCH(F16, VV, WW, 1, true)                   \
+                                 : AWQ_GEMV_LAUNCH(BF16, VV, WW, 1, true);                 \
         break;
     switch (variant) {
-        AWQ_GEMV_CASE(0, 1, 4)
-        AWQ_GEMV_CASE(1, 1, 8)
-        AWQ_GEMV_CASE(2, 1, 16)
-        AWQ_GEMV_CASE(3, 2, 4)
-        AWQ_GEMV_CASE(4, 2, 8)
-        AWQ_GEMV_CASE(5, 4, 4)
-        AWQ_GEMV_CASE(6, 1, 1)
-        AWQ_GEMV_CASE(7, 2, 1)
+        AWQ_GEMV_CASE(0, 1, 4, true)
+        AWQ_GEMV_CASE(1, 1, 8, true)
+        AWQ_GEMV_CASE(2, 2, 4, false)
+        AWQ_GEMV_CASE(3, 2, 8, false)
+        AWQ_GEMV_CASE(4, 2, 4, true)
+        AWQ_GEMV_CASE(5, 1, 16, false)
+        AWQ_GEMV_CASE(6, 1, 1, true)
+        AWQ_GEMV_CASE(7, 2, 1, false)
+        AWQ_GEMV_CASE(8, 1, 4, false)
+        AWQ_GEMV_CASE(9, 1, 8, false)
     }
 #undef AWQ_GEMV_CASE
+#undef AWQ_GEMV_LAUNCH
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }
 

@@ -196,9 +196,9 @@ class WQLinear_GEMM(nn.Module):
             linear_layer.bias is not None,
             output_dtype,
         )
-        awq_linear.qscales = scales.clone().to(output_dtype)
+        awq_linear.qscales = scales.detach().clone().to(output_dtype)
         if linear_layer.bias is not None:
-            awq_linear.bias = linear_layer.bias.clone().to(output_dtype)
+            awq_linear.bias = linear_layer.bias.detach().clone().to(output_dtype)
 
         w = linear_layer.weight.data
         K = awq_linear.in_features

@@ -41,7 +41,7 @@ def test_library_exports_every_declared_symbol():
     assert rc == 1 and b"null pointer" in L.awq_hip_last_error()
     # the published packed-weight workspace rule: 0 bytes when there is nothing to split
     assert L.awq_gemv_ex_workspace_bytes(1, 1024, 1024, 0, 1) == 0
-    assert L.awq_gemv_ex_workspace_bytes(4, 1024, 1024, 0, 4) == 256 + 4 * 4 * 1024 * 4
+    assert L.awq_gemv_ex_workspace_bytes(4, 1024, 1024, 0, 4) == 4096 * 4 + 4 * 4 * 1024 * 4
 
 
 def test_pseudo_quantize_matches_oracle_bitwise():
