@@ -26,13 +26,19 @@ FLAGS = [
 ]
 
 
+# per-source extra flags
+EXTRA = {
+    # keep MFMA results in VGPRs: the GEMV folds every accumulator into fp32 state right away,
+    # AGPR destinations would cost a v_accvgpr_read per value and 4 more registers per wave
+    "awq_gemv.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def sources() -> list[str]:
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
-def build(verbose: bool = True) -> str:
-    """Compile every HIP source into one shared library; returns its path."""
-    cmd = [HIPCC, *FLAGS, *sources(), "-o", LIB_PATH]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -42,6 +48,22 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
     if verbose and out.strip():
         print(out)
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every HIP source (in parallel) and link one shared library; returns its path."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    objdir = os.path.join(PKG_DIR, "build")
+    os.makedirs(objdir, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    jobs = []
+    for src in sources():
+        obj = os.path.join(objdir, os.path.basename(src) + ".o")
+        jobs.append(([HIPCC, *compile_flags, *EXTRA.get(os.path.basename(src), []), "-c", src, "-o", obj], obj))
+    with ThreadPoolExecutor(max_workers=min(4, len(jobs))) as pool:
+        list(pool.map(lambda j: _run(j[0], verbose), jobs))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *[o for _, o in jobs], "-o", LIB_PATH], verbose)
     return LIB_PATH
 
 

@@ -314,6 +314,7 @@ static hipError_t launch_gemm(const void* x, const int32_t* qweight, const void*
             raised = true;
         }
     }
+    (void)hipGetLastError();  // do not report an earlier, unrelated failure as this launch's
     hipLaunchKernelGGL(kern, dim3(tiles_n, tiles_m, splits), dim3(256), lds, stream,
                        reinterpret_cast<const uint16_t*>(x),
                        reinterpret_cast<const uint32_t*>(qweight),

@@ -5,46 +5,80 @@
 // <=16 activation rows, B = 16 output columns x 32 k), because even M = 2
 // would saturate the vector ALUs at HBM speed.
 //
-// Data movement.  A lane is (j = lane % 16, kb = lane / 16).  Per 32-row step
-// it loads V packed words from each of rows k0 + 8*kb + 0..7, word columns
-// (tile*16 + j)*V .. +V-1: 16 lanes x 4V bytes are contiguous per row.  Those
-// 8 rows x V words are 8V columns x 8 consecutive k: exactly the 8 k-slots the
-// MFMA B operand wants per lane, once the nibbles of two rows are paired.
+// Lane roles.  A lane is (j = lane % 16, kb = lane / 16).  Per 32-row step it
+// owns V packed words from each of rows k0 + 8*kb + 0..7, word columns
+// (tile*16 + j)*V .. +V-1.  Those 8 rows x V words are 8V columns x 8
+// consecutive k: exactly the 8 k-slots the MFMA B operand wants per lane, once
+// the nibbles of two rows are paired.
 //
 // In-register transposition.  v_perm_b32 puts byte b of row k into the low
-// half and byte b of row k+1 into the high half of one register; a shift and
-// one v_and_or_b32 then turn the two low (or high) nibbles into a packed pair
-// of 16-bit floats with value 16 + q (the nibble sits in the top mantissa bits
-// under the exponent of 16.0) -- no int->float conversion, no LDS.
+// half and byte b of row k+1 into the high half of one register; one
+// v_and_or_b32 (after a shift for half of the nibbles) turns a nibble pair into
+// two 16-bit floats whose value is c0 + c1*q, the nibble sitting in mantissa
+// bits under a fixed exponent -- no int->float conversion, no LDS transpose.
 //
 // Scale and zero point are applied per quantisation group, in fp32, on the
 // accumulator instead of per weight:
-//   y += s[g,n] * ( sum_k x[k]*(16+q[k,n])  -  (16+z[g,n]) * sum_k x[k] )
+//   y += (s[g,n]/c1) * ( sum_k x[k]*(c0+c1*q[k,n])  -  (c0+c1*z[g,n]) * sum_k x[k] )
 // where sum_k x[k] comes from one extra MFMA per step against a B operand of
-// ones.  The products 16+q are exact, so this differs from the reference's
-// "round W to 16 bits, then multiply" only by not rounding W.
+// ones.  The products x*(c0+c1*q) are exact in the MFMA, so this differs from
+// the reference's "round W to 16 bits, then multiply" only by not rounding W.
+//
+// Work is cut in chunks of CH steps (128 rows when the group size allows) that
+// never straddle a group.  Per chunk and column pair the MFMAs of all CH steps
+// chain on one accumulator, which is folded into the running fp32 result at
+// once, so only 8V x 4 accumulators stay live.
+//
+// Two data paths feed the same arithmetic:
+//   * gemv_kernel      global -> registers (optionally one chunk ahead);
+//   * gemv_dma_kernel  global -> LDS by the load-to-LDS DMA (no registers held
+//                      while the data is in flight), LDS -> registers just
+//                      before use: one chunk per wave always in flight at a
+//                      register cost that allows 4 waves per SIMD.
 //
 // Reduction.  Waves of a workgroup own consecutive K sub-slices and are summed
-// through LDS in a fixed order; workgroups of different K-splits write fp32
-// partials to the workspace and the last one to arrive (an agent-scope counter)
-// adds them in split order, so results are bit-stable run to run.
+// through LDS in a fixed order; workgroups of different K-splits publish fp32
+// partials and the last one to arrive (an arrival counter per tile) adds them
+// in split order, so results are bit-stable run to run.
 #include "awq_common.hpp"
 
 namespace awq {
 
+// Nibble -> 16-bit float embeddings.  lo()/hi() take the v_perm result
+// 0x00HL00HL (two rows of one byte) and return the pair of floats for the low /
+// high nibble; the value is off + mul*q with the constants below.
 template <typename T>
 struct Embed;
 template <>
-struct Embed<F16> {  // 16.0 = 0x4C00, 10 mantissa bits: q << 6
-    static constexpr uint32_t mask = 0x03C003C0u, magic = 0x4C004C00u;
-    static __device__ __forceinline__ uint32_t lo(uint32_t p) { return ((p << 6) & mask) | magic; }
-    static __device__ __forceinline__ uint32_t hi(uint32_t p) { return ((p << 2) & mask) | magic; }
+struct Embed<F16> {
+    // 0x6400 | q<<4 = 1024 + 16 q for both nibbles
+    static constexpr uint32_t kMaskLo = 0x00F000F0u, kMagicLo = 0x64006400u;
+    static constexpr uint32_t kMaskHi = 0x00F000F0u, kMagicHi = 0x64006400u;
+    static constexpr float kMul = 16.f, kOffLo = 1024.f, kOffHi = 1024.f;
+    static __device__ __forceinline__ uint32_t pre_lo(uint32_t p) { return p << 4; }
+    static __device__ __forceinline__ uint32_t pre_hi(uint32_t p) { return p; }
+    static constexpr float kMulLo = 16.f, kMulHi = 16.f;
 };
 template <>
-struct Embed<BF16> {  // 16.0 = 0x4180, 7 mantissa bits: q << 3
-    static constexpr uint32_t mask = 0x00780078u, magic = 0x41804180u;
-    static __device__ __forceinline__ uint32_t lo(uint32_t p) { return ((p << 3) & mask) | magic; }
-    static __device__ __forceinline__ uint32_t hi(uint32_t p) { return ((p >> 1) & mask) | magic; }
+struct Embed<BF16> {
+    // low nibble: 0x4300 | q = 128 + q; high nibble: 0x4180 | q<<3 = 16 + q
+    static constexpr uint32_t kMaskLo = 0x000F000Fu, kMagicLo = 0x43004300u;
+    static constexpr uint32_t kMaskHi = 0x00780078u, kMagicHi = 0x41804180u;
+    static constexpr float kOffLo = 128.f, kOffHi = 16.f;
+    static __device__ __forceinline__ uint32_t pre_lo(uint32_t p) { return p; }
+    static __device__ __forceinline__ uint32_t pre_hi(uint32_t p) { return p >> 1; }
+    static constexpr float kMulLo = 1.f, kMulHi = 1.f;
+};
+
+// (a & mask) | magic as one v_and_or_b32: gfx950's VOP3 takes no literals and a
+// single scalar operand, so the mask is pinned in an SGPR and the magic in a VGPR.
+struct AndOr {
+    uint32_t mask, magic;
+    __device__ __forceinline__ AndOr(uint32_t m, uint32_t g) : mask(m), magic(g) {
+        asm volatile("" : "+s"(mask));
+        asm volatile("" : "+v"(magic));
+    }
+    __device__ __forceinline__ uint32_t operator()(uint32_t a) const { return (a & mask) | magic; }
 };
 
 template <int V>
@@ -70,6 +104,163 @@ struct Chunk {
     u32x4 sv[V];                         // 8 scales per word
 };
 
+// acc[8V] += one chunk.  acc[v*8 + c][r] is output row 4*kb + r, column 8*(word v) + c.
+template <typename T, int V, int CH>
+__device__ __forceinline__ void compute_chunk(const Chunk<V, CH>& d, f32x4 (&acc)[8 * V]) {
+    const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
+    const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+    const AndOr emb_lo(Embed<T>::kMaskLo, Embed<T>::kMagicLo), emb_hi(Embed<T>::kMaskHi, Embed<T>::kMagicHi);
+    f32x4 dones = zero4;
+#pragma unroll
+    for (int s = 0; s < CH; ++s) dones = T::mfma16(d.xa[s], ones, dones);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const uint32_t zw = vget<V>(d.zw, v);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            f32x4 dlo = zero4, dhi = zero4;
+#pragma unroll
+            for (int s = 0; s < CH; ++s) {
+                u32x4 flo, fhi;
+#pragma unroll
+                for (int rp = 0; rp < 4; ++rp) {
+                    // byte b of row 2rp -> bits 0..7, byte b of row 2rp+1 -> bits 16..23
+                    const uint32_t p = __builtin_amdgcn_perm(
+                        vget<V>(d.w[s][2 * rp + 1], v), vget<V>(d.w[s][2 * rp], v),
+                        0x0c000c00u | (uint32_t)b | ((4u + b) << 16));
+                    flo[rp] = emb_lo(Embed<T>::pre_lo(p));
+                    fhi[rp] = emb_hi(Embed<T>::pre_hi(p));
+                }
+                dlo = T::mfma16(d.xa[s], flo, dlo);
+                dhi = T::mfma16(d.xa[s], fhi, dhi);
+            }
+            // byte b holds column {0,4,1,5}[b] in its low and {2,6,3,7}[b] in its high nibble
+            constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int c = h ? kHiCol[b] : kLoCol[b];
+                const f32x4 dq = h ? dhi : dlo;
+                const float mul = h ? Embed<T>::kMulHi : Embed<T>::kMulLo;
+                const float off = h ? Embed<T>::kOffHi : Embed<T>::kOffLo;
+                // value of the embedded zero point, off + mul*z, and the scale / mul
+                const float zf = (float)((zw >> nibble_shift(c)) & 0xFu) * mul + off;
+                const uint32_t pair = d.sv[v][c >> 1];
+                const float sc = T::to_f32((uint16_t)((c & 1) ? (pair >> 16) : (pair & 0xFFFFu))) * (1.f / mul);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[v * 8 + c][r] += sc * (dq[r] - zf * dones[r]);
+            }
+        }
+    }
+}
+
+// A workgroup is WN x WK waves: wave w works on column tile (group*WN + w % WN)
+// and K sub-slice w / WN.  Sum the WK waves of each column tile through LDS
+// (fixed order), then either store y (splits == 1) or publish this split's
+// partial and let the last workgroup of the tile group add the partials in
+// split order.  `group` is the workgroup's index along N.
+template <typename T, int V, int WN, int WK>
+__device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[8 * V], float* red, int* s_last, int lane,
+                                              int wave, int group, int split, int splits,
+                                              const uint16_t* __restrict__ bias,
+                                              uint16_t* __restrict__ y, float* __restrict__ partials,
+                                              int* __restrict__ counters, int M, int N) {
+    constexpr int NF = 8 * V, NQ = 4 * V, WAVES = WN * WK;
+    const int j = lane & 15, kb = lane >> 4;
+    const int words = N >> 3;
+    const int wn = wave % WN, wk = wave / WN;
+    const int wv_col = (group * WN + wn) * 16 + j;  // this lane's column, in units of V words
+    const bool col_ok = wv_col * V < words;
+    // slot q = v*4 + r holds 8 consecutive output columns of row 4*kb + r
+    if constexpr (WK > 1) {
+        float* mine = red + (size_t)wave * (NF * 4 * 64);
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 8; ++c) mine[((v * 4 + r) * 8 + c) * 64 + lane] = acc[v * 8 + c][r];
+        __syncthreads();
+    }
+    for (int q = wk; q < NQ; q += WK) {
+        const int v = q >> 2, r = q & 3;
+        const int m = 4 * kb + r;
+        float out[8];
+        if constexpr (WK > 1) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < WK; ++w)
+                    s += red[(size_t)(w * WN + wn) * (NF * 4 * 64) + (q * 8 + c) * 64 + lane];
+                out[c] = s;
+            }
+        } else {
+            // one wave per column tile: q runs over every slot; pick from registers
+#pragma unroll
+            for (int vv = 0; vv < V; ++vv)
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr)
+                    if (vv == v && rr == r)
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) out[c] = acc[vv * 8 + c][rr];
+        }
+        if (m < M && col_ok) {
+            const size_t n0 = ((size_t)wv_col * V + v) * 8;
+            if (splits == 1) {
+                if (bias) {
+                    const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c)
+                        out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
+                }
+                u32x4 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+                *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
+            } else {
+                float* p = partials + ((size_t)split * M + m) * N + n0;
+#pragma unroll
+                for (int c = 0; c < 8; ++c) publish_f32(p + c, out[c]);
+            }
+        }
+    }
+    if (splits == 1) return;
+
+    if (!arrive_last(&counters[group], splits, s_last)) return;
+    const int group_words = 16 * V * WN;
+    const int w_begin = group * group_words;
+    const int w_count = min(group_words, words - w_begin);
+    for (int idx = threadIdx.x; idx < M * w_count; idx += 64 * WAVES) {
+        const int m = idx / w_count, wc = idx - m * w_count;
+        const size_t n0 = (size_t)(w_begin + wc) * 8;
+        float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < splits; ++s) {
+            const float* p = partials + ((size_t)s * M + m) * N + n0;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) out[c] += fetch_f32(p + c);
+        }
+        if (bias) {
+            const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
+        }
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+        *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(&counters[group], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
+// of column groups so that neighbouring groups share an L2.
+__device__ __forceinline__ int xcd_aware_group(int bid, int ngroups) {
+    if ((ngroups & 7) != 0) return bid;
+    return (bid & 7) * (ngroups >> 3) + (bid >> 3);
+}
+
+// ---- data path 1: global -> registers ------------------------------------------
 template <typename T, int V, int WAVES, int CH, bool PF>
 __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
@@ -102,10 +293,14 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
     const int c0 = c_begin + wave * per_wave;
     const int c1 = min(c0 + per_wave, c_end);
 
-    const WV* wlane = reinterpret_cast<const WV*>(qweight) + (size_t)(kb * 8) * wstride + wv_ld;
-    const WV* zlane = reinterpret_cast<const WV*>(qzeros) + wv_ld;
-    const u32x4* slane = reinterpret_cast<const u32x4*>(scales) + (size_t)wv_ld * V;
-    const uint16_t* xlane = x + (size_t)xrow * K + kb * 8;
+    const WV* wbase = reinterpret_cast<const WV*>(qweight);
+    const WV* zbase = reinterpret_cast<const WV*>(qzeros);
+    const u32x4* sbase = reinterpret_cast<const u32x4*>(scales);
+    // per-lane element offsets, 32-bit so that loads can use scalar base + vector offset
+    uint32_t woff[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) woff[r] = (uint32_t)(kb * 8 + r) * (uint32_t)wstride + (uint32_t)wv_ld;
+    const uint32_t xoff = (uint32_t)xrow * (uint32_t)K + (uint32_t)kb * 8u;
 
     f32x4 acc[NF];
 #pragma unroll
@@ -113,60 +308,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
 
     auto load_chunk = [&](int c, Chunk<V, CH>& d) {
         const int row0 = c * (32 * CH);  // wave-uniform
-        const WV* wp = wlane + (size_t)row0 * wstride;
 #pragma unroll
-        for (int s = 0; s < CH; ++s)
+        for (int s = 0; s < CH; ++s) {
+            const WV* wp = wbase + (size_t)(row0 + s * 32) * wstride;  // uniform
 #pragma unroll
-            for (int r = 0; r < 8; ++r) d.w[s][r] = wp[(size_t)(s * 32 + r) * wstride];
-#pragma unroll
-        for (int s = 0; s < CH; ++s) d.xa[s] = *reinterpret_cast<const u32x4*>(xlane + row0 + s * 32);
-        const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
-        d.zw = zlane[(size_t)gi * wstride];
-#pragma unroll
-        for (int v = 0; v < V; ++v) d.sv[v] = slane[(size_t)gi * words + v];
-    };
-
-    const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
-    const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
-    auto compute_chunk = [&](const Chunk<V, CH>& d) {
-        f32x4 dones = zero4;
-#pragma unroll
-        for (int s = 0; s < CH; ++s) dones = T::mfma16(d.xa[s], ones, dones);
-#pragma unroll
-        for (int v = 0; v < V; ++v) {
-            const uint32_t zw = vget<V>(d.zw, v);
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                f32x4 dlo = zero4, dhi = zero4;
-#pragma unroll
-                for (int s = 0; s < CH; ++s) {
-                    u32x4 flo, fhi;
-#pragma unroll
-                    for (int rp = 0; rp < 4; ++rp) {
-                        // byte b of row 2rp -> bits 0..7, byte b of row 2rp+1 -> bits 16..23
-                        const uint32_t p = __builtin_amdgcn_perm(
-                            vget<V>(d.w[s][2 * rp + 1], v), vget<V>(d.w[s][2 * rp], v),
-                            0x0c000c00u | (uint32_t)b | ((4u + b) << 16));
-                        flo[rp] = Embed<T>::lo(p);
-                        fhi[rp] = Embed<T>::hi(p);
-                    }
-                    dlo = T::mfma16(d.xa[s], flo, dlo);
-                    dhi = T::mfma16(d.xa[s], fhi, dhi);
-                }
-                // byte b holds column {0,4,1,5}[b] in its low and {2,6,3,7}[b] in its high nibble
-                constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int c = h ? kHiCol[b] : kLoCol[b];
-                    const f32x4 dq = h ? dhi : dlo;
-                    const float zf = (float)(((zw >> nibble_shift(c)) & 0xFu) | 16u);
-                    const uint32_t pair = d.sv[v][c >> 1];
-                    const float sc = T::to_f32((uint16_t)((c & 1) ? (pair >> 16) : (pair & 0xFFFFu)));
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[v * 8 + c][r] += sc * (dq[r] - zf * dones[r]);
-                }
-            }
+            for (int r = 0; r < 8; ++r) d.w[s][r] = wp[woff[r]];
         }
+#pragma unroll
+        for (int s = 0; s < CH; ++s) d.xa[s] = *reinterpret_cast<const u32x4*>(x + (row0 + s * 32) + xoff);
+        const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
+        d.zw = (zbase + (size_t)gi * wstride)[wv_ld];
+#pragma unroll
+        for (int v = 0; v < V; ++v) d.sv[v] = (sbase + (size_t)gi * words)[wv_ld * V + v];
     };
 
     if constexpr (PF) {
@@ -174,103 +327,140 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
         if (c0 < c1) load_chunk(c0, a);
         for (int c = c0; c < c1; c += 2) {
             if (c + 1 < c1) load_chunk(c + 1, b);
-            compute_chunk(a);
+            compute_chunk<T, V, CH>(a, acc);
             if (c + 1 < c1) {
                 if (c + 2 < c1) load_chunk(c + 2, a);
-                compute_chunk(b);
+                compute_chunk<T, V, CH>(b, acc);
             }
         }
     } else {
         Chunk<V, CH> a;
         for (int c = c0; c < c1; ++c) {
             load_chunk(c, a);
-            compute_chunk(a);
+            compute_chunk<T, V, CH>(a, acc);
         }
     }
+    gemv_epilogue<T, V, 1, WAVES>(acc, red, &s_last, lane, wave, tile, split, splits, bias, y, partials,
+                                  counters, M, N);
+}
 
-    // ---- sum the waves of this workgroup through LDS (fixed order) ----------
-    // slot q = v*4 + r holds 8 consecutive output columns of row 4*kb + r
-    constexpr int NQ = 4 * V;
-    if constexpr (WAVES > 1) {
-        float* mine = red + (size_t)wave * (NF * 4 * 64);
-#pragma unroll
-        for (int v = 0; v < V; ++v)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-#pragma unroll
-                for (int c = 0; c < 8; ++c) mine[((v * 4 + r) * 8 + c) * 64 + lane] = acc[v * 8 + c][r];
-        __syncthreads();
-    }
-    for (int q = wave; q < NQ; q += WAVES) {
-        const int v = q >> 2, r = q & 3;
-        const int m = 4 * kb + r;
-        float out[8];
-        if constexpr (WAVES > 1) {
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                float s = 0.f;
-#pragma unroll
-                for (int w = 0; w < WAVES; ++w) s += red[(size_t)w * (NF * 4 * 64) + (q * 8 + c) * 64 + lane];
-                out[c] = s;
-            }
-        } else {
-            // WAVES == 1: q runs over every slot in this wave; pick from registers
-#pragma unroll
-            for (int vv = 0; vv < V; ++vv)
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr)
-                    if (vv == v && rr == r)
-#pragma unroll
-                        for (int c = 0; c < 8; ++c) out[c] = acc[vv * 8 + c][rr];
-        }
-        if (m < M && col_ok) {
-            const size_t n0 = ((size_t)wv_col * V + v) * 8;
-            if (splits == 1) {
-                if (bias) {
-                    const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
-#pragma unroll
-                    for (int c = 0; c < 8; ++c)
-                        out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
-                }
-                u32x4 o;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
-                *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
-            } else {
-                float* p = partials + ((size_t)split * M + m) * N + n0;
-#pragma unroll
-                for (int c = 0; c < 8; ++c) publish_f32(p + c, out[c]);
-            }
-        }
-    }
-    if (splits == 1) return;
+// ---- data path 2: global -> LDS (DMA) -> registers -----------------------------
+// V = 1, CH = 4.  Needs N % 128 == 0 and a group size that is a multiple of 128.
+//
+// Per wave and chunk the LDS holds
+//   W  4 steps x 32 slots x 64 B   slot r*4 + kb' = row 8*kb' + r of the step, 16 words wide;
+//                                  the DMA lane (slot%16 = lane/4, quarter = lane%4) brings 16 B;
+//                                  the compute lane (j, kb) reads word j of slots r*4 + kb:
+//                                  64 lanes hit 64 different banks
+//   X  4 steps x M x 64 B          A operand, row m, 4 k-blocks of 16 B
+//   ZS 16 zero words + 16 x 8 scales
+#define AWQ_GPTR(p) ((__attribute__((address_space(1))) const void*)(p))
+#define AWQ_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-    // ---- cross-workgroup: last arriver sums the partials in split order -----
-    if (!arrive_last(&counters[tile], splits, &s_last)) return;
-    const int tile_words = 16 * V;
-    const int w_begin = tile * tile_words;
-    const int w_count = min(tile_words, words - w_begin);
-    for (int idx = threadIdx.x; idx < M * w_count; idx += 64 * WAVES) {
-        const int m = idx / w_count, wc = idx - m * w_count;
-        const size_t n0 = (size_t)(w_begin + wc) * 8;
-        float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < splits; ++s) {
-            const float* p = partials + ((size_t)s * M + m) * N + n0;
+__host__ __device__ constexpr int dma_wave_bytes(int M) { return 8192 + 256 * M + 512; }
+
+template <typename T, int WN, int WK>
+__global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
+    int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
+    int splits) {
+    constexpr int CH = 4;
+    extern __shared__ float red[];  // staging while streaming, [WAVES][32][64] floats afterwards
+    __shared__ int s_last;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 15, kb = lane >> 4;
+    const int words = N >> 3;
+    const int group = xcd_aware_group(blockIdx.x, gridDim.x), split = blockIdx.y;
+    const int tile = group * WN + wave % WN;   // host guarantees N % (128 * WN) == 0
+
+    const int total_chunks = K / 128;
+    const int c_begin = split * chunks_per_split;
+    const int c_end = min(c_begin + chunks_per_split, total_chunks);
+    const int per_wave = (max(c_end - c_begin, 0) + WK - 1) / WK;
+    const int c0 = c_begin + (wave / WN) * per_wave;
+    const int c1 = min(c0 + per_wave, c_end);
+
+    char* stage = reinterpret_cast<char*>(red) + (size_t)wave * dma_wave_bytes(M);
+    uint32_t* w_lds = reinterpret_cast<uint32_t*>(stage);
+    char* x_lds = stage + 8192;
+    char* zs_lds = stage + 8192 + 256 * M;
+
+    // DMA lane roles
+    const int dq = lane & 3, dsl = lane >> 2;  // 16-byte quarter of the 64-byte row piece, slot % 16
+    uint32_t wsrc[2];                          // word offset inside a step, for slots 0..15 / 16..31
 #pragma unroll
-            for (int c = 0; c < 8; ++c) out[c] += fetch_f32(p + c);
-        }
-        if (bias) {
-            const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-                out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
-        }
-        u32x4 o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
-        *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
+    for (int h = 0; h < 2; ++h) {
+        const int slot = h * 16 + dsl;
+        wsrc[h] = (uint32_t)((slot & 3) * 8 + (slot >> 2)) * (uint32_t)words + (uint32_t)(tile * 16 + dq * 4);
     }
-    if (threadIdx.x == 0) __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool x_lane = lane < 4 * M;          // lane = m*4 + k-block
+    const uint32_t xsrc = (uint32_t)(x_lane ? (lane >> 2) : 0) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
+    const bool zs_lane = lane < 16;
+    const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
+
+    auto issue_dma = [&](int c) {
+        const int row0 = c * 128;
+#pragma unroll
+        for (int s = 0; s < CH; ++s) {
+            const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
+                                                 16, 0, 0);
+        }
+        if (x_lane) {
+#pragma unroll
+            for (int s = 0; s < CH; ++s)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc),
+                                                 AWQ_LPTR(x_lds + s * 64 * M), 16, 0, 0);
+        }
+        if (zs_lane) {
+            const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
+            __builtin_amdgcn_global_load_lds(AWQ_GPTR(qzeros + (size_t)gi * words + zsrc), AWQ_LPTR(zs_lds), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(AWQ_GPTR(scales + ((size_t)gi * words + zsrc) * 8),
+                                             AWQ_LPTR(zs_lds + 64), 16, 0, 0);
+        }
+    };
+
+    // compute-lane read positions
+    const uint32_t* w_rd = w_lds + kb * 16 + j;                     // + s*512 + r*64
+    const int xm = j < M ? j : M - 1;
+    const u32x4* x_rd = reinterpret_cast<const u32x4*>(x_lds) + xm * 4 + kb;  // + s*4*M
+    const uint32_t* z_rd = reinterpret_cast<const uint32_t*>(zs_lds) + j;
+    const u32x4* s_rd = reinterpret_cast<const u32x4*>(zs_lds + 64) + j;
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) acc[f] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (c0 < c1) issue_dma(c0);
+    for (int c = c0; c < c1; ++c) {
+        // the DMA of chunk c has landed: vmcnt(0); the compiler does not order LDS reads after it by itself
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" ::: "memory");
+        Chunk<1, CH> d;
+#pragma unroll
+        for (int s = 0; s < CH; ++s) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) d.w[s][r] = w_rd[s * 512 + r * 64];
+            d.xa[s] = x_rd[s * 4 * M];
+        }
+        d.zw = *z_rd;
+        d.sv[0] = *s_rd;
+        // every LDS read has returned before the next chunk's DMA may overwrite the staging area
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        asm volatile("" ::: "memory");
+        if (c + 1 < c1) issue_dma(c + 1);
+        compute_chunk<T, 1, CH>(d, acc);
+    }
+    __syncthreads();  // staging area becomes the reduction buffer
+    gemv_epilogue<T, 1, WN, WK>(acc, red, &s_last, lane, wave, group, split, splits, bias, y, partials,
+                                counters, M, N);
 }
 
 // ---- host side -------------------------------------------------------------
@@ -278,12 +468,19 @@ struct GemvVariant {
     const char* name;
     int V, waves;
     bool prefetch;
+    int wn;  // waves side by side along N (DMA variants), 1 otherwise
 };
 static const GemvVariant kGemvVariants[] = {
-    {"v1w4p", 1, 4, true},  {"v1w8p", 1, 8, true},  {"v2w4", 2, 4, false}, {"v2w8", 2, 8, false},
-    {"v2w4p", 2, 4, true},  {"v1w16", 1, 16, false}, {"v1w1p", 1, 1, true}, {"v2w1", 2, 1, false},
-    {"v1w4", 1, 4, false},  {"v1w8", 1, 8, false},
+    {"v1w4p", 1, 4, true, 1},  {"v1w8p", 1, 8, true, 1},   {"v2w4", 2, 4, false, 1},
+    {"v2w8", 2, 8, false, 1},  {"v2w4p", 2, 4, true, 1},   {"v1w16", 1, 16, false, 1},
+    {"v1w1p", 1, 1, true, 1},  {"v2w1", 2, 1, false, 1},   {"v1w4", 1, 4, false, 1},
+    {"v1w8", 1, 8, false, 1},
+    // DMA variants, named dma<WN>x<WK>
+    {"dma1x4", 1, 4, false, 1}, {"dma2x2", 1, 4, false, 2}, {"dma4x1", 1, 4, false, 4},
+    {"dma2x4", 1, 8, false, 2}, {"dma4x2", 1, 8, false, 4}, {"dma1x8", 1, 8, false, 1},
+    {"dma1x1", 1, 1, false, 1}, {"dma4x4", 1, 16, false, 4}, {"dma2x8", 1, 16, false, 2},
 };
+constexpr int kFirstDmaVariant = 10;
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 
 // rows per chunk: 128 when the group size allows it, else 32
@@ -314,6 +511,7 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
             raised = true;
         }
     }
+    (void)hipGetLastError();  // do not report an earlier, unrelated failure as this launch's
     hipLaunchKernelGGL(kern, dim3(tiles, splits), dim3(64 * WAVES), lds, stream,
                        reinterpret_cast<const uint16_t*>(x),
                        reinterpret_cast<const uint32_t*>(qweight),
@@ -321,6 +519,46 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
                        reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
                        partials, counters, M, N, K, g / (32 * CH), cps, splits);
+    return hipGetLastError();
+}
+
+template <typename T, int WN, int WK>
+static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
+                                  const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
+                                  int g, void* workspace, int split_k, hipStream_t stream) {
+    constexpr int WAVES = WN * WK;
+    const int groups = N / (128 * WN);
+    const int total_chunks = K / 128;
+    const int cps = (int)cdiv(total_chunks, split_k);
+    const int splits = (int)cdiv(total_chunks, cps);
+    int* counters = reinterpret_cast<int*>(workspace);
+    float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
+                                                            kCounterBytes)
+                                : nullptr;
+    size_t lds = (size_t)WAVES * dma_wave_bytes(M);
+    const size_t red_bytes = WK > 1 ? (size_t)WAVES * 32 * 64 * sizeof(float) : 0;
+    if (lds < red_bytes) lds = red_bytes;
+    auto kern = gemv_dma_kernel<T, WN, WK>;
+    // what the largest M that still fits asks for (the dispatcher rejects bigger requests)
+    constexpr size_t kLdsCap = 160 * 1024 - 1024;
+    constexpr size_t kMaxLds = (size_t)WAVES * dma_wave_bytes(16) < kLdsCap ? (size_t)WAVES * dma_wave_bytes(16) : kLdsCap;
+    if (kMaxLds > 64 * 1024) {
+        static bool raised = false;  // once per process and instantiation
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
+            if (e != hipSuccess) return e;
+            raised = true;
+        }
+    }
+    (void)hipGetLastError();  // do not report an earlier, unrelated failure as this launch's
+    hipLaunchKernelGGL(kern, dim3(groups, splits), dim3(64 * WAVES), lds, stream,
+                       reinterpret_cast<const uint16_t*>(x),
+                       reinterpret_cast<const uint32_t*>(qweight),
+                       reinterpret_cast<const uint16_t*>(qscales),
+                       reinterpret_cast<const uint32_t*>(qzeros),
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
+                       partials, counters, M, N, K, g / 128, cps, splits);
     return hipGetLastError();
 }
 
@@ -391,6 +629,34 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
     const bool big_chunk = chunk_steps(g) == 4;
+    if (variant >= kFirstDmaVariant) {
+        if (N % (128 * gv.wn) != 0 || g % 128 != 0) {
+            set_error("%s: variant %s needs N %% %d == 0 and group_size %% 128 == 0", fn, gv.name, 128 * gv.wn);
+            return AWQ_ERR_UNSUPPORTED;
+        }
+        if (gv.waves * (8192 + 256 * (int)M + 512) > 160 * 1024 - 1024) {
+            set_error("%s: variant %s does not fit the LDS at M=%lld", fn, gv.name, (long long)M);
+            return AWQ_ERR_UNSUPPORTED;
+        }
+#define AWQ_DMA_CASE(NN, KK)                                                                       \
+    if (gv.wn == NN && gv.waves == NN * KK)                                                        \
+        e = dtype == AWQ_F16                                                                       \
+                ? launch_gemv_dma<F16, NN, KK>(x, qweight, qscales, qzeros, bias, y, (int)M,       \
+                                               (int)N, (int)K, (int)g, workspace, split_k, s)      \
+                : launch_gemv_dma<BF16, NN, KK>(x, qweight, qscales, qzeros, bias, y, (int)M,      \
+                                                (int)N, (int)K, (int)g, workspace, split_k, s);
+        AWQ_DMA_CASE(1, 4)
+        AWQ_DMA_CASE(2, 2)
+        AWQ_DMA_CASE(4, 1)
+        AWQ_DMA_CASE(2, 4)
+        AWQ_DMA_CASE(4, 2)
+        AWQ_DMA_CASE(1, 8)
+        AWQ_DMA_CASE(1, 1)
+        AWQ_DMA_CASE(4, 4)
+        AWQ_DMA_CASE(2, 8)
+#undef AWQ_DMA_CASE
+        return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+    }
 #define AWQ_GEMV_LAUNCH(TT, VV, WW, CC, PP)                                                        \
     launch_gemv<TT, VV, WW, CC, PP>(x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, \
                                     (int)g, workspace, split_k, s)

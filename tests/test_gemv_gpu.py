@@ -52,7 +52,12 @@ def test_gemv_every_variant_and_split(dtype):
         for v in range(L.awq_gemv_variant_count()):
             for split in (1, 2, 5, 32):
                 print(f"gemv variant {L.awq_gemv_variant_name(v).decode()} split={split} M={M} {dtype}", flush=True)
-                y = awq_gemv_variant(xd, *dev, v, split)
+                try:
+                    y = awq_gemv_variant(xd, *dev, v, split)
+                except _lib.AwqHipError as e:
+                    if "does not fit the LDS" in str(e):    # 16-wave staging variants at large M
+                        continue
+                    raise
                 torch.cuda.synchronize()
                 _check(y, xb, p, dtype)
 
