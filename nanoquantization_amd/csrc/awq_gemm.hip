@@ -261,10 +261,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(
         const int m = m0 + idx / wcount;
         const size_t nn = (size_t)n0 + (size_t)(idx % wcount) * 8;
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < splits; ++s) {
-            const float* p = partials + ((size_t)s * M + m) * N + nn;
+        for (int s0 = 0; s0 < splits; s0 += 8) {   // 8 splits in flight, added in split order
+            float v[8][8];
 #pragma unroll
-            for (int c = 0; c < 8; ++c) out[c] += fetch_f32(p + c);
+            for (int u = 0; u < 8; ++u) {
+                const int s = min(s0 + u, splits - 1);
+                const float* p = partials + ((size_t)s * M + m) * N + nn;
+#pragma unroll
+                for (int c = 0; c < 8; ++c) v[u][c] = fetch_f32(p + c);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < splits) {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) out[c] += v[u][c];
+                }
         }
         if (bias) {
             const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);

@@ -234,10 +234,22 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[8 * V], float* red, i
         const int m = idx / w_count, wc = idx - m * w_count;
         const size_t n0 = (size_t)(w_begin + wc) * 8;
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < splits; ++s) {
-            const float* p = partials + ((size_t)s * M + m) * N + n0;
+        // fetch 8 splits at a time so that their loads overlap; add in split order
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+            float v[8][8];
 #pragma unroll
-            for (int c = 0; c < 8; ++c) out[c] += fetch_f32(p + c);
+            for (int u = 0; u < 8; ++u) {
+                const int s = min(s0 + u, splits - 1);
+                const float* p = partials + ((size_t)s * M + m) * N + n0;
+#pragma unroll
+                for (int c = 0; c < 8; ++c) v[u][c] = fetch_f32(p + c);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < splits) {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) out[c] += v[u][c];
+                }
         }
         if (bias) {
             const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
@@ -571,19 +583,38 @@ static size_t gemv_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
 }
 
 // Launch shape for the default entry point.
-static void pick_gemv(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
-    (void)M;
+//
+// The DMA path (N % 128 == 0, group size % 128 == 0) runs one column tile per
+// workgroup with WK waves over K.  Splitting K across workgroups costs a
+// serial tail (publish, arrival counter, fetch: a few microseconds), so it is
+// used only while one workgroup per column tile leaves most SIMDs empty.
+static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, int* split_k) {
     const int64_t chunks = K / 128 > 0 ? K / 128 : 1;
+    if (N % 128 == 0 && g % 128 == 0) {
+        const int64_t tiles = N / 128;
+        // waves per workgroup: 8 while they fit the LDS at this M and have a chunk each
+        int wk = 8;
+        if (chunks < 8 || 8 * (8192 + 256 * M + 512) > 150 * 1024) wk = 4;
+        const int v = wk == 8 ? 15 /* dma1x8 */ : 10 /* dma1x4 */;
+        int64_t s = 1;
+        const int64_t waves = tiles * wk;
+        if (waves < 1024) s = cdiv(1536, waves);       // aim at ~1.5 waves per SIMD
+        const int64_t max_s = chunks / wk > 0 ? chunks / wk : 1;  // at least one chunk per wave
+        if (s > max_s) s = max_s;
+        if (s > 32) s = 32;
+        *variant = v;
+        *split_k = (int)s;
+        return;
+    }
     const bool wide = (N % 16 == 0) && N >= 4096;
     const int v = wide ? 2 /* v2w4 */ : 0 /* v1w4p */;
     const GemvVariant& gv = kGemvVariants[v];
     const int64_t tiles = cdiv(N / 8, 16 * gv.V);
-    // aim at ~2 workgroups of 4 waves per CU, but never less than one chunk per wave
     int64_t s = cdiv(512, tiles);
     const int64_t max_s = chunks / gv.waves > 0 ? chunks / gv.waves : 1;
     if (s > max_s) s = max_s;
     if (s < 1) s = 1;
-    if (s > 64) s = 64;
+    if (s > 32) s = 32;
     *variant = v;
     *split_k = (int)s;
 }
@@ -703,8 +734,12 @@ extern "C" size_t awq_gemv_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, i
 extern "C" size_t awq_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (K < 32 || N < 8 || M < 1) return 0;
     int v, s;
-    awq::pick_gemv(M, N, K, &v, &s);
-    return awq::gemv_ws_bytes(M, N, K, v, s);
+    // the caller does not pass the group size here: cover both data paths
+    awq::pick_gemv(M, N, K, 128, &v, &s);
+    const size_t a = awq::gemv_ws_bytes(M, N, K, v, s);
+    awq::pick_gemv(M, N, K, 32, &v, &s);
+    const size_t b = awq::gemv_ws_bytes(M, N, K, v, s);
+    return a > b ? a : b;
 }
 
 extern "C" int awq_gemv_ex(const void* x, const int32_t* qweight, const void* qscales,
@@ -721,7 +756,7 @@ extern "C" int awq_gemv(const void* x, const int32_t* qweight, const void* qscal
                         int64_t K, int64_t group_size, int dtype, void* workspace,
                         size_t workspace_bytes, void* stream) {
     int v = 0, s = 1;
-    if (K >= 32 && N >= 8) awq::pick_gemv(M, N, K, &v, &s);
+    if (K >= 32 && N >= 8 && group_size > 0) awq::pick_gemv(M, N, K, group_size, &v, &s);
     return awq::gemv_dispatch("awq_gemv", x, qweight, qscales, qzeros, bias, y, M, N, K, group_size,
                               dtype, workspace, workspace_bytes, stream, v, s);
 }
