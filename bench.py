@@ -1,0 +1,257 @@
+#!/usr/bin/env python3
+"""Benchmark of the AWQ W4A16 linear path on one MI355X.
+
+Headline (`value`): packed-weight GB/s of the decode GEMV sweep -- M in {1,2,4,8,16} over every
+Qwen3-0.6B linear shape, fp16, g=128 -- streaming from HBM: one step walks LAYERS distinct copies of
+the 7 linears of a block (LAYERS * 8.17 MB of packed weights, more than twice the 256 MB Infinity
+Cache) once per M.  The step is captured in a HIP graph (the form a decode loop runs in); the eager
+number is reported next to it.
+
+Also on the JSON line: `roofline` for the GEMV kernel of that sweep, `cpu_baseline` (the torch
+restatement of the reference path on the host cores, bounded sample), and -- as extra objects, not the
+headline -- the same GEMV on the Qwen3-32B MLP shapes where a launch is long enough to be HBM-bound,
+the prefill GEMM TFLOP/s at the Qwen3-8B MLP shapes, the dequantise kernel, and config 1's latency.
+
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16, published
+QWEN3_0P6B = [("q", 1024, 2048), ("k", 1024, 1024), ("v", 1024, 1024), ("o", 2048, 1024),
+              ("gate", 1024, 3072), ("up", 1024, 3072), ("down", 3072, 1024)]
+DECODE_MS = (1, 2, 4, 8, 16)
+G = 128
+
+
+def packed_bytes(K, N, g=G):
+    return K * N // 2 + (K // g) * N // 2 + 2 * (K // g) * N
+
+
+def rand_packed(K, N, tdt, dev, g=G):
+    """Random nibbles/zeros/scales straight on the device (bandwidth does not depend on the values)."""
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device=dev)
+    qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, device=dev)
+    sc = (torch.rand(K // g, N, device=dev) * 0.02 + 0.001).to(tdt)
+    return qw, sc, qz
+
+
+def time_graph(fn, steps, warmup):
+    """Capture fn() once on a side stream, replay `steps` times between two events on that stream."""
+    s = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        fn()                              # allocations (outputs, workspace) happen before capture
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=s):
+            fn()
+        torch.cuda.synchronize()
+        for _ in range(warmup):
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(s)
+        for _ in range(steps):
+            g.replay()
+        e1.record(s)
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps    # ms per step
+
+
+def time_eager(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=64, help="distinct weight copies of one block per step")
+    ap.add_argument("--quick", action="store_true", help="skip the extra (non-headline) measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the AWQ linear path has no multi-GPU part); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        sys.exit(1)
+
+    from nanoquantization_amd import _lib
+    import nanoquantization_amd as nq
+    if not os.path.exists(_lib.LIB_PATH):
+        from nanoquantization_amd.build import build
+        build(verbose=False)
+    _lib.lib()
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tdt = torch.float16
+    torch.manual_seed(0)
+
+    # ---------------- headline: decode GEMV sweep, streaming ----------------------------------------------
+    layers = [[rand_packed(K, N, tdt, dev) for (_, K, N) in QWEN3_0P6B] for _ in range(args.layers)]
+    xs = {(M, K): torch.randn(M, K, device=dev).to(tdt) for M in DECODE_MS for K in (1024, 2048, 3072)}
+    bytes_per_pass = sum(packed_bytes(K, N) for (_, K, N) in QWEN3_0P6B) * args.layers
+    launches_per_step = len(DECODE_MS) * len(QWEN3_0P6B) * args.layers
+    bytes_per_step = bytes_per_pass * len(DECODE_MS)
+
+    def sweep_step():
+        for M in DECODE_MS:
+            for layer in layers:
+                for (qw, sc, qz), (_, K, N) in zip(layer, QWEN3_0P6B):
+                    nq.awq_gemm(xs[(M, K)], qw, sc, qz, 8)
+
+    ms_graph = time_graph(sweep_step, args.steps, args.warmup)
+    ms_eager = time_eager(sweep_step, max(2, args.steps // 4), 1)
+    value = bytes_per_step / (ms_graph * 1e-3) / 1e9
+    avg_launch_us = ms_graph * 1e3 / launches_per_step
+    avg_bytes = bytes_per_step / launches_per_step
+    roofline = {
+        "kernel": "awq::gemv_dma_kernel<F16,1,4|8>", "bound": "hbm",
+        "achieved": avg_bytes / (avg_launch_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+        "avg_launch_us": avg_launch_us, "algorithmic_bytes_per_launch": avg_bytes,
+        "note": "packed-weight bytes (0.5195 B/weight) / HIP-event time per launch over the timed graph replays; "
+                "0.5-1.6 MB per launch: latency-bound, see roofline_large for the HBM-bound regime",
+    }
+
+    # per-shape hot-cache numbers (single buffer, stays in L2 / Infinity Cache), labelled as such
+    per_shape = {}
+    for (name, K, N), w in zip(QWEN3_0P6B, layers[0]):
+        for M in (1, 16):
+            fn = lambda: [nq.awq_gemm(xs[(M, K)], *w, 8) for _ in range(50)]
+            us = time_graph(fn, 5, 1) * 1e3 / 50
+            per_shape[f"{name}_{K}x{N}_M{M}"] = {"hot_us": round(us, 2),
+                                                   "hot_GBs": round(packed_bytes(K, N) / us / 1e3, 1)}
+    del layers
+    torch.cuda.empty_cache()
+
+    out = {
+        "metric": "W4A16 GEMM TFLOP/s & weight GB/s vs roofline; Qwen3-0.6B decode tok/s",
+        "value": value, "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_graph,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "cfg2: decode GEMV sweep, M in {1,2,4,8,16} x Qwen3-0.6B linear shapes "
+                               "(q 1024x2048, k/v 1024x1024, o 2048x1024, gate/up 1024x3072, down 3072x1024), "
+                               "fp16 x ~N(0,1), AWQ-packed g=128",
+                   "distinct_weight_copies": args.layers, "launches_per_step": launches_per_step,
+                   "packed_bytes_per_step": bytes_per_step, "launch": "HIP graph replay",
+                   "eager_GBs": bytes_per_step / (ms_eager * 1e-3) / 1e9, "eager_ms_per_step": ms_eager},
+        "roofline": roofline,
+        "per_shape_hot_cache": per_shape,
+    }
+
+    if not args.quick:
+        # ---------------- extra: HBM-bound GEMV at the Qwen3-32B MLP shapes -----------------------------
+        large = {}
+        for (K, N) in ((5120, 25600), (25600, 5120)):
+            copies = [rand_packed(K, N, tdt, dev) for _ in range(6)]   # 6 x 68 MB > Infinity Cache
+            for M in (1, 16):
+                x = torch.randn(M, K, device=dev).to(tdt)
+                fn = lambda: [nq.awq_gemm(x, *w, 8) for w in copies]
+                us = time_graph(fn, 10, 2) * 1e3 / len(copies)
+                gbs = packed_bytes(K, N) / us / 1e3
+                large[f"{K}x{N}_M{M}"] = {"us": round(us, 2), "GBs": round(gbs, 1), "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4)}
+            del copies
+            torch.cuda.empty_cache()
+        best = max(v["GBs"] for v in large.values())
+        out["roofline_large"] = {"kernel": "awq::gemv_dma_kernel", "bound": "hbm", "achieved": best,
+                                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best / HBM_PEAK_GBS,
+                                 "workload": "Qwen3-32B MLP shapes (68.1 MB packed), HBM-streaming over 6 copies",
+                                 "cases": large}
+
+        # ---------------- extra: prefill fused dequant + MFMA GEMM, cfg3 --------------------------------
+        prefill = {}
+        bdt = torch.bfloat16
+        for (K, N) in ((4096, 12288), (12288, 4096)):
+            w = rand_packed(K, N, bdt, dev)
+            for M in (512, 2048, 8192):
+                x = torch.randn(M, K, device=dev).to(bdt)
+                fn = lambda: [nq.awq_gemm(x, *w, 8) for _ in range(4)]
+                us = time_graph(fn, 5, 1) * 1e3 / 4
+                tf = 2.0 * M * N * K / us / 1e6
+                prefill[f"M{M}_{K}x{N}"] = {"us": round(us, 1), "TFLOPs": round(tf, 1),
+                                             "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4)}
+            del w
+        bestp = max(v["TFLOPs"] for v in prefill.values())
+        out["roofline_prefill"] = {"kernel": "awq::gemm_kernel<BF16,...>", "bound": "mfma", "achieved": bestp,
+                                   "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": bestp / MFMA_PEAK_TFLOPS,
+                                   "workload": "cfg3: Qwen3-8B MLP shapes, bf16, M in {512,2048,8192}", "cases": prefill}
+
+        # ---------------- extra: dequantise kernel ------------------------------------------------------
+        K, N = 4096, 12288
+        copies = [rand_packed(K, N, bdt, dev) for _ in range(4)]
+        fn = lambda: [nq.awq_dequantize(*w) for w in copies]
+        us = time_graph(fn, 10, 2) * 1e3 / len(copies)
+        db = packed_bytes(K, N) + 2 * K * N
+        out["dequant"] = {"shape": f"{K}x{N} bf16", "us": round(us, 1), "GBs": round(db / us / 1e3, 1),
+                          "frac_of_8TBs": round(db / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": db}
+        del copies
+        torch.cuda.empty_cache()
+
+        # ---------------- extra: cfg1 latency -----------------------------------------------------------
+        w = rand_packed(1024, 3072, tdt, dev)
+        x = torch.randn(16, 1024, device=dev).to(tdt)
+        fn = lambda: [nq.awq_gemm(x, *w, 8) for _ in range(50)]
+        out["cfg1_single_linear"] = {"shape": "x[16,1024] @ W[1024,3072]", "graph_us": round(time_graph(fn, 5, 1) * 1e3 / 50, 2),
+                                     "eager_us": round(time_eager(lambda: nq.awq_gemm(x, *w, 8), 200, 20) * 1e3, 2)}
+
+    # ---------------- CPU baseline: the reference's path restated on host tensors (bounded sample) ----------
+    if not args.no_cpu:
+        from oracle import torch_cpu_path as cpu
+        torch.set_num_threads(os.cpu_count() or 1)
+        K, N, M = 1024, 3072, 16
+        qw, sc, qz = [t.cpu() for t in rand_packed(K, N, tdt, dev)]
+        xc = torch.randn(M, K).to(tdt)
+        t_end = time.time() + 12.0
+        times_native, times_up, times_dq = [], [], []
+        for _ in range(3):
+            cpu.linear(xc, qw, sc, qz, upcast=True)
+        while time.time() < t_end and len(times_up) < 200:
+            t0 = time.perf_counter(); wd = cpu.dequant(qw, sc, qz); t1 = time.perf_counter()
+            torch.matmul(xc.float(), wd.float()).to(tdt); t2 = time.perf_counter()
+            times_dq.append(t1 - t0); times_up.append(t2 - t0)
+        t_end = time.time() + 6.0
+        while time.time() < t_end and len(times_native) < 50:
+            t0 = time.perf_counter(); cpu.linear(xc, qw, sc, qz, upcast=False); times_native.append(time.perf_counter() - t0)
+        med = lambda v: sorted(v)[len(v) // 2]
+        t_up = med(times_up)
+        out["cpu_baseline"] = {
+            "value": packed_bytes(K, N) / t_up / 1e9, "unit": "GB/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"cfg1 single linear x[16,1024] @ W[1024,3072] fp16 g=128, torch unpack + (q-z)*s + matmul on CPU "
+                      f"tensors, fp32-upcast matmul, median of {len(times_up)} iterations",
+            "ms_total_fp32_upcast": t_up * 1e3, "ms_dequant": med(times_dq) * 1e3,
+            "ms_total_native_fp16": med(times_native) * 1e3 if times_native else None,
+            "TFLOPs": 2.0 * M * N * K / t_up / 1e12, "os_cpu_count": os.cpu_count(),
+        }
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
