@@ -89,6 +89,11 @@ struct BF16 {
 __device__ __forceinline__ void publish_f32(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// 16-byte form of publish_f32.  The store is invisible to the compiler's wait-count
+// bookkeeping, which is why arrive_last waits for vmcnt = 0 explicitly.
+__device__ __forceinline__ void publish_f32x4(float* p, f32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
 __device__ __forceinline__ float fetch_f32(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -97,6 +102,7 @@ __device__ __forceinline__ float fetch_f32(const float* p) {
 // counter; returns true in the workgroup that arrived last.
 __device__ __forceinline__ bool arrive_last(int* counter, int splits, int* s_flag) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): also covers the inline-asm stores of publish_f32x4
     __syncthreads();
     if (threadIdx.x == 0) {
         const int prev = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -51,13 +51,15 @@ template <typename T>
 struct Embed;
 template <>
 struct Embed<F16> {
-    // 0x6400 | q<<4 = 1024 + 16 q for both nibbles
-    static constexpr uint32_t kMaskLo = 0x00F000F0u, kMagicLo = 0x64006400u;
+    // low nibble: 0x6400 | q = 1024 + q; high nibble: 0x6400 | q<<4 = 1024 + 16 q.  No shifts.
+    // The 1024 offset costs ~8 of fp32's 24 bits when it is subtracted again per group
+    // (|sum x*(q-z)| is ~2^-8 of |1024*sum x|), leaving ~2^-16 relative error on a group sum.
+    static constexpr uint32_t kMaskLo = 0x000F000Fu, kMagicLo = 0x64006400u;
     static constexpr uint32_t kMaskHi = 0x00F000F0u, kMagicHi = 0x64006400u;
-    static constexpr float kMul = 16.f, kOffLo = 1024.f, kOffHi = 1024.f;
-    static __device__ __forceinline__ uint32_t pre_lo(uint32_t p) { return p << 4; }
+    static constexpr float kOffLo = 1024.f, kOffHi = 1024.f;
+    static __device__ __forceinline__ uint32_t pre_lo(uint32_t p) { return p; }
     static __device__ __forceinline__ uint32_t pre_hi(uint32_t p) { return p; }
-    static constexpr float kMulLo = 16.f, kMulHi = 16.f;
+    static constexpr float kMulLo = 1.f, kMulHi = 16.f;
 };
 template <>
 struct Embed<BF16> {
@@ -219,8 +221,8 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[8 * V], float* red, i
                 *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
             } else {
                 float* p = partials + ((size_t)split * M + m) * N + n0;
-#pragma unroll
-                for (int c = 0; c < 8; ++c) publish_f32(p + c, out[c]);
+                publish_f32x4(p, f32x4{out[0], out[1], out[2], out[3]});
+                publish_f32x4(p + 4, f32x4{out[4], out[5], out[6], out[7]});
             }
         }
     }
@@ -371,7 +373,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
 
 __host__ __device__ constexpr int dma_wave_bytes(int M) { return 8192 + 256 * M + 512; }
 
-template <typename T, int WN, int WK>
+template <typename T, int WN, int WK, int DEPTH>
 __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
@@ -396,10 +398,10 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const int c0 = c_begin + (wave / WN) * per_wave;
     const int c1 = min(c0 + per_wave, c_end);
 
-    char* stage = reinterpret_cast<char*>(red) + (size_t)wave * dma_wave_bytes(M);
-    uint32_t* w_lds = reinterpret_cast<uint32_t*>(stage);
-    char* x_lds = stage + 8192;
-    char* zs_lds = stage + 8192 + 256 * M;
+    // DEPTH staging buffers per wave: chunk c lives in buffer (c - c0) % DEPTH
+    const int buf_bytes = dma_wave_bytes(M);
+    char* stage = reinterpret_cast<char*>(red) + (size_t)wave * (DEPTH * buf_bytes);
+    const int x_off = 8192, zs_off = 8192 + 256 * M;
 
     // DMA lane roles
     const int dq = lane & 3, dsl = lane >> 2;  // 16-byte quarter of the 64-byte row piece, slot % 16
@@ -414,8 +416,16 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const bool zs_lane = lane < 16;
     const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
 
-    auto issue_dma = [&](int c) {
+    // exactly kDmaOps vector-memory instructions per call (the vmcnt arithmetic below counts on it):
+    // lanes 0..3 and 0..15 exist in every wave, so neither guarded block is ever skipped
+    constexpr int kDmaOps = 2 * CH + CH + 2;
+    static_assert(kDmaOps == 14, "vmcnt immediates below assume 14 DMA instructions per chunk");
+    auto issue_dma = [&](int c, int buf) {
         const int row0 = c * 128;
+        char* base = stage + buf * buf_bytes;
+        uint32_t* w_lds = reinterpret_cast<uint32_t*>(base);
+        char* x_lds = base + x_off;
+        char* zs_lds = base + zs_off;
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
             const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
@@ -438,36 +448,46 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         }
     };
 
-    // compute-lane read positions
-    const uint32_t* w_rd = w_lds + kb * 16 + j;                     // + s*512 + r*64
+    // compute-lane read offsets inside a staging buffer (bytes)
     const int xm = j < M ? j : M - 1;
-    const u32x4* x_rd = reinterpret_cast<const u32x4*>(x_lds) + xm * 4 + kb;  // + s*4*M
-    const uint32_t* z_rd = reinterpret_cast<const uint32_t*>(zs_lds) + j;
-    const u32x4* s_rd = reinterpret_cast<const u32x4*>(zs_lds + 64) + j;
+    const int w_rd_off = (kb * 16 + j) * 4;                   // + (s*512 + r*64) * 4
+    const int x_rd_off = x_off + (xm * 4 + kb) * 16;          // + s * 64 * M
+    const int z_rd_off = zs_off + j * 4;
+    const int s_rd_off = zs_off + 64 + j * 16;
 
     f32x4 acc[8];
 #pragma unroll
     for (int f = 0; f < 8; ++f) acc[f] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    if (c0 < c1) issue_dma(c0);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (c0 + d < c1) issue_dma(c0 + d, d);
+    int buf = 0;
     for (int c = c0; c < c1; ++c) {
-        // the DMA of chunk c has landed: vmcnt(0); the compiler does not order LDS reads after it by itself
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+        // chunk c has landed once at most the DMA of the chunks issued after it is outstanding.
+        // The compiler does not order LDS reads after the DMA by itself.
+        const int newer = min(c1 - 1 - c, DEPTH - 1);
+        if (DEPTH == 1 || newer == 0) __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
+        else if (newer == 1) __builtin_amdgcn_s_waitcnt(0x0F7E);                 // vmcnt(14)
+        else __builtin_amdgcn_s_waitcnt(0x4F7C);                                 // vmcnt(28)
         asm volatile("" ::: "memory");
+        const char* base = stage + buf * buf_bytes;
+        const uint32_t* w_rd = reinterpret_cast<const uint32_t*>(base + w_rd_off);
         Chunk<1, CH> d;
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) d.w[s][r] = w_rd[s * 512 + r * 64];
-            d.xa[s] = x_rd[s * 4 * M];
+            d.xa[s] = *reinterpret_cast<const u32x4*>(base + x_rd_off + s * 64 * M);
         }
-        d.zw = *z_rd;
-        d.sv[0] = *s_rd;
-        // every LDS read has returned before the next chunk's DMA may overwrite the staging area
+        d.zw = *reinterpret_cast<const uint32_t*>(base + z_rd_off);
+        d.sv[0] = *reinterpret_cast<const u32x4*>(base + s_rd_off);
+        // every LDS read has returned before a later chunk's DMA may overwrite this buffer
         asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_waitcnt(0xC07F);                                      // lgkmcnt(0)
         asm volatile("" ::: "memory");
-        if (c + 1 < c1) issue_dma(c + 1);
+        if (c + DEPTH < c1) issue_dma(c + DEPTH, buf);
+        buf = (buf + 1 == DEPTH) ? 0 : buf + 1;
         compute_chunk<T, 1, CH>(d, acc);
     }
     __syncthreads();  // staging area becomes the reduction buffer
@@ -480,20 +500,22 @@ struct GemvVariant {
     const char* name;
     int V, waves;
     bool prefetch;
-    int wn;  // waves side by side along N (DMA variants), 1 otherwise
+    int wn;     // waves side by side along N (DMA variants), 1 otherwise
+    int depth;  // DMA staging buffers per wave (DMA variants), 0 otherwise
 };
 static const GemvVariant kGemvVariants[] = {
-    {"v1w4p", 1, 4, true, 1},  {"v1w8p", 1, 8, true, 1},   {"v2w4", 2, 4, false, 1},
-    {"v2w8", 2, 8, false, 1},  {"v2w4p", 2, 4, true, 1},   {"v1w16", 1, 16, false, 1},
-    {"v1w1p", 1, 1, true, 1},  {"v2w1", 2, 1, false, 1},   {"v1w4", 1, 4, false, 1},
-    {"v1w8", 1, 8, false, 1},
-    // DMA variants, named dma<WN>x<WK>
-    {"dma1x4", 1, 4, false, 1}, {"dma2x2", 1, 4, false, 2}, {"dma4x1", 1, 4, false, 4},
-    {"dma2x4", 1, 8, false, 2}, {"dma4x2", 1, 8, false, 4}, {"dma1x8", 1, 8, false, 1},
-    {"dma1x1", 1, 1, false, 1}, {"dma4x4", 1, 16, false, 4}, {"dma2x8", 1, 16, false, 2},
+    {"v1w4p", 1, 4, true, 1, 0},  {"v1w8p", 1, 8, true, 1, 0},   {"v2w4", 2, 4, false, 1, 0},
+    {"v2w8", 2, 8, false, 1, 0},  {"v2w4p", 2, 4, true, 1, 0},   {"v1w16", 1, 16, false, 1, 0},
+    {"v1w1p", 1, 1, true, 1, 0},  {"v2w1", 2, 1, false, 1, 0},   {"v1w4", 1, 4, false, 1, 0},
+    {"v1w8", 1, 8, false, 1, 0},
+    // DMA variants, named dma<WN>x<WK>d<DEPTH>
+    {"dma1x4d1", 1, 4, false, 1, 1},  {"dma1x8d1", 1, 8, false, 1, 1},  {"dma1x16d1", 1, 16, false, 1, 1},
+    {"dma1x4d2", 1, 4, false, 1, 2},  {"dma1x8d2", 1, 8, false, 1, 2},  {"dma1x4d3", 1, 4, false, 1, 3},
+    {"dma2x4d1", 1, 8, false, 2, 1},  {"dma2x4d2", 1, 8, false, 2, 2},  {"dma1x1d1", 1, 1, false, 1, 1},
+    {"dma1x2d2", 1, 2, false, 1, 2},
 };
-constexpr int kFirstDmaVariant = 10;
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
+constexpr int kFirstDmaVariant = 10;
 
 // rows per chunk: 128 when the group size allows it, else 32
 static inline int chunk_steps(int64_t g) { return g % 128 == 0 ? 4 : 1; }
@@ -534,7 +556,7 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
     return hipGetLastError();
 }
 
-template <typename T, int WN, int WK>
+template <typename T, int WN, int WK, int DEPTH>
 static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                                   int g, void* workspace, int split_k, hipStream_t stream) {
@@ -547,13 +569,14 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
                                                             kCounterBytes)
                                 : nullptr;
-    size_t lds = (size_t)WAVES * dma_wave_bytes(M);
+    size_t lds = (size_t)WAVES * DEPTH * dma_wave_bytes(M);
     const size_t red_bytes = WK > 1 ? (size_t)WAVES * 32 * 64 * sizeof(float) : 0;
     if (lds < red_bytes) lds = red_bytes;
-    auto kern = gemv_dma_kernel<T, WN, WK>;
+    auto kern = gemv_dma_kernel<T, WN, WK, DEPTH>;
     // what the largest M that still fits asks for (the dispatcher rejects bigger requests)
     constexpr size_t kLdsCap = 160 * 1024 - 1024;
-    constexpr size_t kMaxLds = (size_t)WAVES * dma_wave_bytes(16) < kLdsCap ? (size_t)WAVES * dma_wave_bytes(16) : kLdsCap;
+    constexpr size_t kWant = (size_t)WAVES * DEPTH * dma_wave_bytes(16);
+    constexpr size_t kMaxLds = kWant < kLdsCap ? kWant : kLdsCap;
     if (kMaxLds > 64 * 1024) {
         static bool raised = false;  // once per process and instantiation
         if (!raised) {
@@ -591,17 +614,23 @@ static size_t gemv_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
 static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, int* split_k) {
     const int64_t chunks = K / 128 > 0 ? K / 128 : 1;
     if (N % 128 == 0 && g % 128 == 0) {
+        // From sweeps on MI355X (HBM-streaming): short K runs best as one workgroup of 8 waves per
+        // column tile; otherwise 4-wave workgroups, split over K for M <= 4 until ~3000 waves exist
+        // (the split's serial tail grows with M, so larger M splits only to cover the CUs).
         const int64_t tiles = N / 128;
-        // waves per workgroup: 8 while they fit the LDS at this M and have a chunk each
-        int wk = 8;
-        if (chunks < 8 || 8 * (8192 + 256 * M + 512) > 150 * 1024) wk = 4;
-        const int v = wk == 8 ? 15 /* dma1x8 */ : 10 /* dma1x4 */;
+        int v = 10 /* dma1x4d1 */;
         int64_t s = 1;
-        const int64_t waves = tiles * wk;
-        if (waves < 1024) s = cdiv(1536, waves);       // aim at ~1.5 waves per SIMD
-        const int64_t max_s = chunks / wk > 0 ? chunks / wk : 1;  // at least one chunk per wave
-        if (s > max_s) s = max_s;
-        if (s > 32) s = 32;
+        if (chunks <= 8) {
+            v = 11 /* dma1x8d1 */;
+        } else if (M <= 4) {
+            s = cdiv(3072, tiles * 4);
+            const int64_t cap = chunks / 2 < 10 ? chunks / 2 : 10;
+            if (s > cap) s = cap;
+        } else if (tiles * 4 < 512) {
+            s = cdiv(512, tiles * 4);
+            if (s > chunks / 4) s = chunks / 4;
+        }
+        if (s < 1) s = 1;
         *variant = v;
         *split_k = (int)s;
         return;
@@ -665,26 +694,27 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
             set_error("%s: variant %s needs N %% %d == 0 and group_size %% 128 == 0", fn, gv.name, 128 * gv.wn);
             return AWQ_ERR_UNSUPPORTED;
         }
-        if (gv.waves * (8192 + 256 * (int)M + 512) > 160 * 1024 - 1024) {
+        if ((size_t)gv.waves * gv.depth * dma_wave_bytes((int)M) > 160 * 1024 - 1024) {
             set_error("%s: variant %s does not fit the LDS at M=%lld", fn, gv.name, (long long)M);
             return AWQ_ERR_UNSUPPORTED;
         }
-#define AWQ_DMA_CASE(NN, KK)                                                                       \
-    if (gv.wn == NN && gv.waves == NN * KK)                                                        \
-        e = dtype == AWQ_F16                                                                       \
-                ? launch_gemv_dma<F16, NN, KK>(x, qweight, qscales, qzeros, bias, y, (int)M,       \
-                                               (int)N, (int)K, (int)g, workspace, split_k, s)      \
-                : launch_gemv_dma<BF16, NN, KK>(x, qweight, qscales, qzeros, bias, y, (int)M,      \
-                                                (int)N, (int)K, (int)g, workspace, split_k, s);
-        AWQ_DMA_CASE(1, 4)
-        AWQ_DMA_CASE(2, 2)
-        AWQ_DMA_CASE(4, 1)
-        AWQ_DMA_CASE(2, 4)
-        AWQ_DMA_CASE(4, 2)
-        AWQ_DMA_CASE(1, 8)
-        AWQ_DMA_CASE(1, 1)
-        AWQ_DMA_CASE(4, 4)
-        AWQ_DMA_CASE(2, 8)
+#define AWQ_DMA_CASE(NN, KK, DD)                                                                    \
+    if (gv.wn == NN && gv.waves == NN * KK && gv.depth == DD)                                       \
+        e = dtype == AWQ_F16                                                                        \
+                ? launch_gemv_dma<F16, NN, KK, DD>(x, qweight, qscales, qzeros, bias, y, (int)M,    \
+                                                   (int)N, (int)K, (int)g, workspace, split_k, s)   \
+                : launch_gemv_dma<BF16, NN, KK, DD>(x, qweight, qscales, qzeros, bias, y, (int)M,   \
+                                                    (int)N, (int)K, (int)g, workspace, split_k, s);
+        AWQ_DMA_CASE(1, 4, 1)
+        AWQ_DMA_CASE(1, 8, 1)
+        AWQ_DMA_CASE(1, 16, 1)
+        AWQ_DMA_CASE(1, 4, 2)
+        AWQ_DMA_CASE(1, 8, 2)
+        AWQ_DMA_CASE(1, 4, 3)
+        AWQ_DMA_CASE(2, 4, 1)
+        AWQ_DMA_CASE(2, 4, 2)
+        AWQ_DMA_CASE(1, 1, 1)
+        AWQ_DMA_CASE(1, 2, 2)
 #undef AWQ_DMA_CASE
         return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
     }
