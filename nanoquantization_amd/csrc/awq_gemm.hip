@@ -94,24 +94,28 @@ __device__ __forceinline__ int b_slot(int wc, int c, int kblk) {
 }
 
 template <typename T, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(256) void gemm_kernel(
+__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int g, int iters_per_split, int splits) {
-    static_assert(WM * WN == 4, "4 wavefronts per workgroup");
+    constexpr int NW = WM * WN, NT = 64 * NW;
+    static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts per workgroup");
     static_assert(BN == 256 || BN == 128, "BN is 128 or 256");
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     static_assert(TM >= 1 && TN >= 1, "wave tile at least 32x32");
-    constexpr int UR = BN / 32;          // k rows per lane per step: 8 (BN=256) or 4 (BN=128)
-    constexpr int WCOLS = BN / 8;        // packed word columns per tile
-    constexpr int ACH = BM / 32;         // 16-byte A chunks per thread per step
+    constexpr int WCOLS = BN / 8;                  // packed word columns per tile
+    constexpr int UR = kBK * WCOLS / NT;           // k rows per lane per step
+    static_assert(UR == 8 || UR == 4 || UR == 2, "a lane unpacks 2, 4 or 8 rows of one word column");
+    constexpr int ACH = BM * 8 / NT;               // 16-byte A chunks per thread per step
+    static_assert(ACH >= 1, "at least one A chunk per thread");
     constexpr int A_SLOTS = 8 * BM, B_SLOTS = 8 * BN;
 
     extern __shared__ u32x4 lds[];  // [2][A_SLOTS + B_SLOTS]
     __shared__ int s_last;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int split = blockIdx.z;
@@ -120,10 +124,22 @@ __global__ __launch_bounds__(256) void gemm_kernel(
     const int it_begin = split * iters_per_split;
     const int it_end = min(it_begin + iters_per_split, total_iters);
 
-    // B loader coordinates
+    // ---- loader coordinates (rows / columns past the edge read a valid neighbour; their
+    //      results are never stored) -------------------------------------------------------------
+    const uint16_t* a_src[ACH];
+    int a_dst[ACH];
+#pragma unroll
+    for (int i = 0; i < ACH; ++i) {
+        const int id = tid + NT * i;
+        const int row = id >> 3, kc = id & 7;
+        a_src[i] = x + (size_t)min(m0 + row, M - 1) * K + kc * 8;
+        a_dst[i] = a_slot<BM>(row, kc);
+    }
     const int wc = tid % WCOLS, rb = tid / WCOLS;  // word column, row block (UR rows)
-    const int gwc = (n0 >> 3) + wc;
-    const bool wc_ok = gwc < words;
+    const int gwc = min((n0 >> 3) + wc, words - 1);
+    const uint32_t w_off = (uint32_t)(rb * UR) * (uint32_t)words + (uint32_t)gwc;
+    // group of row k0 + rb*UR: k0/g + (rb*UR)/g (host guarantees g % 64 == 0 or 64 % g == 0)
+    const int g_lane = (rb * UR) / g;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -141,37 +157,20 @@ __global__ __launch_bounds__(256) void gemm_kernel(
     auto load_global = [&](int it) {
         const int k0 = it * kBK;
 #pragma unroll
-        for (int i = 0; i < ACH; ++i) {
-            const int id = tid + 256 * i;
-            const int row = id >> 3, kc = id & 7;
-            if (m0 + row < M)
-                areg[i] = *reinterpret_cast<const u32x4*>(x + (size_t)(m0 + row) * K + k0 + kc * 8);
-            else
-                areg[i] = u32x4{0u, 0u, 0u, 0u};
-        }
-        const int krow = k0 + rb * UR;
-        if (wc_ok) {
+        for (int i = 0; i < ACH; ++i) areg[i] = *reinterpret_cast<const u32x4*>(a_src[i] + k0);
+        const uint32_t* wp = qweight + (size_t)k0 * words;  // uniform
 #pragma unroll
-            for (int r = 0; r < UR; ++r) wreg[r] = qweight[(size_t)(krow + r) * words + gwc];
-            const int gi = krow / g;
-            zreg = qzeros[(size_t)gi * words + gwc];
-            sreg = *reinterpret_cast<const u32x4*>(scales + (size_t)gi * N + (size_t)gwc * 8);
-        } else {
-#pragma unroll
-            for (int r = 0; r < UR; ++r) wreg[r] = 0u;
-            zreg = 0u;
-            sreg = u32x4{0u, 0u, 0u, 0u};
-        }
+        for (int r = 0; r < UR; ++r) wreg[r] = (wp + (size_t)r * words)[w_off];
+        const int gi = k0 / g + g_lane;
+        zreg = qzeros[(size_t)gi * words + gwc];
+        sreg = *reinterpret_cast<const u32x4*>(scales + ((size_t)gi * words + gwc) * 8);
     };
 
     auto store_lds = [&](int buf) {
         u32x4* abase = lds + buf * (A_SLOTS + B_SLOTS);
         u32x4* bbase = abase + A_SLOTS;
 #pragma unroll
-        for (int i = 0; i < ACH; ++i) {
-            const int id = tid + 256 * i;
-            abase[a_slot<BM>(id >> 3, id & 7)] = areg[i];
-        }
+        for (int i = 0; i < ACH; ++i) abase[a_dst[i]] = areg[i];
         UnpackRows<T> up;
         up.set_group(zreg, sreg);
         uint32_t cols[8][UR / 2];
@@ -182,33 +181,44 @@ __global__ __launch_bounds__(256) void gemm_kernel(
 #pragma unroll
             for (int c = 0; c < 8; ++c) cols[c][rp] = o[c];
         }
+        constexpr int PER_BLK = 8 / UR;  // lanes sharing one 16-byte slot
+        const int kblk = rb / PER_BLK, sub = rb % PER_BLK;
         if constexpr (UR == 8) {
 #pragma unroll
             for (int c = 0; c < 8; ++c)
-                bbase[b_slot<BN>(wc, c, rb)] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
-        } else {  // UR == 4: two lanes share a 16-byte slot, 8 bytes each
+                bbase[b_slot<BN>(wc, c, kblk)] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
+        } else if constexpr (UR == 4) {
             u32x2* b2 = reinterpret_cast<u32x2*>(bbase);
 #pragma unroll
-            for (int c = 0; c < 8; ++c)
-                b2[b_slot<BN>(wc, c, rb >> 1) * 2 + (rb & 1)] = u32x2{cols[c][0], cols[c][1]};
+            for (int c = 0; c < 8; ++c) b2[b_slot<BN>(wc, c, kblk) * 2 + sub] = u32x2{cols[c][0], cols[c][1]};
+        } else {
+            uint32_t* b1 = reinterpret_cast<uint32_t*>(bbase);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) b1[b_slot<BN>(wc, c, kblk) * 4 + sub] = cols[c][0];
         }
     };
 
+    // ---- MFMA operand addresses, hoisted: only the k-step changes inside the loop -------------------
     const int li = lane & 31, kb2 = lane >> 5;
+    int a_rd[kBK / 16];  // slot of A row wm0 + li at k-block 2*ks + kb2; + a*32 for the other tiles
+#pragma unroll
+    for (int ks = 0; ks < kBK / 16; ++ks) a_rd[ks] = a_slot<BM>(wm0 + li, ks * 2 + kb2);
+    int b_rd[TN];        // slot of B column wn0 + b*32 + li at k-block kb2; + ks*2*BN
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+        const int n = wn0 + b * 32 + li;
+        b_rd[b] = b_slot<BN>(n >> 3, n & 7, kb2);
+    }
     auto compute = [&](int buf) {
         const u32x4* abase = lds + buf * (A_SLOTS + B_SLOTS);
         const u32x4* bbase = abase + A_SLOTS;
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) {
-            const int kblk = ks * 2 + kb2;
             u32x4 af[TM], bf[TN];
 #pragma unroll
-            for (int a = 0; a < TM; ++a) af[a] = abase[a_slot<BM>(wm0 + a * 32 + li, kblk)];
+            for (int a = 0; a < TM; ++a) af[a] = abase[a_rd[ks] + a * 32];
 #pragma unroll
-            for (int b = 0; b < TN; ++b) {
-                const int n = wn0 + b * 32 + li;
-                bf[b] = bbase[b_slot<BN>(n >> 3, n & 7, kblk)];
-            }
+            for (int b = 0; b < TN; ++b) bf[b] = bbase[b_rd[b] + ks * 2 * BN];
 #pragma unroll
             for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -216,6 +226,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(
         }
     };
 
+    // With 8 waves, waves w and w+4 share a SIMD: one of them unpacks the next tile (vector ALU)
+    // while the other multiplies the current one (matrix core), then they swap.
+    const bool unpack_first = NW == 8 && (wave & 4);
     if (it_begin < it_end) {
         load_global(it_begin);
         store_lds(0);
@@ -224,8 +237,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(
             const int buf = (it - it_begin) & 1;
             const bool more = it + 1 < it_end;
             if (more) load_global(it + 1);
-            compute(buf);
-            if (more) store_lds(buf ^ 1);
+            if (unpack_first) {
+                if (more) store_lds(buf ^ 1);
+                compute(buf);
+            } else {
+                compute(buf);
+                if (more) store_lds(buf ^ 1);
+            }
             __syncthreads();
         }
     }
@@ -257,7 +275,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(
     if (!arrive_last(&counters[tile], splits, &s_last)) return;
     const int rows = min(BM, M - m0);
     const int wcount = min(WCOLS, words - (n0 >> 3));
-    for (int idx = tid; idx < rows * wcount; idx += 256) {
+    for (int idx = tid; idx < rows * wcount; idx += NT) {
         const int m = m0 + idx / wcount;
         const size_t nn = (size_t)n0 + (size_t)(idx % wcount) * 8;
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -294,11 +312,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(
 // ---- host side -------------------------------------------------------------
 struct GemmVariant {
     const char* name;
-    int BM, BN;
+    int BM, BN, waves;
 };
 static const GemmVariant kGemmVariants[] = {
-    {"256x256", 256, 256}, {"128x256", 128, 256}, {"128x128", 128, 128},
-    {"64x256", 64, 256},   {"32x256", 32, 256},   {"64x128", 64, 128},
+    {"256x256w8", 256, 256, 8}, {"128x256w8", 128, 256, 8}, {"128x128", 128, 128, 4},
+    {"64x256", 64, 256, 4},     {"32x256", 32, 256, 4},     {"64x128", 64, 128, 4},
+    {"256x256", 256, 256, 4},   {"128x256", 128, 256, 4},   {"256x128w8", 256, 128, 8},
 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
@@ -326,7 +345,7 @@ static hipError_t launch_gemm(const void* x, const int32_t* qweight, const void*
         }
     }
     (void)hipGetLastError();  // do not report an earlier, unrelated failure as this launch's
-    hipLaunchKernelGGL(kern, dim3(tiles_n, tiles_m, splits), dim3(256), lds, stream,
+    hipLaunchKernelGGL(kern, dim3(tiles_n, tiles_m, splits), dim3(64 * WM * WN), lds, stream,
                        reinterpret_cast<const uint16_t*>(x),
                        reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales),
@@ -379,9 +398,9 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                          void* stream, int variant, int split_k) {
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
-    if (K % kBK != 0 || g % 8 != 0) {
-        set_error("%s: needs K %% 64 == 0 and group_size %% 8 == 0 (K=%lld, g=%lld)", fn,
-                  (long long)K, (long long)g);
+    if (K % kBK != 0 || !(g % 64 == 0 || (64 % g == 0 && g % 8 == 0))) {
+        set_error("%s: needs K %% 64 == 0 and a group size of 8, 16, 32 or a multiple of 64 (K=%lld, g=%lld)",
+                  fn, (long long)K, (long long)g);
         return AWQ_ERR_UNSUPPORTED;
     }
     if (bias && (reinterpret_cast<uintptr_t>(bias) & 15u)) {
@@ -420,12 +439,15 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                                                         workspace, split_k, s);                   \
         break;
     switch (variant) {
-        AWQ_GEMM_CASE(0, 256, 256, 2, 2)
-        AWQ_GEMM_CASE(1, 128, 256, 2, 2)
+        AWQ_GEMM_CASE(0, 256, 256, 2, 4)
+        AWQ_GEMM_CASE(1, 128, 256, 2, 4)
         AWQ_GEMM_CASE(2, 128, 128, 2, 2)
         AWQ_GEMM_CASE(3, 64, 256, 1, 4)
         AWQ_GEMM_CASE(4, 32, 256, 1, 4)
         AWQ_GEMM_CASE(5, 64, 128, 1, 4)
+        AWQ_GEMM_CASE(6, 256, 256, 2, 2)
+        AWQ_GEMM_CASE(7, 128, 256, 2, 2)
+        AWQ_GEMM_CASE(8, 256, 128, 4, 2)
     }
 #undef AWQ_GEMM_CASE
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
