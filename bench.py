@@ -220,6 +220,31 @@ def main():
         out["cfg1_single_linear"] = {"shape": "x[16,1024] @ W[1024,3072]", "graph_us": round(time_graph(fn, 5, 1) * 1e3 / 50, 2),
                                      "eager_us": round(time_eager(lambda: nq.awq_gemm(x, *w, 8), 200, 20) * 1e3, 2)}
 
+    if not args.quick:
+        # ---------------- extra: cfg4, end-to-end Qwen3-0.6B-architecture decode ------------------------
+        try:
+            from nanoquantization_amd.engine import LLMEngine
+            from nanoquantization_amd.models.random_init import QWEN3_0P6B, random_awq_qwen3
+            model = random_awq_qwen3(QWEN3_0P6B, seed=0, device=dev, dtype=torch.bfloat16)
+            B, P, NEW = 32, 512, 256
+            eng = LLMEngine(model, max_batch=B, max_seq_len=P + NEW, block_size=64, use_graph=True)
+            prompts = torch.randint(0, QWEN3_0P6B["vocab_size"], (B, P), generator=torch.Generator().manual_seed(1)).tolist()
+            eng.generate(prompts, 8)                      # warm-up: graph capture, workspaces
+            st = {}
+            eng.generate(prompts, NEW, stats=st)
+            out["e2e_qwen3_0p6b"] = {
+                "workload": "cfg4: Qwen3-0.6B architecture, random AWQ g=128 weights, bf16, paged KV (block 64), "
+                            "batch 32 x 512-token random prompts, 256 greedy tokens, decode step in a HIP graph",
+                "decode_tok_per_s": round(B * st["decode_steps"] / st["decode_s"], 1),
+                "decode_ms_per_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
+                "prefill_s": round(st["prefill_s"], 4),
+                "prefill_tok_per_s": round(B * P / st["prefill_s"], 1),
+            }
+            del eng, model
+            torch.cuda.empty_cache()
+        except Exception as e:  # the headline must still be printed
+            out["e2e_qwen3_0p6b"] = {"error": repr(e)}
+
     # ---------------- CPU baseline: the reference's path restated on host tensors (bounded sample) ----------
     if not args.no_cpu:
         from oracle import torch_cpu_path as cpu

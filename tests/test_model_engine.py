@@ -1,0 +1,148 @@
+"""The callers of the hot path: Qwen3 model contract (CPU), checkpoint round trip (CPU), and on the GPU
+the paged-KV engine against the model's own no-cache forward (the reference semantics)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import nanoquantization_amd as nq
+from nanoquantization_amd.layers.norm import RMSNorm
+from nanoquantization_amd.layers.rope import RoPE
+from nanoquantization_amd.models.qwen3_quantized import Qwen3QuantizedForCausalLM
+from nanoquantization_amd.utils.loader import load_model, model_from_config, save_quantized_model
+
+TINY = dict(num_hidden_layers=2, vocab_size=512, hidden_size=256, total_num_heads=4, total_num_kv_heads=2,
+            max_position_embeddings=256, intermediate_size=512, head_dim=64, tie_word_embeddings=True,
+            rope_theta=10000.0, rms_norm_eps=1e-6)
+
+
+def test_rmsnorm_and_rope_closed_forms():
+    torch.manual_seed(0)
+    x = torch.randn(3, 5, 64)
+    n = RMSNorm(64, 1e-6)
+    n.weight.data = torch.linspace(0.5, 1.5, 64)
+    expect = x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-6) * n.weight
+    assert torch.allclose(n(x), expect, atol=1e-6)
+    r = RoPE(64, 128, 10000.0)
+    q, k = torch.randn(2, 7, 4, 64), torch.randn(2, 7, 2, 64)
+    pos = torch.arange(7).unsqueeze(0).expand(2, 7)
+    q2, k2 = r(q, k, pos)
+    # rotation preserves the norm of each (i, i+32) pair and position 0 is the identity
+    assert torch.allclose(q2[:, 0], q[:, 0], atol=1e-6)
+    pair = lambda t: t[..., :32] ** 2 + t[..., 32:] ** 2
+    assert torch.allclose(pair(q2), pair(q), atol=1e-4) and torch.allclose(pair(k2), pair(k), atol=1e-4)
+    # angle of pair i at position p is p * base^(-2i/d)
+    ang = torch.atan2(q2[0, 3, 0, 32:] * q[0, 3, 0, :32] - q2[0, 3, 0, :32] * q[0, 3, 0, 32:],
+                      q2[0, 3, 0, :32] * q[0, 3, 0, :32] + q2[0, 3, 0, 32:] * q[0, 3, 0, 32:])
+    inv = 1.0 / (10000.0 ** (torch.arange(0, 64, 2).float() / 64))
+    assert torch.allclose(torch.remainder(ang, 2 * np.pi), torch.remainder(3 * inv, 2 * np.pi), atol=1e-3)
+    # the angle table survives model.to(bfloat16) in fp32
+    assert r.to(torch.bfloat16).cos_sin_cache.dtype == torch.float32
+
+
+def test_model_state_dict_keys_match_reference_contract():
+    m = Qwen3QuantizedForCausalLM(**TINY)
+    keys = set(m.state_dict())
+    for i in range(2):
+        for proj in ("q_proj", "k_proj", "v_proj", "o_proj"):
+            for buf in ("qweight", "qscales", "qzeros"):
+                assert f"model.layers.{i}.self_attn.{proj}.{buf}" in keys
+        for proj in ("gate_proj", "up_proj", "down_proj"):
+            for buf in ("qweight", "qscales", "qzeros"):
+                assert f"model.layers.{i}.mlp.{proj}.{buf}" in keys
+        for nrm in ("input_layernorm", "post_attention_layernorm", "self_attn.q_norm", "self_attn.k_norm"):
+            assert f"model.layers.{i}.{nrm}.weight" in keys
+    assert {"model.norm.weight", "model.embed_tokens.weight", "lm_head.weight", "lm_head.bias"} <= keys
+    assert not any("cos_sin_cache" in k for k in keys)       # non-persistent, as in the reference
+    assert m.model.layers[0].self_attn.q_proj.qscales.dtype == torch.bfloat16
+    assert m.lm_head.weight.data_ptr() == m.model.embed_tokens.weight.data_ptr()   # tied
+
+
+def test_checkpoint_roundtrip(tmp_path):
+    torch.manual_seed(1)
+    m = Qwen3QuantizedForCausalLM(**TINY).to(torch.bfloat16)
+    for name, buf in m.named_buffers():
+        if buf.dtype == torch.int32:
+            buf.copy_(torch.randint(-2 ** 31, 2 ** 31 - 1, buf.shape, dtype=torch.int32))
+        elif "qscales" in name:
+            buf.copy_(torch.rand(buf.shape) * 0.01)
+    cfg = dict(num_hidden_layers=2, vocab_size=512, hidden_size=256, num_attention_heads=4, num_key_value_heads=2,
+               max_position_embeddings=256, intermediate_size=512, head_dim=64, tie_word_embeddings=True,
+               rope_theta=10000.0, rms_norm_eps=1e-6)
+    save_quantized_model(m, str(tmp_path), cfg, 4, 128)
+    saved = json.load(open(tmp_path / "config.json"))
+    assert saved["quantization_config"]["quant_method"] == "awq" and saved["quantization_config"]["version"] == "gemm"
+    assert os.path.exists(tmp_path / "model.safetensors") and os.path.exists(tmp_path / "model.safetensors.index.json")
+    m2 = model_from_config(str(tmp_path))
+    for (k1, v1), (k2, v2) in zip(m.state_dict().items(), m2.state_dict().items()):
+        assert k1 == k2 and torch.equal(v1, v2), k1
+    m3 = Qwen3QuantizedForCausalLM(**TINY).to(torch.bfloat16)
+    load_model(m3, str(tmp_path))
+    assert torch.equal(m3.model.layers[1].mlp.down_proj.qweight, m.model.layers[1].mlp.down_proj.qweight)
+    with pytest.raises(AttributeError):
+        from safetensors.torch import save_file
+        save_file({"no.such.tensor": torch.zeros(1)}, str(tmp_path / "extra.safetensors"))
+        load_model(m3, str(tmp_path))
+
+
+@pytest.mark.gpu
+def test_engine_greedy_matches_full_recompute():
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import random_awq_qwen3
+    print("engine vs recompute", flush=True)
+    model = random_awq_qwen3(TINY, seed=3, std=0.05)
+    torch.manual_seed(4)
+    prompts = torch.randint(0, 512, (3, 19)).tolist()
+    new = 12
+    for use_graph in (False, True):
+        eng = LLMEngine(model, max_batch=4, max_seq_len=64, block_size=16, use_graph=use_graph)
+        got = eng.generate(prompts, new)
+        # reference semantics: full-sequence causal forward, no cache.  Teacher-force the engine's own
+        # continuation through it: every token the engine chose must be the recompute's argmax up to the
+        # bf16 noise of a near-tie, and where the logits are not near-tied the tokens must be identical.
+        seqs = torch.tensor([p + g for p, g in zip(prompts, got)], device="cuda")
+        pos = torch.arange(seqs.shape[1], device="cuda").unsqueeze(0)
+        logits = model.lm_head(model(seqs, pos)).float()[:, 18:-1]            # predictions for the new tokens
+        chosen = torch.tensor(got, device="cuda")
+        top = logits.max(-1).values
+        gap = top - logits.gather(-1, chosen.unsqueeze(-1)).squeeze(-1)
+        scale = logits.abs().max().item()
+        assert gap.max().item() <= 2e-2 * scale, (use_graph, gap.max().item(), scale)
+        top2 = logits.topk(2, dim=-1).values
+        clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
+        assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
+        assert clear.float().mean().item() > 0.5
+        assert [g[0] for g in got] == logits[:, 0].argmax(-1).tolist() or not clear[:, 0].all()
+        # a second call reuses the freed blocks and the captured graph
+        assert eng.generate(prompts, new) == got
+
+
+@pytest.mark.gpu
+def test_model_forward_matches_dequantised_torch_model():
+    from nanoquantization_amd.models.random_init import random_awq_qwen3
+    print("model forward vs dequantised linears", flush=True)
+    model = random_awq_qwen3(TINY, seed=5, std=0.05)
+    ids = torch.randint(0, 512, (2, 24), device="cuda")
+    pos = torch.arange(24, device="cuda").unsqueeze(0)
+    h = model(ids, pos).float()
+    # same network with every AWQ linear replaced by x @ dequant(W) in fp32
+    import torch.nn.functional as F
+
+    class Deq(torch.nn.Module):
+        def __init__(self, m):
+            super().__init__()
+            self.w = nq.awq_dequantize(m.qweight, m.qscales, m.qzeros).float()
+        def forward(self, x):
+            return (x.float() @ self.w).to(x.dtype)
+
+    import copy
+    ref = copy.deepcopy(model)
+    for blk in ref.model.layers:
+        for parent, names in ((blk.self_attn, ("q_proj", "k_proj", "v_proj", "o_proj")), (blk.mlp, ("gate_proj", "up_proj", "down_proj"))):
+            for nme in names:
+                setattr(parent, nme, Deq(getattr(parent, nme)))
+    h_ref = ref(ids, pos).float()
+    err = (h - h_ref).abs().max().item() / h_ref.abs().max().item()
+    assert err <= 3e-2, err
