@@ -224,11 +224,11 @@ def main():
         # ---------------- extra: cfg4, end-to-end Qwen3-0.6B-architecture decode ------------------------
         try:
             from nanoquantization_amd.engine import LLMEngine
-            from nanoquantization_amd.models.random_init import QWEN3_0P6B, random_awq_qwen3
-            model = random_awq_qwen3(QWEN3_0P6B, seed=0, device=dev, dtype=torch.bfloat16)
+            from nanoquantization_amd.models.random_init import QWEN3_0P6B as Q06B_CFG, random_awq_qwen3
+            model = random_awq_qwen3(Q06B_CFG, seed=0, device=dev, dtype=torch.bfloat16)
             B, P, NEW = 32, 512, 256
             eng = LLMEngine(model, max_batch=B, max_seq_len=P + NEW, block_size=64, use_graph=True)
-            prompts = torch.randint(0, QWEN3_0P6B["vocab_size"], (B, P), generator=torch.Generator().manual_seed(1)).tolist()
+            prompts = torch.randint(0, Q06B_CFG["vocab_size"], (B, P), generator=torch.Generator().manual_seed(1)).tolist()
             eng.generate(prompts, 8)                      # warm-up: graph capture, workspaces
             st = {}
             eng.generate(prompts, NEW, stats=st)

@@ -372,21 +372,19 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
 // yields at least one workgroup per CU, then split K until the chip is covered.
 static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     const int kCUs = 256;
+    // indices into kGemmVariants
+    constexpr int k256x256 = 6, k128x128 = 2, k64x256 = 3, k32x256 = 4;
     int v;
-    if (M <= 32) v = 4;
-    else if (M <= 64) v = 3;
-    else {
-        v = 0;
-        if (cdiv(M, 256) * cdiv(N, 256) < kCUs) v = 1;
-        if (cdiv(M, 128) * cdiv(N, 256) < kCUs) v = 2;
-    }
+    if (M <= 32) v = k32x256;
+    else if (M <= 64) v = k64x256;
+    else v = (cdiv(M, 256) * cdiv(N, 256) >= 2 * kCUs) ? k256x256 : k128x128;
     const GemmVariant& gv = kGemmVariants[v];
     const int64_t tiles = cdiv(M, gv.BM) * cdiv(N, gv.BN);
     int64_t s = 1;
     if (tiles < kCUs) s = kCUs / tiles;
     const int64_t max_s = K / kBK / 4 > 0 ? K / kBK / 4 : 1;  // at least 4 K-steps per split
     if (s > max_s) s = max_s;
-    if (s > 32) s = 32;
+    if (s > 16) s = 16;
     if (s < 1) s = 1;
     *variant = v;
     *split_k = (int)s;
@@ -495,14 +493,19 @@ extern "C" int awq_gemm(const void* x, const int32_t* qweight, const void* qscal
 }
 
 extern "C" size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-    return M <= 16 ? awq_gemv_workspace_bytes(M, N, K) : awq_gemm_workspace_bytes(M, N, K);
+    // the regime depends on the group size, which this query does not get: cover both
+    const size_t a = M <= 64 ? awq_gemv_workspace_bytes(M, N, K) : 0;
+    const size_t b = M > 16 ? awq_gemm_workspace_bytes(M, N, K) : 0;
+    return a > b ? a : b;
 }
 
 extern "C" int awq_linear(const void* x, const int32_t* qweight, const void* qscales,
                           const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                           int64_t K, int64_t group_size, int dtype, void* workspace,
                           size_t workspace_bytes, void* stream) {
-    if (M >= 1 && M <= 16 && group_size % 32 == 0)
+    // decode regime: up to 16 rows on any GEMV path, up to 64 on the staged one
+    const bool staged = N % 128 == 0 && group_size > 0 && group_size % 128 == 0;
+    if (M >= 1 && ((M <= 16 && group_size % 32 == 0) || (M <= 64 && staged)))
         return awq_gemv(x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, workspace,
                         workspace_bytes, stream);
     return awq_gemm(x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, workspace,

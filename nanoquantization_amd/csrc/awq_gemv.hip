@@ -97,30 +97,37 @@ __device__ __forceinline__ uint32_t vget(const typename WordVec<V>::type& v, int
     if constexpr (V == 1) return v; else return v[i];
 }
 
-// One chunk = CH steps of 32 rows inside one quantisation group.
-template <int V, int CH>
+// One chunk = CH steps of 32 rows inside one quantisation group; MT tiles of 16 activation rows.
+template <int V, int CH, int MT = 1>
 struct Chunk {
     typename WordVec<V>::type w[CH][8];  // per step: 8 rows x V words
-    u32x4 xa[CH];                        // per step: A operand x[m = j][k0 + 8kb .. +7]
+    u32x4 xa[CH][MT];                    // per step and m-tile: A operand x[16*mt + j][k0 + 8kb .. +7]
     typename WordVec<V>::type zw;        // V zero words of the group
     u32x4 sv[V];                         // 8 scales per word
 };
 
-// acc[8V] += one chunk.  acc[v*8 + c][r] is output row 4*kb + r, column 8*(word v) + c.
-template <typename T, int V, int CH>
-__device__ __forceinline__ void compute_chunk(const Chunk<V, CH>& d, f32x4 (&acc)[8 * V]) {
+// acc[mt][8V] += one chunk.  acc[mt][v*8 + c][r] is output row 16*mt + 4*kb + r, column 8*(word v) + c.
+// The unpacked B fragments are built once and multiplied against every m-tile.
+template <typename T, int V, int CH, int MT = 1>
+__device__ __forceinline__ void compute_chunk(const Chunk<V, CH, MT>& d, f32x4 (&acc)[MT][8 * V]) {
     const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
     const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
     const AndOr emb_lo(Embed<T>::kMaskLo, Embed<T>::kMagicLo), emb_hi(Embed<T>::kMaskHi, Embed<T>::kMagicHi);
-    f32x4 dones = zero4;
+    f32x4 dones[MT];
 #pragma unroll
-    for (int s = 0; s < CH; ++s) dones = T::mfma16(d.xa[s], ones, dones);
+    for (int mt = 0; mt < MT; ++mt) {
+        dones[mt] = zero4;
+#pragma unroll
+        for (int s = 0; s < CH; ++s) dones[mt] = T::mfma16(d.xa[s][mt], ones, dones[mt]);
+    }
 #pragma unroll
     for (int v = 0; v < V; ++v) {
         const uint32_t zw = vget<V>(d.zw, v);
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
-            f32x4 dlo = zero4, dhi = zero4;
+            f32x4 dlo[MT], dhi[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) dlo[mt] = dhi[mt] = zero4;
 #pragma unroll
             for (int s = 0; s < CH; ++s) {
                 u32x4 flo, fhi;
@@ -133,15 +140,17 @@ __device__ __forceinline__ void compute_chunk(const Chunk<V, CH>& d, f32x4 (&acc
                     flo[rp] = emb_lo(Embed<T>::pre_lo(p));
                     fhi[rp] = emb_hi(Embed<T>::pre_hi(p));
                 }
-                dlo = T::mfma16(d.xa[s], flo, dlo);
-                dhi = T::mfma16(d.xa[s], fhi, dhi);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    dlo[mt] = T::mfma16(d.xa[s][mt], flo, dlo[mt]);
+                    dhi[mt] = T::mfma16(d.xa[s][mt], fhi, dhi[mt]);
+                }
             }
             // byte b holds column {0,4,1,5}[b] in its low and {2,6,3,7}[b] in its high nibble
             constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int c = h ? kHiCol[b] : kLoCol[b];
-                const f32x4 dq = h ? dhi : dlo;
                 const float mul = h ? Embed<T>::kMulHi : Embed<T>::kMulLo;
                 const float off = h ? Embed<T>::kOffHi : Embed<T>::kOffLo;
                 // value of the embedded zero point, off + mul*z, and the scale / mul
@@ -149,7 +158,11 @@ __device__ __forceinline__ void compute_chunk(const Chunk<V, CH>& d, f32x4 (&acc
                 const uint32_t pair = d.sv[v][c >> 1];
                 const float sc = T::to_f32((uint16_t)((c & 1) ? (pair >> 16) : (pair & 0xFFFFu))) * (1.f / mul);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[v * 8 + c][r] += sc * (dq[r] - zf * dones[r]);
+                for (int mt = 0; mt < MT; ++mt) {
+                    const f32x4 dq = h ? dhi[mt] : dlo[mt];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[mt][v * 8 + c][r] += sc * (dq[r] - zf * dones[mt][r]);
+                }
             }
         }
     }
@@ -161,18 +174,18 @@ __device__ __forceinline__ void compute_chunk(const Chunk<V, CH>& d, f32x4 (&acc
 // partial and let the last workgroup of the tile group add the partials in
 // split order.  `group` is the workgroup's index along N.
 template <typename T, int V, int WN, int WK>
-__device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[8 * V], float* red, int* s_last, int lane,
-                                              int wave, int group, int split, int splits,
-                                              const uint16_t* __restrict__ bias,
-                                              uint16_t* __restrict__ y, float* __restrict__ partials,
-                                              int* __restrict__ counters, int M, int N) {
-    constexpr int NF = 8 * V, NQ = 4 * V, WAVES = WN * WK;
+__device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_base, float* red, int lane,
+                                                  int wave, int group, int split, int splits,
+                                                  const uint16_t* __restrict__ bias,
+                                                  uint16_t* __restrict__ y, float* __restrict__ partials,
+                                                  int M, int N) {
+    constexpr int NF = 8 * V, NQ = 4 * V;
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
     const int wn = wave % WN, wk = wave / WN;
     const int wv_col = (group * WN + wn) * 16 + j;  // this lane's column, in units of V words
     const bool col_ok = wv_col * V < words;
-    // slot q = v*4 + r holds 8 consecutive output columns of row 4*kb + r
+    // slot q = v*4 + r holds 8 consecutive output columns of row m_base + 4*kb + r
     if constexpr (WK > 1) {
         float* mine = red + (size_t)wave * (NF * 4 * 64);
 #pragma unroll
@@ -185,7 +198,7 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[8 * V], float* red, i
     }
     for (int q = wk; q < NQ; q += WK) {
         const int v = q >> 2, r = q & 3;
-        const int m = 4 * kb + r;
+        const int m = m_base + 4 * kb + r;
         float out[8];
         if constexpr (WK > 1) {
 #pragma unroll
@@ -226,8 +239,15 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[8 * V], float* red, i
             }
         }
     }
-    if (splits == 1) return;
+}
 
+template <typename T, int V, int WN, int WK>
+__device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int splits,
+                                                const uint16_t* __restrict__ bias,
+                                                uint16_t* __restrict__ y, float* __restrict__ partials,
+                                                int* __restrict__ counters, int M, int N) {
+    constexpr int WAVES = WN * WK;
+    const int words = N >> 3;
     if (!arrive_last(&counters[group], splits, s_last)) return;
     const int group_words = 16 * V * WN;
     const int w_begin = group * group_words;
@@ -265,6 +285,30 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[8 * V], float* red, i
         *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
     }
     if (threadIdx.x == 0) __hip_atomic_store(&counters[group], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// A workgroup is WN x WK waves: wave w works on column tile (group*WN + w % WN)
+// and K sub-slice w / WN.  Sum the WK waves of each column tile through LDS
+// (fixed order), then either store y (splits == 1) or publish this split's
+// partial and let the last workgroup of the tile group add the partials in
+// split order.  `group` is the workgroup's index along N.
+template <typename T, int V, int WN, int WK, int MT = 1>
+__device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* red, int* s_last, int lane,
+                                              int wave, int group, int split, int splits,
+                                              const uint16_t* __restrict__ bias,
+                                              uint16_t* __restrict__ y, float* __restrict__ partials,
+                                              int* __restrict__ counters, int M, int N) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        if (mt > 0) {
+            if (16 * mt >= M) break;  // uniform
+            __syncthreads();          // the reduction buffer is reused per m-tile
+        }
+        gemv_reduce_store<T, V, WN, WK>(acc[mt], 16 * mt, red, lane, wave, group, split, splits, bias, y,
+                                        partials, M, N);
+    }
+    if (splits == 1) return;
+    gemv_split_tail<T, V, WN, WK>(s_last, group, splits, bias, y, partials, counters, M, N);
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
@@ -316,9 +360,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
     for (int r = 0; r < 8; ++r) woff[r] = (uint32_t)(kb * 8 + r) * (uint32_t)wstride + (uint32_t)wv_ld;
     const uint32_t xoff = (uint32_t)xrow * (uint32_t)K + (uint32_t)kb * 8u;
 
-    f32x4 acc[NF];
+    f32x4 acc[1][NF];
 #pragma unroll
-    for (int f = 0; f < NF; ++f) acc[f] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int f = 0; f < NF; ++f) acc[0][f] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     auto load_chunk = [&](int c, Chunk<V, CH>& d) {
         const int row0 = c * (32 * CH);  // wave-uniform
@@ -329,7 +373,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
             for (int r = 0; r < 8; ++r) d.w[s][r] = wp[woff[r]];
         }
 #pragma unroll
-        for (int s = 0; s < CH; ++s) d.xa[s] = *reinterpret_cast<const u32x4*>(x + (row0 + s * 32) + xoff);
+        for (int s = 0; s < CH; ++s) d.xa[s][0] = *reinterpret_cast<const u32x4*>(x + (row0 + s * 32) + xoff);
         const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
         d.zw = (zbase + (size_t)gi * wstride)[wv_ld];
 #pragma unroll
@@ -373,7 +417,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
 
 __host__ __device__ constexpr int dma_wave_bytes(int M) { return 8192 + 256 * M + 512; }
 
-template <typename T, int WN, int WK, int DEPTH>
+template <typename T, int WN, int WK, int DEPTH, int MT = 1>
 __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
@@ -411,15 +455,23 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         const int slot = h * 16 + dsl;
         wsrc[h] = (uint32_t)((slot & 3) * 8 + (slot >> 2)) * (uint32_t)words + (uint32_t)(tile * 16 + dq * 4);
     }
-    const bool x_lane = lane < 4 * M;          // lane = m*4 + k-block
-    const uint32_t xsrc = (uint32_t)(x_lane ? (lane >> 2) : 0) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
+    // x: per m-tile one DMA instruction per step; lane = (m - 16*mt)*4 + k-block
+    static_assert(MT == 1 || DEPTH == 1, "the vmcnt arithmetic of deeper pipelines assumes one m-tile");
+    bool x_lane[MT];
+    uint32_t xsrc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = 16 * mt + (lane >> 2);
+        x_lane[mt] = m < M;
+        xsrc[mt] = (uint32_t)(x_lane[mt] ? m : 0) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
+    }
     const bool zs_lane = lane < 16;
     const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
 
     // exactly kDmaOps vector-memory instructions per call (the vmcnt arithmetic below counts on it):
     // lanes 0..3 and 0..15 exist in every wave, so neither guarded block is ever skipped
     constexpr int kDmaOps = 2 * CH + CH + 2;
-    static_assert(kDmaOps == 14, "vmcnt immediates below assume 14 DMA instructions per chunk");
+    static_assert(kDmaOps == 14, "vmcnt immediates below assume 14 DMA instructions per chunk (one m-tile)");
     auto issue_dma = [&](int c, int buf) {
         const int row0 = c * 128;
         char* base = stage + buf * buf_bytes;
@@ -434,12 +486,14 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
                                                  16, 0, 0);
         }
-        if (x_lane) {
 #pragma unroll
-            for (int s = 0; s < CH; ++s)
-                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc),
-                                                 AWQ_LPTR(x_lds + s * 64 * M), 16, 0, 0);
-        }
+        for (int mt = 0; mt < MT; ++mt)
+            if (x_lane[mt]) {
+#pragma unroll
+                for (int s = 0; s < CH; ++s)
+                    __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc[mt]),
+                                                     AWQ_LPTR(x_lds + s * 64 * M + mt * 1024), 16, 0, 0);
+            }
         if (zs_lane) {
             const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
             __builtin_amdgcn_global_load_lds(AWQ_GPTR(qzeros + (size_t)gi * words + zsrc), AWQ_LPTR(zs_lds), 4, 0, 0);
@@ -449,15 +503,18 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     };
 
     // compute-lane read offsets inside a staging buffer (bytes)
-    const int xm = j < M ? j : M - 1;
     const int w_rd_off = (kb * 16 + j) * 4;                   // + (s*512 + r*64) * 4
-    const int x_rd_off = x_off + (xm * 4 + kb) * 16;          // + s * 64 * M
+    int x_rd_off[MT];                                         // + s * 64 * M
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) x_rd_off[mt] = x_off + (min(16 * mt + j, M - 1) * 4 + kb) * 16;
     const int z_rd_off = zs_off + j * 4;
     const int s_rd_off = zs_off + 64 + j * 16;
 
-    f32x4 acc[8];
+    f32x4 acc[MT][8];
 #pragma unroll
-    for (int f = 0; f < 8; ++f) acc[f] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int f = 0; f < 8; ++f) acc[mt][f] = f32x4{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d)
@@ -473,12 +530,14 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         asm volatile("" ::: "memory");
         const char* base = stage + buf * buf_bytes;
         const uint32_t* w_rd = reinterpret_cast<const uint32_t*>(base + w_rd_off);
-        Chunk<1, CH> d;
+        Chunk<1, CH, MT> d;
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) d.w[s][r] = w_rd[s * 512 + r * 64];
-            d.xa[s] = *reinterpret_cast<const u32x4*>(base + x_rd_off + s * 64 * M);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                d.xa[s][mt] = *reinterpret_cast<const u32x4*>(base + x_rd_off[mt] + s * 64 * M);
         }
         d.zw = *reinterpret_cast<const uint32_t*>(base + z_rd_off);
         d.sv[0] = *reinterpret_cast<const u32x4*>(base + s_rd_off);
@@ -488,10 +547,10 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         asm volatile("" ::: "memory");
         if (c + DEPTH < c1) issue_dma(c + DEPTH, buf);
         buf = (buf + 1 == DEPTH) ? 0 : buf + 1;
-        compute_chunk<T, 1, CH>(d, acc);
+        compute_chunk<T, 1, CH, MT>(d, acc);
     }
     __syncthreads();  // staging area becomes the reduction buffer
-    gemv_epilogue<T, 1, WN, WK>(acc, red, &s_last, lane, wave, group, split, splits, bias, y, partials,
+    gemv_epilogue<T, 1, WN, WK, MT>(acc, red, &s_last, lane, wave, group, split, splits, bias, y, partials,
                                 counters, M, N);
 }
 
@@ -502,17 +561,19 @@ struct GemvVariant {
     bool prefetch;
     int wn;     // waves side by side along N (DMA variants), 1 otherwise
     int depth;  // DMA staging buffers per wave (DMA variants), 0 otherwise
+    int mt;     // tiles of 16 activation rows: M <= 16 * mt
 };
 static const GemvVariant kGemvVariants[] = {
-    {"v1w4p", 1, 4, true, 1, 0},  {"v1w8p", 1, 8, true, 1, 0},   {"v2w4", 2, 4, false, 1, 0},
-    {"v2w8", 2, 8, false, 1, 0},  {"v2w4p", 2, 4, true, 1, 0},   {"v1w16", 1, 16, false, 1, 0},
-    {"v1w1p", 1, 1, true, 1, 0},  {"v2w1", 2, 1, false, 1, 0},   {"v1w4", 1, 4, false, 1, 0},
-    {"v1w8", 1, 8, false, 1, 0},
-    // DMA variants, named dma<WN>x<WK>d<DEPTH>
-    {"dma1x4d1", 1, 4, false, 1, 1},  {"dma1x8d1", 1, 8, false, 1, 1},  {"dma1x16d1", 1, 16, false, 1, 1},
-    {"dma1x4d2", 1, 4, false, 1, 2},  {"dma1x8d2", 1, 8, false, 1, 2},  {"dma1x4d3", 1, 4, false, 1, 3},
-    {"dma2x4d1", 1, 8, false, 2, 1},  {"dma2x4d2", 1, 8, false, 2, 2},  {"dma1x1d1", 1, 1, false, 1, 1},
-    {"dma1x2d2", 1, 2, false, 1, 2},
+    {"v1w4p", 1, 4, true, 1, 0, 1},  {"v1w8p", 1, 8, true, 1, 0, 1},   {"v2w4", 2, 4, false, 1, 0, 1},
+    {"v2w8", 2, 8, false, 1, 0, 1},  {"v2w4p", 2, 4, true, 1, 0, 1},   {"v1w16", 1, 16, false, 1, 0, 1},
+    {"v1w1p", 1, 1, true, 1, 0, 1},  {"v2w1", 2, 1, false, 1, 0, 1},   {"v1w4", 1, 4, false, 1, 0, 1},
+    {"v1w8", 1, 8, false, 1, 0, 1},
+    // DMA variants, named dma<WN>x<WK>d<DEPTH>[m<MT>]
+    {"dma1x4d1", 1, 4, false, 1, 1, 1},  {"dma1x8d1", 1, 8, false, 1, 1, 1},  {"dma1x16d1", 1, 16, false, 1, 1, 1},
+    {"dma1x4d2", 1, 4, false, 1, 2, 1},  {"dma1x8d2", 1, 8, false, 1, 2, 1},  {"dma1x4d3", 1, 4, false, 1, 3, 1},
+    {"dma2x4d1", 1, 8, false, 2, 1, 1},  {"dma2x4d2", 1, 8, false, 2, 2, 1},  {"dma1x1d1", 1, 1, false, 1, 1, 1},
+    {"dma1x2d2", 1, 2, false, 1, 2, 1},
+    {"dma1x4d1m2", 1, 4, false, 1, 1, 2}, {"dma1x8d1m2", 1, 8, false, 1, 1, 2}, {"dma1x4d1m4", 1, 4, false, 1, 1, 4},
 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = 10;
@@ -556,7 +617,7 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
     return hipGetLastError();
 }
 
-template <typename T, int WN, int WK, int DEPTH>
+template <typename T, int WN, int WK, int DEPTH, int MT>
 static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                                   int g, void* workspace, int split_k, hipStream_t stream) {
@@ -572,10 +633,10 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     size_t lds = (size_t)WAVES * DEPTH * dma_wave_bytes(M);
     const size_t red_bytes = WK > 1 ? (size_t)WAVES * 32 * 64 * sizeof(float) : 0;
     if (lds < red_bytes) lds = red_bytes;
-    auto kern = gemv_dma_kernel<T, WN, WK, DEPTH>;
+    auto kern = gemv_dma_kernel<T, WN, WK, DEPTH, MT>;
     // what the largest M that still fits asks for (the dispatcher rejects bigger requests)
     constexpr size_t kLdsCap = 160 * 1024 - 1024;
-    constexpr size_t kWant = (size_t)WAVES * DEPTH * dma_wave_bytes(16);
+    constexpr size_t kWant = (size_t)WAVES * DEPTH * dma_wave_bytes(16 * MT);
     constexpr size_t kMaxLds = kWant < kLdsCap ? kWant : kLdsCap;
     if (kMaxLds > 64 * 1024) {
         static bool raised = false;  // once per process and instantiation
@@ -620,7 +681,11 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         const int64_t tiles = N / 128;
         int v = 10 /* dma1x4d1 */;
         int64_t s = 1;
-        if (chunks <= 8) {
+        if (M > 32) {
+            v = 22 /* dma1x4d1m4 */;   // 17..64 rows: never split K, the tail grows with M
+        } else if (M > 16) {
+            v = chunks >= 8 ? 21 /* dma1x8d1m2 */ : 20 /* dma1x4d1m2 */;
+        } else if (chunks <= 8) {
             v = 11 /* dma1x8d1 */;
         } else if (M <= 4) {
             s = cdiv(3072, tiles * 4);
@@ -654,8 +719,8 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                          void* stream, int variant, int split_k) {
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
-    if (M > 16) {
-        set_error("%s: M=%lld is outside the decode regime (1..16); use awq_gemm", fn, (long long)M);
+    if (M > 64) {
+        set_error("%s: M=%lld is outside the decode regime (1..64); use awq_gemm", fn, (long long)M);
         return AWQ_ERR_UNSUPPORTED;
     }
     if (g % 32 != 0 || K % 32 != 0) {
@@ -671,6 +736,11 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         return AWQ_ERR_INVALID_ARG;
     }
     const GemvVariant& gv = kGemvVariants[variant];
+    if (M > 16 * gv.mt) {
+        set_error("%s: variant %s takes at most %d rows (M=%lld); rows 17..64 need the staged path "
+                  "(N %% 128 == 0, group_size %% 128 == 0)", fn, gv.name, 16 * gv.mt, (long long)M);
+        return AWQ_ERR_UNSUPPORTED;
+    }
     if ((N / 8) % gv.V != 0) {
         set_error("%s: variant %s needs N %% %d == 0 (N=%lld)", fn, gv.name, 8 * gv.V, (long long)N);
         return AWQ_ERR_UNSUPPORTED;
@@ -698,23 +768,26 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
             set_error("%s: variant %s does not fit the LDS at M=%lld", fn, gv.name, (long long)M);
             return AWQ_ERR_UNSUPPORTED;
         }
-#define AWQ_DMA_CASE(NN, KK, DD)                                                                    \
-    if (gv.wn == NN && gv.waves == NN * KK && gv.depth == DD)                                       \
+#define AWQ_DMA_CASE(NN, KK, DD, MM)                                                                \
+    if (gv.wn == NN && gv.waves == NN * KK && gv.depth == DD && gv.mt == MM)                        \
         e = dtype == AWQ_F16                                                                        \
-                ? launch_gemv_dma<F16, NN, KK, DD>(x, qweight, qscales, qzeros, bias, y, (int)M,    \
-                                                   (int)N, (int)K, (int)g, workspace, split_k, s)   \
-                : launch_gemv_dma<BF16, NN, KK, DD>(x, qweight, qscales, qzeros, bias, y, (int)M,   \
-                                                    (int)N, (int)K, (int)g, workspace, split_k, s);
-        AWQ_DMA_CASE(1, 4, 1)
-        AWQ_DMA_CASE(1, 8, 1)
-        AWQ_DMA_CASE(1, 16, 1)
-        AWQ_DMA_CASE(1, 4, 2)
-        AWQ_DMA_CASE(1, 8, 2)
-        AWQ_DMA_CASE(1, 4, 3)
-        AWQ_DMA_CASE(2, 4, 1)
-        AWQ_DMA_CASE(2, 4, 2)
-        AWQ_DMA_CASE(1, 1, 1)
-        AWQ_DMA_CASE(1, 2, 2)
+                ? launch_gemv_dma<F16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
+                                                       (int)N, (int)K, (int)g, workspace, split_k, s) \
+                : launch_gemv_dma<BF16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
+                                                        (int)N, (int)K, (int)g, workspace, split_k, s);
+        AWQ_DMA_CASE(1, 4, 1, 1)
+        AWQ_DMA_CASE(1, 8, 1, 1)
+        AWQ_DMA_CASE(1, 16, 1, 1)
+        AWQ_DMA_CASE(1, 4, 2, 1)
+        AWQ_DMA_CASE(1, 8, 2, 1)
+        AWQ_DMA_CASE(1, 4, 3, 1)
+        AWQ_DMA_CASE(2, 4, 1, 1)
+        AWQ_DMA_CASE(2, 4, 2, 1)
+        AWQ_DMA_CASE(1, 1, 1, 1)
+        AWQ_DMA_CASE(1, 2, 2, 1)
+        AWQ_DMA_CASE(1, 4, 1, 2)
+        AWQ_DMA_CASE(1, 8, 1, 2)
+        AWQ_DMA_CASE(1, 4, 1, 4)
 #undef AWQ_DMA_CASE
         return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
     }

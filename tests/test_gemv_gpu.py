@@ -46,7 +46,7 @@ def test_gemv_every_variant_and_split(dtype):
     K, N = 1024, 1024
     p = random_packed(K, N, 128, dtype, seed=21)
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
-    for M in (1, 3, 16):
+    for M in (1, 3, 16, 24, 40):
         xb = make_x(M, K, dtype, seed=30 + M)
         xd = to_dev(xb, dtype)
         for v in range(L.awq_gemv_variant_count()):
@@ -55,8 +55,8 @@ def test_gemv_every_variant_and_split(dtype):
                 try:
                     y = awq_gemv_variant(xd, *dev, v, split)
                 except _lib.AwqHipError as e:
-                    if "does not fit the LDS" in str(e):    # 16-wave staging variants at large M
-                        continue
+                    if "does not fit the LDS" in str(e) or "takes at most" in str(e):
+                        continue    # 16-wave staging variants at large M; single-m-tile variants above 16 rows
                     raise
                 torch.cuda.synchronize()
                 _check(y, xb, p, dtype)
@@ -71,6 +71,20 @@ def test_gemv_ragged_shapes_and_groups(dtype, K, N, g):
         xb = make_x(M, K, dtype, seed=M + 3)
         y = nq.awq_gemm(to_dev(xb, dtype), to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"]), 8)
         torch.cuda.synchronize()
+        _check(y, xb, p, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [17, 32, 33, 48, 64])
+def test_gemv_batched_decode_rows(dtype, M):
+    # decode batches of 17..64 rows (Qwen3 configs 4 and 5 decode at batch 32 / 64) run on the staged GEMV
+    print(f"gemv batched decode {dtype} M={M}", flush=True)
+    for (K, N) in [(1024, 3072), (3072, 1024), (2048, 1024)]:
+        p = make_case(K, N, 128, dtype, seed=K + N + M)
+        xb = make_x(M, K, dtype, seed=M)
+        y = nq.awq_gemm(to_dev(xb, dtype), to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"]), 8)
+        torch.cuda.synchronize()
+        assert tuple(y.shape) == (M, N)
         _check(y, xb, p, dtype)
 
 
@@ -122,8 +136,10 @@ def test_gemv_errors():
     p = random_packed(256, 64, 128, "f16")
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], "f16"), to_dev(p["qzeros"])]
     x = torch.zeros(17, 256, dtype=torch.float16, device="cuda")
-    with pytest.raises(_lib.AwqHipError, match="decode regime"):
+    with pytest.raises(_lib.AwqHipError, match="takes at most 16 rows"):
         awq_gemv_variant(x, *dev, 0, 1)
+    with pytest.raises(_lib.AwqHipError, match="decode regime"):
+        awq_gemv_variant(torch.zeros(65, 256, dtype=torch.float16, device="cuda"), *dev, 0, 1)
     with pytest.raises(AssertionError):
         nq.awq_gemm(x[:, :128], *dev, 8)
     with pytest.raises(AssertionError):
