@@ -1,0 +1,72 @@
+/* C ABI of libawq_hip.so, part 2 -- the kernels of a Qwen3 decode step that sit between the AWQ
+ * linears (include/awq_hip.h): residual add + RMSNorm, per-head q/k RMSNorm + rotary + KV-cache
+ * write, attention of one new token per sequence over a paged KV cache, SiLU(gate) * up.
+ *
+ * Conventions are those of awq_hip.h: device pointers, dense row-major tensors, `dtype` is AWQ_F16
+ * or AWQ_BF16 for every 16-bit tensor of a call, `stream` is a hipStream_t as void*, the return
+ * value is an awq_status and awq_hip_last_error() holds the message of a failure.
+ *
+ * The reference runs these steps as torch modules inside its model (no kernels, no KV cache);
+ * citations name the module code whose arithmetic each entry point reproduces.
+ */
+#ifndef NQ_ENGINE_OPS_H_
+#define NQ_ENGINE_OPS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* residual [rows, hidden] += delta (skipped when delta is NULL; the sum is rounded to dtype as
+ * `x + sublayer(x)` is), then y = dtype(residual_f32 * rsqrt(mean(residual_f32^2) + eps)) * weight.
+ * hidden % 8 == 0, hidden <= 8192.
+ * RMSNorm.rms_norm, nanoquantization/layers/norm.py:18-32; the residual adds of
+ * Qwen3QuantizedBlock.forward, nanoquantization/models/qwen3_quantized.py:194-215. */
+int nq_add_rmsnorm(void* residual, const void* delta, const void* weight, void* y, int64_t rows,
+                   int64_t hidden, float eps, int dtype, void* stream);
+
+/* qkv [rows, (num_heads + 2*num_kv_heads) * head_dim] is the output of the q|k|v projections
+ * side by side.  Every q and k head is RMS-normalised (q_weight / k_weight, [head_dim]) and rotated
+ * (half-split rotary, angle table cos_sin f32 [max_positions, head_dim] = cos | sin) at
+ * positions[row]; q goes to q_out [rows, num_heads, head_dim], k and the untouched v go to
+ * k_cache / v_cache [num_slots, num_kv_heads, head_dim] at slots[row] (a row whose slot is outside
+ * [0, num_slots) writes no k/v).  head_dim even, <= 256.
+ * Qwen3QuantizedAttention.forward, nanoquantization/models/qwen3_quantized.py:79-93;
+ * RoPE.apply_rope / forward, nanoquantization/layers/rope.py:24-45. */
+int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, const void* k_weight,
+                          const float* cos_sin, const int64_t* positions, const int64_t* slots,
+                          void* q_out, void* k_cache, void* v_cache, int64_t rows, int64_t num_heads,
+                          int64_t num_kv_heads, int64_t head_dim, int64_t max_positions,
+                          int64_t num_slots, float eps, int dtype, void* stream);
+
+/* Bytes of device workspace nq_paged_attention_decode needs (0 is possible); no initialisation
+ * needed.  max_context = block_size * max_blocks_per_seq. */
+size_t nq_paged_attention_workspace_bytes(int64_t batch, int64_t num_heads, int64_t num_kv_heads,
+                                          int64_t head_dim, int64_t max_context);
+
+/* out[b, h, :] = softmax(scale * q[b, h, :] . K_b^T) V_b over the first context_lens[b] tokens of
+ * sequence b (the new token's k/v already written).  Token t of sequence b lives in cache slot
+ * block_table[b, t / block_size] * block_size + t % block_size of k_cache / v_cache
+ * [num_blocks * block_size, num_kv_heads, head_dim]; query head h reads kv head
+ * h / (num_heads / num_kv_heads).  q, out: [batch, num_heads, head_dim].  head_dim 64 or 128,
+ * num_heads / num_kv_heads in {1, 2, 4, 8}; block indices are clamped to the cache.
+ * F.scaled_dot_product_attention(..., enable_gqa) of Qwen3QuantizedAttention.forward,
+ * nanoquantization/models/qwen3_quantized.py:94-99, restricted to the last query position. */
+int nq_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
+                              const int32_t* block_table, const int32_t* context_lens, void* out,
+                              int64_t batch, int64_t num_heads, int64_t num_kv_heads,
+                              int64_t head_dim, int64_t block_size, int64_t max_blocks_per_seq,
+                              int64_t num_blocks, float scale, int dtype, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
+/* out[r, i] = dtype(SiLU(gate_up[r, i])) * gate_up[r, inter + i]; gate_up [rows, 2*inter] is the
+ * output of the gate|up projections side by side, out [rows, inter].  inter % 8 == 0.
+ * Qwen3QuantizedMLP.forward, nanoquantization/models/qwen3_quantized.py:147-152. */
+int nq_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NQ_ENGINE_OPS_H_ */

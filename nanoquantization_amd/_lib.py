@@ -23,7 +23,7 @@ _lock = threading.Lock()
 _vp, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
 _LINEAR_ARGS = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]
 
-# symbol -> (restype, argtypes); every symbol of include/awq_hip.h
+# symbol -> (restype, argtypes); every symbol of include/awq_hip.h and include/nq_engine_ops.h
 SYMBOLS = {
     "awq_hip_version": (_int, []),
     "awq_hip_last_error": (ctypes.c_char_p, []),
@@ -42,6 +42,12 @@ SYMBOLS = {
     "awq_gemm_ex_workspace_bytes": (_sz, [_i64, _i64, _i64, _int, _int]),
     "awq_gemv_ex": (_int, _LINEAR_ARGS + [_int, _int]),
     "awq_gemm_ex": (_int, _LINEAR_ARGS + [_int, _int]),
+    # include/nq_engine_ops.h
+    "nq_add_rmsnorm": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_float, _int, _vp]),
+    "nq_qk_norm_rope_store": (_int, [_vp] * 9 + [_i64] * 6 + [ctypes.c_float, _int, _vp]),
+    "nq_paged_attention_workspace_bytes": (_sz, [_i64] * 5),
+    "nq_paged_attention_decode": (_int, [_vp] * 6 + [_i64] * 7 + [ctypes.c_float, _int, _vp, _sz, _vp]),
+    "nq_silu_mul": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
 }
 
 

@@ -1,0 +1,517 @@
+// Kernels of the decode step that sit between the AWQ linears of a Qwen3 block:
+// residual-add + RMSNorm, per-head q/k RMSNorm + rotary + KV-cache write, attention over
+// the paged KV cache, and SiLU(gate)*up.  All of them are HBM/latency bound byte movers;
+// arithmetic is fp32 with the rounding points of the torch modules they stand in for.
+#include "awq_common.hpp"
+#include "../../include/nq_engine_ops.h"
+
+namespace awq {
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T>
+__device__ __forceinline__ void unpack8(u32x4 v, float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t w = v[i];
+        f[2 * i] = T::to_f32((uint16_t)(w & 0xFFFFu));
+        f[2 * i + 1] = T::to_f32((uint16_t)(w >> 16));
+    }
+}
+template <typename T>
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (uint32_t)T::from_f32(f[2 * i]) | ((uint32_t)T::from_f32(f[2 * i + 1]) << 16);
+    return v;
+}
+template <typename T>
+__device__ __forceinline__ float round_to(float f) { return T::to_f32(T::from_f32(f)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// residual (+= delta); y = RMSNorm(residual) * weight.  One workgroup per row, 8 values per lane
+// and pass, at most 4 passes (hidden <= 8192).
+constexpr int kNormThreads = 256;
+constexpr int kNormPasses = 4;
+
+template <typename T>
+__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __restrict__ residual,
+                                                                  const uint16_t* __restrict__ delta,
+                                                                  const uint16_t* __restrict__ weight,
+                                                                  uint16_t* __restrict__ y, int hidden, float eps) {
+    __shared__ float s_part[kNormThreads / kWave];
+    const int64_t base = (int64_t)blockIdx.x * hidden;
+    float v[kNormPasses][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int p = 0; p < kNormPasses; ++p) {
+        const int i = (p * kNormThreads + threadIdx.x) * 8;
+        if (i < hidden) {
+            unpack8<T>(*reinterpret_cast<const u32x4*>(residual + base + i), v[p]);
+            if (delta) {
+                float d[8];
+                unpack8<T>(*reinterpret_cast<const u32x4*>(delta + base + i), d);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[p][e] = round_to<T>(v[p][e] + d[e]);
+                *reinterpret_cast<u32x4*>(residual + base + i) = pack8<T>(v[p]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += v[p][e] * v[p][e];
+        }
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < kNormThreads / kWave; ++w) tot += s_part[w];
+    const float r = rsqrtf(tot / (float)hidden + eps);
+#pragma unroll
+    for (int p = 0; p < kNormPasses; ++p) {
+        const int i = (p * kNormThreads + threadIdx.x) * 8;
+        if (i < hidden) {
+            float w[8], o[8];
+            unpack8<T>(*reinterpret_cast<const u32x4*>(weight + i), w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = round_to<T>(v[p][e] * r) * w[e];
+            *reinterpret_cast<u32x4*>(y + base + i) = pack8<T>(o);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// One wave per (token row, head) of the fused q|k|v projection output.  q and k heads: RMSNorm over
+// the head, then the half-split rotary at the row's position; q goes to q_out, k to its cache
+// slot; v heads are copied to their cache slot.  A lane owns the rotary pairs (i, i + hd/2).
+constexpr int kMaxPairs = 2;  // head_dim <= 256
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
+    const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ q_weight, const uint16_t* __restrict__ k_weight,
+    const float* __restrict__ cos_sin, const int64_t* __restrict__ positions, const int64_t* __restrict__ slots,
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache, int rows, int nh,
+    int nkv, int hd, int max_positions, int64_t num_slots, float eps) {
+    const int heads = nh + 2 * nkv;
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= (int64_t)rows * heads) return;
+    const int row = (int)(item / heads), h = (int)(item % heads), lane = threadIdx.x & 63, half = hd >> 1;
+    const uint16_t* src = qkv + ((int64_t)row * heads + h) * hd;
+    const int64_t slot = slots[row];
+    const bool slot_ok = slot >= 0 && slot < num_slots;
+    uint16_t* dst;
+    if (h < nh) {
+        dst = q_out + ((int64_t)row * nh + h) * hd;
+    } else if (h < nh + nkv) {
+        if (!slot_ok) return;
+        dst = k_cache + (slot * nkv + (h - nh)) * hd;
+    } else {
+        if (!slot_ok) return;
+        dst = v_cache + (slot * nkv + (h - nh - nkv)) * hd;
+    }
+    float a[kMaxPairs], b[kMaxPairs];
+    float ss = 0.f;
+#pragma unroll
+    for (int p = 0; p < kMaxPairs; ++p) {
+        const int i = p * 64 + lane;
+        a[p] = b[p] = 0.f;
+        if (i < half) {
+            a[p] = T::to_f32(src[i]);
+            b[p] = T::to_f32(src[i + half]);
+            ss += a[p] * a[p] + b[p] * b[p];
+        }
+    }
+    if (h >= nh + nkv) {  // v: plain copy
+#pragma unroll
+        for (int p = 0; p < kMaxPairs; ++p) {
+            const int i = p * 64 + lane;
+            if (i < half) {
+                dst[i] = src[i];
+                dst[i + half] = src[i + half];
+            }
+        }
+        return;
+    }
+    const float r = rsqrtf(wave_sum(ss) / (float)hd + eps);
+    const uint16_t* w = h < nh ? q_weight : k_weight;
+    int64_t pos = positions[row];
+    pos = pos < 0 ? 0 : (pos >= max_positions ? max_positions - 1 : pos);
+    const float* cs = cos_sin + pos * hd;
+#pragma unroll
+    for (int p = 0; p < kMaxPairs; ++p) {
+        const int i = p * 64 + lane;
+        if (i < half) {
+            const float x1 = round_to<T>(round_to<T>(a[p] * r) * T::to_f32(w[i]));
+            const float x2 = round_to<T>(round_to<T>(b[p] * r) * T::to_f32(w[i + half]));
+            const float c = cs[i], s = cs[i + half];
+            dst[i] = T::from_f32(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
+            dst[i + half] = T::from_f32(__fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c)));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Attention of one new token per sequence over its paged KV cache (flash-decoding).
+// Workgroup = (sequence, kv head, context split), 4 waves.  A wave covers TPW = 64 / (HD/8) tokens
+// per step: a lane holds 8 head dims of one token's K and V rows (one 16-byte load each), the G
+// query heads of the kv group share those loads.  Every lane group keeps its own online-softmax
+// state (running max, sum, 8 accumulators per query head); the states are merged across lane
+// groups, then waves (LDS), then splits (fp32 partials + a second kernel).
+constexpr float kNegBig = -3.0e38f;
+
+struct SoftState {
+    float m, l;
+};
+
+template <typename T, int G, int HD>
+__global__ __launch_bounds__(256) void paged_attn_decode_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, const int32_t* __restrict__ context_lens, uint16_t* __restrict__ out,
+    float* __restrict__ partial, int nkv, int block_size, int max_blocks, int num_blocks, int nsplit, float scale) {
+    constexpr int LPT = HD / 8;    // lanes per token
+    constexpr int TPW = 64 / LPT;  // tokens per wave step
+    constexpr int U = 2;           // token steps in flight
+    const int sp = blockIdx.x % nsplit;
+    const int kvh = (blockIdx.x / nsplit) % nkv;
+    const int b = blockIdx.x / (nsplit * nkv);
+    const int nh = nkv * G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int dc = lane % LPT, ts = lane / LPT;
+
+    int ctx = context_lens[b];
+    ctx = ctx < 0 ? 0 : (ctx > max_blocks * block_size ? max_blocks * block_size : ctx);
+    const int per = (ctx + nsplit - 1) / nsplit;
+    const int t0 = sp * per, t1 = min(ctx, t0 + per);
+
+    float qf[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        unpack8<T>(*reinterpret_cast<const u32x4*>(q + ((int64_t)b * nh + kvh * G + g) * HD + dc * 8), qf[g]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[g][e] *= scale * kLog2e;
+    }
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = kNegBig;
+        l[g] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    }
+
+    const int32_t* table = block_table + (int64_t)b * max_blocks;
+    for (int t = t0 + wave * TPW + ts; t - ts < t1; t += 4 * TPW * U) {
+        u32x4 kr[U], vr[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int tt = t + u * 4 * TPW;
+            ok[u] = tt < t1;
+            const int tc = ok[u] ? tt : t0;
+            int blk = table[tc / block_size];
+            blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);
+            const int64_t off = (((int64_t)blk * block_size + tc % block_size) * nkv + kvh) * HD + dc * 8;
+            kr[u] = *reinterpret_cast<const u32x4*>(k_cache + off);
+            vr[u] = *reinterpret_cast<const u32x4*>(v_cache + off);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float kf[8], vf[8];
+            unpack8<T>(kr[u], kf);
+            unpack8<T>(vr[u], vf);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float s = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s += qf[g][e] * kf[e];
+#pragma unroll
+                for (int o = LPT / 2; o >= 1; o >>= 1) s += __shfl_xor(s, o);
+                s = ok[u] ? s : kNegBig;
+                const float mn = fmaxf(m[g], s);
+                const float c = exp2f(m[g] - mn);
+                const float p = ok[u] ? exp2f(s - mn) : 0.f;
+                m[g] = mn;
+                l[g] = l[g] * c + p;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * c + p * vf[e];
+            }
+        }
+    }
+
+    // merge the TPW lane groups of this wave
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int o = LPT; o < 64; o <<= 1) {
+            const float mo = __shfl_xor(m[g], o), lo = __shfl_xor(l[g], o);
+            const float mn = fmaxf(m[g], mo);
+            const float ca = exp2f(m[g] - mn), cb = exp2f(mo - mn);
+            l[g] = l[g] * ca + lo * cb;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * ca + __shfl_xor(acc[g][e], o) * cb;
+            m[g] = mn;
+        }
+    }
+    // merge the 4 waves through LDS: [wave][g][HD + 2]
+    __shared__ float s_acc[4][G][HD + 2];
+    if (ts == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s_acc[wave][g][dc * 8 + e] = acc[g][e];
+            if (dc == 0) {
+                s_acc[wave][g][HD] = m[g];
+                s_acc[wave][g][HD + 1] = l[g];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
+        const int g = idx / HD, d = idx % HD;
+        float mn = kNegBig;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) mn = fmaxf(mn, s_acc[w][g][HD]);
+        float lt = 0.f, at = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float c = exp2f(s_acc[w][g][HD] - mn);
+            lt += s_acc[w][g][HD + 1] * c;
+            at += s_acc[w][g][d] * c;
+        }
+        const int64_t head = (int64_t)b * nh + kvh * G + g;
+        if (nsplit == 1) {
+            out[head * HD + d] = T::from_f32(lt > 0.f ? at / lt : 0.f);
+        } else {
+            float* dst = partial + (head * nsplit + sp) * (HD + 2);
+            dst[d] = at;
+            if (d == 0) {
+                dst[HD] = mn;
+                dst[HD + 1] = lt;
+            }
+        }
+    }
+}
+
+// Merge of the context splits: one workgroup of HD threads per (sequence, query head).
+template <typename T, int HD>
+__global__ __launch_bounds__(HD) void paged_attn_merge_kernel(const float* __restrict__ partial,
+                                                              uint16_t* __restrict__ out, int nsplit) {
+    const float* src = partial + (int64_t)blockIdx.x * nsplit * (HD + 2);
+    const int d = threadIdx.x;
+    float mn = kNegBig;
+    for (int s = 0; s < nsplit; ++s) mn = fmaxf(mn, src[s * (HD + 2) + HD]);
+    float lt = 0.f, at = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float c = exp2f(src[s * (HD + 2) + HD] - mn);
+        lt += src[s * (HD + 2) + HD + 1] * c;
+        at += src[s * (HD + 2) + d] * c;
+    }
+    out[(int64_t)blockIdx.x * HD + d] = T::from_f32(lt > 0.f ? at / lt : 0.f);
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[r, i] = SiLU(gate_up[r, i]) * gate_up[r, inter + i], SiLU rounded to the tensor type first.
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate_up,
+                                                       uint16_t* __restrict__ out, int64_t rows, int inter) {
+    const int64_t vec = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int per_row = inter / 8;
+    if (vec >= rows * per_row) return;
+    const int64_t r = vec / per_row;
+    const int i = (int)(vec % per_row) * 8;
+    float g[8], u[8], o[8];
+    unpack8<T>(*reinterpret_cast<const u32x4*>(gate_up + r * 2 * inter + i), g);
+    unpack8<T>(*reinterpret_cast<const u32x4*>(gate_up + r * 2 * inter + inter + i), u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = round_to<T>(g[e] / (1.f + __expf(-g[e]))) * u[e];
+    *reinterpret_cast<u32x4*>(out + r * inter + i) = pack8<T>(o);
+}
+
+int bad(const char* fn, const char* what) {
+    set_error("%s: %s", fn, what);
+    return AWQ_ERR_INVALID_ARG;
+}
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int pick_splits(int64_t batch, int64_t nkv, int64_t max_context) {
+    int64_t s = cdiv(1024, batch * nkv);
+    const int64_t cap = max_context / 64 > 1 ? max_context / 64 : 1;
+    s = s > cap ? cap : s;
+    s = s > 16 ? 16 : s;
+    return (int)(s < 1 ? 1 : s);
+}
+
+template <typename T, int G, int HD>
+void launch_attn(const void* q, const void* kc, const void* vc, const int32_t* table, const int32_t* ctx, void* out,
+                 float* partial, int64_t batch, int nkv, int bs, int max_blocks, int num_blocks, int nsplit,
+                 float scale, hipStream_t st) {
+    paged_attn_decode_kernel<T, G, HD><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(256), 0, st>>>(
+        (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, table, ctx, (uint16_t*)out, partial, nkv, bs,
+        max_blocks, num_blocks, nsplit, scale);
+    if (nsplit > 1)
+        paged_attn_merge_kernel<T, HD><<<dim3((unsigned)(batch * nkv * G)), dim3(HD), 0, st>>>(partial, (uint16_t*)out,
+                                                                                               nsplit);
+}
+
+template <typename T, int HD>
+int launch_attn_g(int G, const void* q, const void* kc, const void* vc, const int32_t* table, const int32_t* ctx,
+                  void* out, float* partial, int64_t batch, int nkv, int bs, int max_blocks, int num_blocks,
+                  int nsplit, float scale, hipStream_t st) {
+    switch (G) {
+#define NQ_CASE(g)                                                                                              \
+    case g:                                                                                                     \
+        launch_attn<T, g, HD>(q, kc, vc, table, ctx, out, partial, batch, nkv, bs, max_blocks, num_blocks,      \
+                              nsplit, scale, st);                                                               \
+        return AWQ_OK;
+        NQ_CASE(1) NQ_CASE(2) NQ_CASE(4) NQ_CASE(8)
+#undef NQ_CASE
+    }
+    set_error("nq_paged_attention_decode: query heads per kv head must be 1, 2, 4 or 8, got %d", G);
+    return AWQ_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+}  // namespace awq
+
+using namespace awq;
+
+extern "C" int nq_add_rmsnorm(void* residual, const void* delta, const void* weight, void* y, int64_t rows,
+                              int64_t hidden, float eps, int dtype, void* stream) {
+    const char* fn = "nq_add_rmsnorm";
+    if (!residual || !weight || !y) return bad(fn, "null pointer argument");
+    if (!aligned16(residual) || !aligned16(weight) || !aligned16(y) || !aligned16(delta))
+        return bad(fn, "every tensor must be 16-byte aligned");
+    if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
+    if (rows <= 0 || hidden <= 0 || hidden % 8 != 0) return bad(fn, "rows > 0 and hidden a positive multiple of 8");
+    if (hidden > kNormThreads * 8 * kNormPasses || rows > 0x7fffffff) {
+        set_error("%s: hidden=%lld exceeds %d", fn, (long long)hidden, kNormThreads * 8 * kNormPasses);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    (void)hipGetLastError();
+    if (dtype == AWQ_F16)
+        add_rmsnorm_kernel<F16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>(
+            (uint16_t*)residual, (const uint16_t*)delta, (const uint16_t*)weight, (uint16_t*)y, (int)hidden, eps);
+    else
+        add_rmsnorm_kernel<BF16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>(
+            (uint16_t*)residual, (const uint16_t*)delta, (const uint16_t*)weight, (uint16_t*)y, (int)hidden, eps);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, const void* k_weight, const float* cos_sin,
+                                     const int64_t* positions, const int64_t* slots, void* q_out, void* k_cache,
+                                     void* v_cache, int64_t rows, int64_t num_heads, int64_t num_kv_heads,
+                                     int64_t head_dim, int64_t max_positions, int64_t num_slots, float eps, int dtype,
+                                     void* stream) {
+    const char* fn = "nq_qk_norm_rope_store";
+    if (!qkv || !q_weight || !k_weight || !cos_sin || !positions || !slots || !q_out || !k_cache || !v_cache)
+        return bad(fn, "null pointer argument");
+    if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
+    if (rows <= 0 || num_heads <= 0 || num_kv_heads <= 0 || max_positions <= 0 || num_slots <= 0)
+        return bad(fn, "rows, head counts, max_positions and num_slots must be positive");
+    if (head_dim <= 0 || head_dim % 2 != 0 || head_dim > 128 * kMaxPairs) {
+        set_error("%s: head_dim must be even and at most %d, got %lld", fn, 128 * kMaxPairs, (long long)head_dim);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    const int64_t items = rows * (num_heads + 2 * num_kv_heads);
+    if (items > ((int64_t)1 << 32)) return bad(fn, "too many rows");
+    hipStream_t st = (hipStream_t)stream;
+    (void)hipGetLastError();
+    const dim3 grid((unsigned)cdiv(items, 4)), block(256);
+    if (dtype == AWQ_F16)
+        qk_norm_rope_store_kernel<F16><<<grid, block, 0, st>>>(
+            (const uint16_t*)qkv, (const uint16_t*)q_weight, (const uint16_t*)k_weight, cos_sin, positions, slots,
+            (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads, (int)num_kv_heads,
+            (int)head_dim, (int)max_positions, num_slots, eps);
+    else
+        qk_norm_rope_store_kernel<BF16><<<grid, block, 0, st>>>(
+            (const uint16_t*)qkv, (const uint16_t*)q_weight, (const uint16_t*)k_weight, cos_sin, positions, slots,
+            (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads, (int)num_kv_heads,
+            (int)head_dim, (int)max_positions, num_slots, eps);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" size_t nq_paged_attention_workspace_bytes(int64_t batch, int64_t num_heads, int64_t num_kv_heads,
+                                                     int64_t head_dim, int64_t max_context) {
+    if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || max_context <= 0) return 0;
+    const int s = pick_splits(batch, num_kv_heads, max_context);
+    return s > 1 ? (size_t)(batch * num_heads * s * (head_dim + 2)) * sizeof(float) : 0;
+}
+
+extern "C" int nq_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
+                                         const int32_t* block_table, const int32_t* context_lens, void* out,
+                                         int64_t batch, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                                         int64_t block_size, int64_t max_blocks_per_seq, int64_t num_blocks, float scale,
+                                         int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "nq_paged_attention_decode";
+    if (!q || !k_cache || !v_cache || !block_table || !context_lens || !out) return bad(fn, "null pointer argument");
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+        return bad(fn, "q, caches and out must be 16-byte aligned");
+    if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
+    if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks_per_seq <= 0 ||
+        num_blocks <= 0 || num_heads % num_kv_heads != 0)
+        return bad(fn, "sizes must be positive and num_heads a multiple of num_kv_heads");
+    if (head_dim != 64 && head_dim != 128) {
+        set_error("%s: head_dim must be 64 or 128, got %lld", fn, (long long)head_dim);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    const int64_t max_context = block_size * max_blocks_per_seq;
+    if (max_context > 0x7fffffff || num_blocks * block_size > 0x7fffffff || batch * num_kv_heads * 16 > 0x7fffffff)
+        return bad(fn, "problem too large");
+    const int nsplit = pick_splits(batch, num_kv_heads, max_context);
+    const size_t need = nq_paged_attention_workspace_bytes(batch, num_heads, num_kv_heads, head_dim, max_context);
+    if (need && (!workspace || workspace_bytes < need || !aligned16(workspace))) {
+        set_error("%s: workspace of %zu bytes needed, %zu given", fn, need, workspace ? workspace_bytes : (size_t)0);
+        return AWQ_ERR_WORKSPACE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    (void)hipGetLastError();
+    const int G = (int)(num_heads / num_kv_heads);
+    int rc;
+    if (dtype == AWQ_F16)
+        rc = head_dim == 128
+                 ? launch_attn_g<F16, 128>(G, q, k_cache, v_cache, block_table, context_lens, out, (float*)workspace,
+                                           batch, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,
+                                           (int)num_blocks, nsplit, scale, st)
+                 : launch_attn_g<F16, 64>(G, q, k_cache, v_cache, block_table, context_lens, out, (float*)workspace,
+                                          batch, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,
+                                          (int)num_blocks, nsplit, scale, st);
+    else
+        rc = head_dim == 128
+                 ? launch_attn_g<BF16, 128>(G, q, k_cache, v_cache, block_table, context_lens, out, (float*)workspace,
+                                            batch, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,
+                                            (int)num_blocks, nsplit, scale, st)
+                 : launch_attn_g<BF16, 64>(G, q, k_cache, v_cache, block_table, context_lens, out, (float*)workspace,
+                                           batch, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,
+                                           (int)num_blocks, nsplit, scale, st);
+    if (rc != AWQ_OK) return rc;
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" int nq_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream) {
+    const char* fn = "nq_silu_mul";
+    if (!gate_up || !out) return bad(fn, "null pointer argument");
+    if (!aligned16(gate_up) || !aligned16(out)) return bad(fn, "tensors must be 16-byte aligned");
+    if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
+    if (rows <= 0 || inter <= 0 || inter % 8 != 0) return bad(fn, "rows > 0 and inter a positive multiple of 8");
+    const int64_t vecs = rows * (inter / 8);
+    if (cdiv(vecs, 256) > 0x7fffffff || inter > 0x3fffffff) return bad(fn, "problem too large");
+    hipStream_t st = (hipStream_t)stream;
+    (void)hipGetLastError();
+    const dim3 grid((unsigned)cdiv(vecs, 256)), block(256);
+    if (dtype == AWQ_F16)
+        silu_mul_kernel<F16><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
+    else
+        silu_mul_kernel<BF16><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}

@@ -9,9 +9,12 @@ linear each -- legal because a packed word holds 8 consecutive output columns an
 multiple of 8 -- so a block costs 4 AWQ launches instead of 7.  The fused buffers are derived at
 start-up; the checkpoint layout is untouched.
 
-Decode.  All per-step inputs live in fixed device buffers (token ids, positions, slots, context
-lengths, block table), attention always spans the table's full width under a length mask, so the
-step has static shapes and is captured once in a HIP graph and replayed.
+Decode.  One step = embedding, then per block: add+RMSNorm kernel, fused q|k|v AWQ GEMV, a kernel that
+does per-head q/k RMSNorm + rotary and writes k/v into their cache slots, paged attention (flash
+decoding over the block table), o_proj GEMV, add+RMSNorm, fused gate|up GEMV, SiLU*up kernel, down GEMV
+(include/nq_engine_ops.h + include/awq_hip.h).  All per-step state lives in fixed device buffers (token
+ids, positions, active mask, block table, step counter, output tokens) and the step advances that
+state itself, so it is captured once in a HIP graph and replayed with no host work between steps.
 """
 from __future__ import annotations
 
@@ -21,6 +24,7 @@ import torch
 import torch.nn.functional as F
 
 from ..layers.gemm import _linear
+from . import ops
 from ..models.qwen3_quantized import Qwen3QuantizedForCausalLM
 
 
@@ -79,14 +83,15 @@ class LLMEngine:
         self.use_graph = use_graph
         self._graph = None
         B, dev = max_batch, self.device
-        # static decode inputs / outputs
-        self.s_ids = torch.zeros(B, dtype=torch.long, device=dev)
-        self.s_pos = torch.zeros(B, dtype=torch.long, device=dev)
-        self.s_slots = torch.zeros(B, dtype=torch.long, device=dev)
-        self.s_ctx = torch.ones(B, dtype=torch.long, device=dev)
-        self.s_table = torch.zeros(B, self.max_blocks, dtype=torch.long, device=dev)
-        self.s_next = torch.zeros(B, dtype=torch.long, device=dev)
-        self._arange_ctx = torch.arange(self.max_ctx, device=dev)
+        # static decode state, advanced on the device by the step itself
+        self.s_ids = torch.zeros(B, dtype=torch.long, device=dev)       # token fed at this step
+        self.s_pos = torch.zeros(B, dtype=torch.long, device=dev)       # its position
+        self.s_active = torch.zeros(B, dtype=torch.bool, device=dev)    # rows that own cache blocks
+        self.s_table = torch.zeros(B, self.max_blocks, dtype=torch.int32, device=dev)
+        self.s_step = torch.zeros(1, dtype=torch.long, device=dev)      # row of s_out the step writes
+        self.s_out = torch.zeros(self.max_ctx + 1, B, dtype=torch.long, device=dev)
+        self.eps = layers[0].input_layernorm.eps
+        self.scale = float(self.hd) ** -0.5
 
     # ---- one transformer block on the cache --------------------------------------------------------
     def _block(self, li: int, x: torch.Tensor, pos: torch.Tensor, slots: torch.Tensor, attend):
@@ -134,34 +139,46 @@ class LLMEngine:
 
     # ---- decode: one token per sequence, attention over the paged cache --------------------------
     def _decode_step(self) -> None:
-        B = self.max_batch
-        mask = (self._arange_ctx.unsqueeze(0) < self.s_ctx.unsqueeze(1)).view(B, 1, 1, self.max_ctx)
-        gqa = self.nh != self.nkv
+        m, bs, eps = self.model.model, self.block_size, self.eps
+        pos = self.s_pos
+        blk = self.s_table.gather(1, (pos // bs).unsqueeze(1)).squeeze(1).long()
+        # idle rows read row 0's table but write nothing: slot -1 is skipped by the kernel
+        slots = torch.where(self.s_active, blk * bs + pos % bs, torch.full_like(pos, -1))
+        ctx = (pos + 1).to(torch.int32)
+        x = m.embed_tokens(self.s_ids)                                   # residual stream [B, hidden]
+        delta = None
+        for li, layer in enumerate(m.layers):
+            attn = layer.self_attn
+            h = ops.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps)
+            q = ops.qk_norm_rope_store(self.qkv[li](h), attn.q_norm.weight, attn.k_norm.weight,
+                                       attn.rope.cos_sin_cache, pos, slots, self.cache.k[li], self.cache.v[li],
+                                       self.nh, self.nkv, self.hd, attn.q_norm.eps)
+            o = ops.paged_attention_decode(q, self.cache.k[li], self.cache.v[li], self.s_table, ctx, self.scale)
+            h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
+            delta = layer.mlp.down_proj(ops.silu_mul(self.gate_up[li](h)))
+        h = ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps)
+        nxt = self.model.lm_head(h).argmax(dim=-1)
+        self.s_out.index_copy_(0, self.s_step, nxt.unsqueeze(0))
+        self.s_ids.copy_(nxt)
+        self.s_pos.add_(1)
+        self.s_step.add_(1)
 
-        def attend(q, k, v, li):
-            kk = self.cache.k[li][self.s_table].view(B, self.max_ctx, self.nkv, self.hd)
-            vv = self.cache.v[li][self.s_table].view(B, self.max_ctx, self.nkv, self.hd)
-            o = F.scaled_dot_product_attention(q.transpose(1, 2), kk.transpose(1, 2), vv.transpose(1, 2),
-                                               attn_mask=mask, enable_gqa=gqa)
-            return o.transpose(1, 2).reshape(B, self.nh * self.hd)
-
-        x = self.model.model.embed_tokens(self.s_ids).unsqueeze(1)
-        pos = self.s_pos.unsqueeze(1)
-        for li in range(len(self.model.model.layers)):
-            x = self._block(li, x, pos, self.s_slots, attend)
-        x = self.model.model.norm(x[:, 0])
-        self.s_next.copy_(self.model.lm_head(x).argmax(dim=-1))
+    def _state(self):
+        return [self.s_ids, self.s_pos, self.s_step]
 
     def _run_decode(self) -> None:
         if not self.use_graph:
             self._decode_step()
             return
         if self._graph is None:
+            saved = [t.clone() for t in self._state()]
             s = torch.cuda.Stream()
             s.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(s):
                 for _ in range(2):          # warm-up: workspaces and library handles exist before capture
                     self._decode_step()
+                    for t, v in zip(self._state(), saved):   # the step advanced the state: put it back
+                        t.copy_(v)
                 torch.cuda.synchronize()
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g, stream=s):
@@ -193,21 +210,19 @@ class LLMEngine:
             nxt = self._prefill(ids, tables)
             out = [nxt.tolist()]
             t1 = time.perf_counter()
-            # batch rows beyond n mirror row 0 (same token, slot and table): they recompute and rewrite
-            # row 0's values, so the step keeps its static shape without touching any other state
+            # batch rows beyond n mirror row 0 (same token, position and table) but are marked idle:
+            # they recompute row 0's token and write nothing to the cache
             rows = list(range(n)) + [0] * (self.max_batch - n)
-            tbl_cpu = torch.tensor(tables)[rows]
-            self.s_table.copy_(tbl_cpu)
-            bs = self.block_size
-            for step in range(1, max_new_tokens):
-                t = plen + step - 1                                  # position of the token being fed
-                self.s_ids.copy_(nxt[rows] if n < self.max_batch else nxt)
-                self.s_pos.fill_(t)
-                self.s_slots.copy_(tbl_cpu[:, t // bs] * bs + t % bs)
-                self.s_ctx.fill_(t + 1)
+            self.s_table.copy_(torch.tensor(tables, dtype=torch.int32)[rows])
+            self.s_active.copy_(torch.tensor([True] * n + [False] * (self.max_batch - n)))
+            self.s_ids.copy_(nxt[rows] if n < self.max_batch else nxt)
+            self.s_pos.fill_(plen)                                   # position of the token being fed
+            self.s_step.zero_()
+            steps = max_new_tokens - 1
+            for _ in range(steps):
                 self._run_decode()
-                nxt = self.s_next[:n].clone()
-                out.append(nxt.tolist())
+            toks = self.s_out[:steps, :n].tolist()                   # one synchronisation for the whole run
+            out.extend(toks)
             if stats is not None:
                 torch.cuda.synchronize()
                 stats.update(prefill_s=t1 - t0, decode_s=time.perf_counter() - t1, decode_steps=max_new_tokens - 1,

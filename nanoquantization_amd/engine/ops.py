@@ -1,0 +1,101 @@
+"""torch-tensor wrappers of the decode-step kernels declared in include/nq_engine_ops.h.
+
+Each function checks shapes on the host, allocates its output with torch (graph-capture safe:
+the caching allocator) and launches on the current stream.  HIP device tensors only."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib
+
+
+def _dev(*ts: torch.Tensor) -> torch.device:
+    dev = ts[0].device
+    if dev.type != "cuda":
+        raise _lib.AwqHipError(f"engine kernels run on a HIP device only (tensor is on {dev})")
+    for t in ts:
+        if t is not None and t.device != dev:
+            raise _lib.AwqHipError(f"tensors on different devices: {t.device} vs {dev}")
+        if t is not None and not t.is_contiguous():
+            raise _lib.AwqHipError("engine kernels take contiguous tensors")
+    return dev
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """residual [rows, hidden] += delta IN PLACE (if given); returns RMSNorm(residual) * weight."""
+    dev = _dev(residual, weight) if delta is None else _dev(residual, delta, weight)
+    rows, hidden = residual.shape
+    assert weight.shape == (hidden,) and weight.dtype == residual.dtype
+    assert delta is None or (delta.shape == residual.shape and delta.dtype == residual.dtype)
+    y = torch.empty_like(residual)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_add_rmsnorm(residual.data_ptr(), None if delta is None else delta.data_ptr(),
+                                             weight.data_ptr(), y.data_ptr(), rows, hidden, eps,
+                                             _lib.dtype_id(residual.dtype), _stream()))
+    return y
+
+
+def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, cos_sin: torch.Tensor,
+                       positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                       num_heads: int, num_kv_heads: int, head_dim: int, eps: float) -> torch.Tensor:
+    """qkv [rows, (nh + 2 nkv) * hd]; caches [..., nkv, hd] viewed as slots; returns q [rows, nh, hd]."""
+    dev = _dev(qkv, q_weight, k_weight, cos_sin, positions, slots, k_cache, v_cache)
+    rows = qkv.shape[0]
+    assert qkv.shape[1] == (num_heads + 2 * num_kv_heads) * head_dim
+    assert q_weight.shape == (head_dim,) and k_weight.shape == (head_dim,)
+    assert q_weight.dtype == qkv.dtype and k_weight.dtype == qkv.dtype
+    assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and k_cache.shape == v_cache.shape
+    assert k_cache.shape[-2:] == (num_kv_heads, head_dim)
+    assert cos_sin.dtype == torch.float32 and cos_sin.numel() % head_dim == 0
+    assert positions.dtype == torch.int64 and slots.dtype == torch.int64
+    assert positions.numel() == rows and slots.numel() == rows
+    num_slots = k_cache.numel() // (num_kv_heads * head_dim)
+    q = torch.empty(rows, num_heads, head_dim, dtype=qkv.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_qk_norm_rope_store(
+            qkv.data_ptr(), q_weight.data_ptr(), k_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(),
+            slots.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), rows, num_heads, num_kv_heads,
+            head_dim, cos_sin.numel() // head_dim, num_slots, eps, _lib.dtype_id(qkv.dtype), _stream()))
+    return q
+
+
+def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                           context_lens: torch.Tensor, scale: float) -> torch.Tensor:
+    """q [batch, nh, hd]; caches [num_blocks, block_size, nkv, hd]; block_table int32 [batch, max_blocks];
+    context_lens int32 [batch].  Returns [batch, nh * hd]."""
+    dev = _dev(q, k_cache, v_cache, block_table, context_lens)
+    batch, nh, hd = q.shape
+    num_blocks, block_size, nkv, hd2 = k_cache.shape
+    assert hd2 == hd and v_cache.shape == k_cache.shape and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype
+    assert block_table.dtype == torch.int32 and context_lens.dtype == torch.int32
+    assert block_table.shape[0] == batch and context_lens.shape == (batch,)
+    max_blocks = block_table.shape[1]
+    out = torch.empty(batch, nh * hd, dtype=q.dtype, device=dev)
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        nbytes = L.nq_paged_attention_workspace_bytes(batch, nh, nkv, hd, block_size * max_blocks)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+        _lib.check(L.nq_paged_attention_decode(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), context_lens.data_ptr(),
+            out.data_ptr(), batch, nh, nkv, hd, block_size, max_blocks, num_blocks, scale, _lib.dtype_id(q.dtype),
+            None if ws is None else ws.data_ptr(), nbytes, _stream()))
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """gate_up [rows, 2*inter] -> SiLU(gate) * up [rows, inter]."""
+    dev = _dev(gate_up)
+    rows, two = gate_up.shape
+    inter = two // 2
+    assert two == 2 * inter
+    out = torch.empty(rows, inter, dtype=gate_up.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_silu_mul(gate_up.data_ptr(), out.data_ptr(), rows, inter,
+                                          _lib.dtype_id(gate_up.dtype), _stream()))
+    return out

@@ -1,0 +1,147 @@
+"""The decode-step kernels (include/nq_engine_ops.h) against plain torch fp32 restatements of the
+module code they stand in for: nanoquantization/layers/norm.py:18-32, layers/rope.py:24-45,
+models/qwen3_quantized.py:79-99 and :147-152.  Tolerances: one rounding step of the tensor type
+(2^-8 relative for bf16, 2^-11 for fp16) on top of fp32 reduction-order noise."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16]
+
+
+def _ulp(dtype):
+    return 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+
+
+def _close(got, want, dtype, scale=1.0, what=""):
+    got, want = got.float(), want.float()
+    err = (got - want).abs().max().item()
+    ref = max(want.abs().max().item(), 1e-6)
+    assert err <= 2.5 * _ulp(dtype) * ref * scale, f"{what}: max err {err} vs max |ref| {ref}"
+
+
+def _rmsnorm_ref(x, w, eps):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * w
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,hidden", [(1, 1024), (32, 1024), (7, 5120), (3, 8192), (5, 136)])
+def test_add_rmsnorm(dtype, rows, hidden):
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator().manual_seed(rows * 131 + hidden)
+    x = torch.randn(rows, hidden, generator=g).to(dtype).cuda()
+    d = torch.randn(rows, hidden, generator=g).to(dtype).cuda()
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype).cuda()
+    y0 = ops.add_rmsnorm(x.clone(), None, w, 1e-6)
+    _close(y0, _rmsnorm_ref(x, w, 1e-6), dtype, what="norm only")
+    res = x.clone()
+    y1 = ops.add_rmsnorm(res, d, w, 1e-6)
+    assert torch.equal(res, x + d), "the residual sum is one rounded add: bit-exact"
+    _close(y1, _rmsnorm_ref(x + d, w, 1e-6), dtype, what="add + norm")
+
+
+def test_add_rmsnorm_rejects_bad_shapes():
+    from nanoquantization_amd import _lib
+    from nanoquantization_amd.engine import ops
+    w = torch.ones(8200, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.AwqHipError, match="exceeds"):
+        ops.add_rmsnorm(torch.zeros(2, 8200, dtype=torch.bfloat16, device="cuda"), None, w, 1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd", [(16, 8, 128), (4, 4, 64), (8, 1, 256), (64, 8, 128)])
+def test_qk_norm_rope_store(dtype, nh, nkv, hd):
+    from nanoquantization_amd.engine import ops
+    from nanoquantization_amd.layers.rope import RoPE
+    rows, num_slots, max_pos = 37, 256, 512
+    g = torch.Generator().manual_seed(nh * 7 + hd)
+    qkv = torch.randn(rows, (nh + 2 * nkv) * hd, generator=g).to(dtype).cuda()
+    qw = (1 + 0.1 * torch.randn(hd, generator=g)).to(dtype).cuda()
+    kw = (1 + 0.1 * torch.randn(hd, generator=g)).to(dtype).cuda()
+    pos = torch.randint(0, max_pos, (rows,), generator=g).cuda()
+    slots = torch.randperm(num_slots, generator=g)[:rows].cuda()
+    slots[5] = -1            # a row that owns no cache slot
+    rope = RoPE(hd, max_pos).cuda()
+    kc = torch.zeros(num_slots, nkv, hd, dtype=dtype, device="cuda")
+    vc = torch.zeros_like(kc)
+    q = ops.qk_norm_rope_store(qkv, qw, kw, rope.cos_sin_cache, pos, slots, kc, vc, nh, nkv, hd, 1e-6)
+
+    qr, kr, vr = torch.split(qkv, [nh * hd, nkv * hd, nkv * hd], dim=-1)
+    qr = _rmsnorm_ref(qr.view(rows, 1, nh, hd), qw, 1e-6)
+    kr = _rmsnorm_ref(kr.view(rows, 1, nkv, hd), kw, 1e-6)
+    qr, kr = rope(qr, kr, pos.view(rows, 1))
+    _close(q, qr.view(rows, nh, hd), dtype, what="q")
+    keep = slots >= 0
+    _close(kc[slots[keep]], kr.view(rows, nkv, hd)[keep], dtype, what="k cache")
+    assert torch.equal(vc[slots[keep]], vr.reshape(rows, nkv, hd)[keep]), "v is copied bit for bit"
+    untouched = torch.ones(num_slots, dtype=torch.bool, device="cuda")
+    untouched[slots[keep]] = False
+    assert not kc[untouched].any() and not vc[untouched].any(), "slots of other tokens must stay untouched"
+
+
+def _attn_ref(q, kc, vc, table, ctx, scale):
+    B, nh, hd = q.shape
+    nb, bs, nkv, _ = kc.shape
+    G = nh // nkv
+    out = torch.empty(B, nh, hd, dtype=torch.float32, device=q.device)
+    for b in range(B):
+        n = int(ctx[b])
+        t = torch.arange(n, device=q.device)
+        sl = table[b, t // bs].long() * bs + t % bs
+        k = kc.view(-1, nkv, hd)[sl].float().repeat_interleave(G, dim=1)      # [n, nh, hd]
+        v = vc.view(-1, nkv, hd)[sl].float().repeat_interleave(G, dim=1)
+        s = torch.einsum("hd,nhd->hn", q[b].float(), k) * scale
+        out[b] = torch.einsum("hn,nhd->hd", torch.softmax(s, dim=-1), v)
+    return out.view(B, nh * hd)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,nh,nkv,hd,bs,max_blocks", [
+    (32, 16, 8, 128, 64, 12),     # Qwen3-0.6B decode, context splits
+    (3, 16, 8, 128, 16, 5),       # tiny context: fewer tokens than lanes
+    (64, 64, 8, 128, 64, 4),      # 8 query heads per kv head
+    (5, 4, 4, 64, 32, 9),         # head_dim 64, no grouping
+    (130, 8, 8, 128, 64, 1),      # one block per sequence, single split
+    (2, 4, 1, 128, 48, 7),        # block size that is not a power of two
+])
+def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator().manual_seed(B * 1000 + nh)
+    nb = B * max_blocks + 3
+    kc = torch.randn(nb, bs, nkv, hd, generator=g).to(dtype).cuda()
+    vc = torch.randn(nb, bs, nkv, hd, generator=g).to(dtype).cuda()
+    q = torch.randn(B, nh, hd, generator=g).to(dtype).cuda()
+    table = torch.randperm(nb, generator=g)[: B * max_blocks].view(B, max_blocks).to(torch.int32).cuda()
+    ctx = torch.randint(1, bs * max_blocks + 1, (B,), generator=g).to(torch.int32)
+    ctx[0] = 1
+    ctx[-1] = bs * max_blocks
+    ctx = ctx.cuda()
+    scale = 1.0 / math.sqrt(hd)
+    out = ops.paged_attention_decode(q, kc, vc, table, ctx, scale)
+    _close(out, _attn_ref(q, kc, vc, table, ctx, scale), dtype, scale=2.0, what="attention")
+    assert torch.equal(out, ops.paged_attention_decode(q, kc, vc, table, ctx, scale)), "run-to-run bit-stable"
+
+
+def test_paged_attention_rejects_unsupported():
+    from nanoquantization_amd import _lib
+    from nanoquantization_amd.engine import ops
+    kc = torch.zeros(4, 16, 1, 128, dtype=torch.bfloat16, device="cuda")
+    q = torch.zeros(1, 3, 128, dtype=torch.bfloat16, device="cuda")
+    tb = torch.zeros(1, 2, dtype=torch.int32, device="cuda")
+    cx = torch.ones(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(_lib.AwqHipError, match="1, 2, 4 or 8"):
+        ops.paged_attention_decode(q, kc, kc, tb, cx, 1.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,inter", [(1, 3072), (32, 3072), (9, 25600), (3, 8)])
+def test_silu_mul(dtype, rows, inter):
+    import torch.nn.functional as F
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator().manual_seed(rows + inter)
+    gu = (2 * torch.randn(rows, 2 * inter, generator=g)).to(dtype).cuda()
+    _close(ops.silu_mul(gu), F.silu(gu[:, :inter]) * gu[:, inter:], dtype, what="silu*up")

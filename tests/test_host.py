@@ -25,12 +25,13 @@ def _ensure_built():
 def test_library_exports_every_declared_symbol():
     _ensure_built()
     header = open(os.path.join(ROOT, "include", "awq_hip.h")).read()
-    declared = set(re.findall(r"\b(awq_[a-z0-9_]+)\s*\(", header))
+    header += open(os.path.join(ROOT, "include", "nq_engine_ops.h")).read()
+    declared = set(re.findall(r"\b((?:awq|nq)_[a-z0-9_]+)\s*\(", header))
     declared -= {"awq_status", "awq_dtype"}
     assert declared, "no declarations parsed"
     handle = ctypes.CDLL(_lib.LIB_PATH)
     for name in sorted(declared):
-        assert hasattr(handle, name), f"{name} declared in include/awq_hip.h but not exported"
+        assert hasattr(handle, name), f"{name} declared in include/*.h but not exported"
     assert declared == set(_lib.SYMBOLS), "ctypes table and header disagree"
     L = _lib.lib()
     assert L.awq_hip_version() >= 100
