@@ -23,65 +23,11 @@
 // Split-K: as in the GEMV, fp32 partials + an arrival counter per tile; the
 // last workgroup adds the partials in split order.
 #include "awq_common.hpp"
+#include "awq_gemm_parts.hpp"
 
 namespace awq {
 
 constexpr int kBK = 64;
-
-template <typename T>
-struct UnpackRows;
-
-// fp16: returns, for byte-pair i (columns 2i, 2i+1) of one word, the packed
-// pair of dequantised halves.
-template <>
-struct UnpackRows<F16> {
-    uint32_t zp[4];
-    f16x2 sc[4];
-    __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            zp[i] = ((zw >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            sc[i] = as_f16x2(sv[i]);
-        }
-    }
-    // out[c] = (W[k, c], W[k+1, c]) for the 8 columns of the word pair (w0 = row k, w1 = row k+1)
-    __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t q0 = ((w0 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            uint32_t q1 = ((w1 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
-            f16x2 d0 = (as_f16x2(q0) - as_f16x2(zp[i])) * sc[i];
-            f16x2 d1 = (as_f16x2(q1) - as_f16x2(zp[i])) * sc[i];
-            uint32_t u0 = as_u32(d0), u1 = as_u32(d1);
-            // columns 2i (low halves) and 2i+1 (high halves), rows k / k+1
-            out[2 * i] = __builtin_amdgcn_perm(u1, u0, 0x05040100u);
-            out[2 * i + 1] = __builtin_amdgcn_perm(u1, u0, 0x07060302u);
-        }
-    }
-};
-
-template <>
-struct UnpackRows<BF16> {
-    float sc[8], nzs[8];  // s and -(z * s), both exact in fp32
-    __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const uint32_t pr = sv[c >> 1];
-            sc[c] = __builtin_bit_cast(float, (c & 1) ? (pr & 0xFFFF0000u) : (pr << 16));
-            nzs[c] = -(float)((zw >> nibble_shift(c)) & 0xFu) * sc[c];
-        }
-    }
-    __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const float q0 = (float)((w0 >> nibble_shift(c)) & 0xFu);
-            const float q1 = (float)((w1 >> nibble_shift(c)) & 0xFu);
-            // q*s - z*s: the exact value (q-z)*s has <= 13 significant bits, so the
-            // fused multiply-add returns it exactly.
-            out[c] = BF16::pack2(__builtin_fmaf(q0, sc[c], nzs[c]), __builtin_fmaf(q1, sc[c], nzs[c]));
-        }
-    }
-};
 
 // LDS slot (16-byte unit) of A row `row`, k-chunk `kc` (8 k's) inside a [8][BM] buffer
 template <int BM>
@@ -248,65 +194,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
         }
     }
 
-    // ---- epilogue -----------------------------------------------------------
-    // acc[a][b][v]: row (v/4)*8 + kb2*4 + v%4, column li of the 32x32 tile
-    const bool direct = splits == 1;
-#pragma unroll
-    for (int a = 0; a < TM; ++a)
-#pragma unroll
-        for (int b = 0; b < TN; ++b) {
-            const int n = n0 + wn0 + b * 32 + li;
-            if (n >= N) continue;
-            float bv = 0.f;
-            if (direct && bias) bv = T::to_f32(bias[n]);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = m0 + wm0 + a * 32 + (v >> 2) * 8 + kb2 * 4 + (v & 3);
-                if (m >= M) continue;
-                if (direct)
-                    y[(size_t)m * N + n] = T::from_f32(acc[a][b][v] + bv);
-                else
-                    publish_f32(&partials[((size_t)split * M + m) * N + n], acc[a][b][v]);
-            }
-        }
-    if (direct) return;
-
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
-    if (!arrive_last(&counters[tile], splits, &s_last)) return;
-    const int rows = min(BM, M - m0);
-    const int wcount = min(WCOLS, words - (n0 >> 3));
-    for (int idx = tid; idx < rows * wcount; idx += NT) {
-        const int m = m0 + idx / wcount;
-        const size_t nn = (size_t)n0 + (size_t)(idx % wcount) * 8;
-        float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int s0 = 0; s0 < splits; s0 += 8) {   // 8 splits in flight, added in split order
-            float v[8][8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int s = min(s0 + u, splits - 1);
-                const float* p = partials + ((size_t)s * M + m) * N + nn;
-#pragma unroll
-                for (int c = 0; c < 8; ++c) v[u][c] = fetch_f32(p + c);
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (s0 + u < splits) {
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) out[c] += v[u][c];
-                }
-        }
-        if (bias) {
-            const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-                out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
-        }
-        u32x4 o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
-        *reinterpret_cast<u32x4*>(y + (size_t)m * N + nn) = o;
-    }
-    if (tid == 0) __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, counters, &s_last, M, N, m0, n0, wm0, wn0, split, splits);
 }
 
 // ---- host side -------------------------------------------------------------
@@ -318,7 +206,9 @@ static const GemmVariant kGemmVariants[] = {
     {"256x256w8", 256, 256, 8}, {"128x256w8", 128, 256, 8}, {"128x128", 128, 128, 4},
     {"64x256", 64, 256, 4},     {"32x256", 32, 256, 4},     {"64x128", 64, 128, 4},
     {"256x256", 256, 256, 4},   {"128x256", 128, 256, 4},   {"256x128w8", 256, 128, 8},
+    {"256x256p", 256, 256, 4},  // the software-pipelined kernel of awq_gemm_pipe.hip
 };
+constexpr int kPipeVariant = 9;
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 template <typename T, int BM, int BN, int WM, int WN>
@@ -373,7 +263,7 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
 static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     const int kCUs = 256;
     // indices into kGemmVariants
-    constexpr int k256x256 = 6, k128x128 = 2, k64x256 = 3, k32x256 = 4;
+    constexpr int k256x256 = kPipeVariant, k128x128 = 2, k64x256 = 3, k32x256 = 4;
     int v;
     if (M <= 32) v = k32x256;
     else if (M <= 64) v = k64x256;
@@ -446,6 +336,10 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         AWQ_GEMM_CASE(6, 256, 256, 2, 2)
         AWQ_GEMM_CASE(7, 128, 256, 2, 2)
         AWQ_GEMM_CASE(8, 256, 128, 4, 2)
+        case kPipeVariant:
+            e = launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+                                 workspace, split_k, s);
+            break;
     }
 #undef AWQ_GEMM_CASE
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);

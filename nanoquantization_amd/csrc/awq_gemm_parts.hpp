@@ -1,0 +1,142 @@
+// Pieces shared by the fused dequant+GEMM kernels: the register unpack of packed words into
+// k-pairs of dequantised values, and the epilogue: direct store (+ bias) of a workgroup's
+// BM x BN tile, or the split-K exchange (fp32 partials, arrival counter, in-order sum by the
+// last workgroup to arrive).
+#pragma once
+
+#include "awq_common.hpp"
+
+namespace awq {
+
+template <typename T>
+struct UnpackRows;
+
+// fp16: returns, for byte-pair i (columns 2i, 2i+1) of one word, the packed
+// pair of dequantised halves.
+template <>
+struct UnpackRows<F16> {
+    uint32_t zp[4];
+    f16x2 sc[4];
+    __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            zp[i] = ((zw >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            sc[i] = as_f16x2(sv[i]);
+        }
+    }
+    // out[c] = (W[k, c], W[k+1, c]) for the 8 columns of the word pair (w0 = row k, w1 = row k+1)
+    __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t q0 = ((w0 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            uint32_t q1 = ((w1 >> (4 * i)) & 0x000F000Fu) | 0x64006400u;
+            f16x2 d0 = (as_f16x2(q0) - as_f16x2(zp[i])) * sc[i];
+            f16x2 d1 = (as_f16x2(q1) - as_f16x2(zp[i])) * sc[i];
+            uint32_t u0 = as_u32(d0), u1 = as_u32(d1);
+            // columns 2i (low halves) and 2i+1 (high halves), rows k / k+1
+            out[2 * i] = __builtin_amdgcn_perm(u1, u0, 0x05040100u);
+            out[2 * i + 1] = __builtin_amdgcn_perm(u1, u0, 0x07060302u);
+        }
+    }
+};
+
+template <>
+struct UnpackRows<BF16> {
+    float sc[8], nzs[8];  // s and -(z * s), both exact in fp32
+    __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t pr = sv[c >> 1];
+            sc[c] = __builtin_bit_cast(float, (c & 1) ? (pr & 0xFFFF0000u) : (pr << 16));
+            nzs[c] = -(float)((zw >> nibble_shift(c)) & 0xFu) * sc[c];
+        }
+    }
+    __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float q0 = (float)((w0 >> nibble_shift(c)) & 0xFu);
+            const float q1 = (float)((w1 >> nibble_shift(c)) & 0xFu);
+            // q*s - z*s: the exact value (q-z)*s has <= 13 significant bits, so the
+            // fused multiply-add returns it exactly.
+            out[c] = BF16::pack2(__builtin_fmaf(q0, sc[c], nzs[c]), __builtin_fmaf(q1, sc[c], nzs[c]));
+        }
+    }
+};
+
+
+// acc[a][b][v] of the 32x32x16 MFMA: row (v/4)*8 + (lane/32)*4 + v%4, column lane%32 of tile
+// (a, b) of the wave's sub-tile at (wm0, wn0).
+template <typename T, int BM, int BN, int TM, int TN, int NT>
+__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const uint16_t* __restrict__ bias,
+                                              uint16_t* __restrict__ y, float* __restrict__ partials,
+                                              int* __restrict__ counters, int* s_last_p, int M, int N, int m0,
+                                              int n0, int wm0, int wn0, int split, int splits) {
+    constexpr int WCOLS = BN / 8;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int li = lane & 31, kb2 = lane >> 5;
+    const int words = N >> 3;
+    const bool direct = splits == 1;
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b) {
+            const int n = n0 + wn0 + b * 32 + li;
+            if (n >= N) continue;
+            float bv = 0.f;
+            if (direct && bias) bv = T::to_f32(bias[n]);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm0 + a * 32 + (v >> 2) * 8 + kb2 * 4 + (v & 3);
+                if (m >= M) continue;
+                if (direct)
+                    y[(size_t)m * N + n] = T::from_f32(acc[a][b][v] + bv);
+                else
+                    publish_f32(&partials[((size_t)split * M + m) * N + n], acc[a][b][v]);
+            }
+        }
+    if (direct) return;
+
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    if (!arrive_last(&counters[tile], splits, s_last_p)) return;
+    const int rows = min(BM, M - m0);
+    const int wcount = min(WCOLS, words - (n0 >> 3));
+    for (int idx = tid; idx < rows * wcount; idx += NT) {
+        const int m = m0 + idx / wcount;
+        const size_t nn = (size_t)n0 + (size_t)(idx % wcount) * 8;
+        float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int s0 = 0; s0 < splits; s0 += 8) {   // 8 splits in flight, added in split order
+            float v[8][8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int s = min(s0 + u, splits - 1);
+                const float* p = partials + ((size_t)s * M + m) * N + nn;
+#pragma unroll
+                for (int c = 0; c < 8; ++c) v[u][c] = fetch_f32(p + c);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < splits) {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) out[c] += v[u][c];
+                }
+        }
+        if (bias) {
+            const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
+        }
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+        *reinterpret_cast<u32x4*>(y + (size_t)m * N + nn) = o;
+    }
+    if (tid == 0) __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// awq_gemm_pipe.hip: the 256 x 256 software-pipelined kernel (same arguments as the tiled launcher).
+hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
+                            const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
+                            void* workspace, int split_k, hipStream_t stream);
+
+}  // namespace awq

@@ -1,0 +1,295 @@
+// Kernel (c), large-M form: fused dequant + GEMM on the 32x32x16 MFMA with the unpack hidden
+// behind the matrix cores.
+//
+// A workgroup of 4 wavefronts (2 x 2) owns a 256 x 256 output tile and walks K in steps of 64.
+// LDS holds two buffers of { A tile, dequantised B tile }:
+//   A: x[m0.., k0..k0+63] lands straight from global memory (global_load_lds, no registers, no
+//      vector ALU), row-major, the eight 16-byte chunks of a row XOR-swizzled by the row number;
+//   B: packed words go global -> registers one step ahead; while the MFMAs of step i run, the
+//      same wave turns the words of step i+1 into RN_dtype((q - z) * s) -- two k rows at a time,
+//      one pair of rows per quarter of the MFMAs -- and stores them k-contiguous for step i+1.
+// The instruction order of a step is pinned with scheduling-group barriers: one MFMA, a few
+// vector-ALU instructions, an LDS read of the next operands, and so on, so that the matrix core
+// never waits for the unpack.
+//
+// bf16 unpack: a nibble is masked in place at mantissa bit 8, 12 or 16 of the fp32 pattern
+// 0x4B000000 (value 2^23 + q * 2^e), so  fma(f, s * 2^-e, -(2^(23-e) + z) * s) = (q - z) * s
+// exactly: the product and the constant have at most 24 significant bits each, and the sum has at
+// most 13.  Nibbles 0-1 and 5-7 are brought to those positions by one shift of the word each.
+#include "awq_common.hpp"
+#include "awq_gemm_parts.hpp"
+
+namespace awq {
+namespace {
+
+constexpr int kPBK = 64;
+
+#define AWQ_GPTR(p) ((__attribute__((address_space(1))) const void*)(p))
+#define AWQ_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// ---- LDS layouts (16-byte slots) ----------------------------------------------------------------
+// A [256 rows][8 chunks]: chunk kc of `row` sits at row*8 + (kc ^ swz(row)).  32 consecutive rows
+// at one kc (an MFMA operand read) touch every 16-byte bank group once, whether the LDS serves 8
+// or 16 lanes per cycle.
+__device__ __forceinline__ int row_swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+// B [8 k-blocks][2][8 columns c][16 word columns]: conflict-free for the writer (32 word columns
+// at one c) and the reader (32 consecutive columns at one k-block).
+__device__ __forceinline__ int b_slot_p(int wc, int c, int kblk) {
+    return kblk * 256 + ((wc >> 4) << 7) + (c << 4) + ((wc & 15) ^ c ^ ((c & 1) << 3));
+}
+
+// ---- unpack of two k rows of one word column ----------------------------------------------------
+template <typename T>
+struct PipeUnpack : UnpackRows<T> {
+    __device__ __forceinline__ void init() {}
+};
+
+template <>
+struct PipeUnpack<BF16> {
+    float sc[8], off[8];
+    uint32_t mask8, mask12, mask16, magic;
+    // column c lives in nibble 4*(c&1) + (c>>1); where it is picked up after the shifts:
+    static __device__ __forceinline__ constexpr int src_of(int c) {   // 0: w << 8, 1: w, 2: w >> 12
+        const int jn = 4 * (c & 1) + (c >> 1);
+        return jn < 2 ? 0 : (jn < 5 ? 1 : 2);
+    }
+    static __device__ __forceinline__ constexpr int bit_of(int c) {   // 8, 12 or 16
+        const int jn = 4 * (c & 1) + (c >> 1);
+        return jn < 2 ? 4 * jn + 8 : (jn < 5 ? 4 * jn : 4 * jn - 12);
+    }
+    __device__ __forceinline__ void init() {
+        mask8 = 0xF00u; mask12 = 0xF000u; mask16 = 0xF0000u; magic = 0x4B000000u;
+        asm volatile("" : "+s"(mask8), "+s"(mask12), "+s"(mask16));
+        asm volatile("" : "+v"(magic));
+    }
+    __device__ __forceinline__ float embed(uint32_t w, uint32_t wl, uint32_t wh, int c) const {
+        const uint32_t src = src_of(c) == 0 ? wl : (src_of(c) == 1 ? w : wh);
+        const uint32_t m = bit_of(c) == 8 ? mask8 : (bit_of(c) == 12 ? mask12 : mask16);
+        return __builtin_bit_cast(float, (src & m) | magic);
+    }
+    __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
+        const uint32_t zl = zw << 8, zh = zw >> 12;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t pr = sv[c >> 1];
+            const float s = __builtin_bit_cast(float, (c & 1) ? (pr & 0xFFFF0000u) : (pr << 16));
+            const float down = bit_of(c) == 8 ? 0x1p-8f : (bit_of(c) == 12 ? 0x1p-12f : 0x1p-16f);
+            sc[c] = s * down;                               // exact: a power of two
+            off[c] = -(embed(zw, zl, zh, c) * sc[c]);       // (2^(23-e) + z) * s, <= 24 significant bits
+        }
+    }
+    __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
+        const uint32_t l0 = w0 << 8, h0 = w0 >> 12, l1 = w1 << 8, h1 = w1 >> 12;
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            out[c] = BF16::pack2(__builtin_fmaf(embed(w0, l0, h0, c), sc[c], off[c]),
+                                 __builtin_fmaf(embed(w1, l1, h1, c), sc[c], off[c]));
+    }
+};
+
+struct Raw {
+    uint32_t w[8];
+    uint32_t z;
+    u32x4 s;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_pipe_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
+    const uint32_t* __restrict__ qzeros, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
+    float* __restrict__ partials, int* __restrict__ counters, int M, int N, int K, int g, int iters_per_split,
+    int splits) {
+    constexpr int BM = 256, BN = 256, TM = 4, TN = 4, NT = 256;
+    constexpr int A_SLOTS = 8 * BM, B_SLOTS = 8 * BN, BUF = A_SLOTS + B_SLOTS;
+    extern __shared__ u32x4 lds[];  // [2][BUF]
+    __shared__ int s_last;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int split = blockIdx.z;
+    const int words = N >> 3;
+    const int total_iters = K / kPBK;
+    const int it_begin = split * iters_per_split;
+    const int it_end = min(it_begin + iters_per_split, total_iters);
+
+    // ---- A: 8 direct-to-LDS loads per wave and step; load i of wave w fills slots (8w+i)*64 + lane,
+    //      i.e. rows 8*(8w+i) + lane/8, whose chunk at position lane%8 is kc = lane%8 ^ swz(row).
+    //      Rows past M read the last row; their results are never stored.
+    const uint16_t* a_src[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = (wave * 8 + i) * 8 + (lane >> 3);
+        const int kc = (lane & 7) ^ row_swz(row);
+        a_src[i] = x + (size_t)min(m0 + row, M - 1) * K + kc * 8;
+    }
+    auto dma_a = [&](int it, int buf) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            __builtin_amdgcn_global_load_lds(AWQ_GPTR(a_src[i] + it * kPBK),
+                                             AWQ_LPTR(lds + buf * BUF + (wave * 8 + i) * 64), 16, 0, 0);
+    };
+
+    // ---- B: a lane owns word column wc for the 8 k rows of block rb ---------------------------------
+    const int wc = tid & 31, rb = tid >> 5;
+    const int gwc = min((n0 >> 3) + wc, words - 1);
+    const uint32_t w_off = (uint32_t)(rb * 8) * (uint32_t)words + (uint32_t)gwc;
+    const int g_lane = (rb * 8) / g;  // host guarantees g % 64 == 0 or 64 % g == 0
+    auto load_raw = [&](int it, Raw& r) {
+        const int k0 = it * kPBK;
+        const uint32_t* wp = qweight + (size_t)k0 * words;  // uniform
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r.w[i] = (wp + (size_t)i * words)[w_off];
+        const int gi = k0 / g + g_lane;
+        r.z = qzeros[(size_t)gi * words + gwc];
+        r.s = *reinterpret_cast<const u32x4*>(scales + ((size_t)gi * words + gwc) * 8);
+    };
+    int b_wr[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) b_wr[c] = b_slot_p(wc, c, rb);
+
+    // ---- MFMA operand addresses ------------------------------------------------------------------
+    const int li = lane & 31, kb2 = lane >> 5;
+    int a_rd[4];  // row wm0 + li at k-step ks; + 256 slots per further 32 rows
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) a_rd[ks] = (wm0 + li) * 8 + ((2 * ks + kb2) ^ row_swz(wm0 + li));
+    int b_rd[TN];  // column wn0 + 32b + li at k-block kb2; + 512 slots per k-step
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+        const int n = wn0 + b * 32 + li;
+        b_rd[b] = b_slot_p(n >> 3, n & 7, kb2);
+    }
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+
+    PipeUnpack<T> up;
+    up.init();
+
+    // one K step: MFMAs of tile `it` (LDS buffer `buf`) interleaved with the unpack of tile it+1 (`cur`,
+    // stored to the other buffer), while the packed words of tile it+2 travel to `nxt`
+    auto step = [&](int it, int buf, Raw& cur, Raw& nxt) {
+        load_raw(min(it + 2, it_end - 1), nxt);
+        const u32x4* abase = lds + buf * BUF;
+        const u32x4* bbase = abase + A_SLOTS;
+        up.set_group(cur.z, cur.s);
+        uint32_t cols[8][4];
+        u32x4 af[2][TM], bf[2][TN];
+#pragma unroll
+        for (int a = 0; a < TM; ++a) af[0][a] = abase[a_rd[0] + a * 256];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) bf[0][b] = bbase[b_rd[b]];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int p = ks & 1;
+            if (ks < 3) {
+#pragma unroll
+                for (int a = 0; a < TM; ++a) af[p ^ 1][a] = abase[a_rd[ks + 1] + a * 256];
+#pragma unroll
+                for (int b = 0; b < TN; ++b) bf[p ^ 1][b] = bbase[b_rd[b] + (ks + 1) * 512];
+            }
+            uint32_t o[8];
+            up.pair(cur.w[2 * ks], cur.w[2 * ks + 1], o);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) cols[c][ks] = o[c];
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b) acc[a][b] = T::mfma32(af[p][a], bf[p][b], acc[a][b]);
+        }
+        u32x4* wbase = lds + (buf ^ 1) * BUF + A_SLOTS;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) wbase[b_wr[c]] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
+        // pinned order: first the operands of k-step 0, then per MFMA a slice of the unpack, with the
+        // operand reads of the next k-step spread over the first half of each k-step
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // 8 LDS reads
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // 4 vector ALU
+                if (ks < 3 && m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+        __builtin_amdgcn_sched_group_barrier(0x200, 8, 0);  // 8 LDS writes
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the A tile of step it+1 has landed
+        asm volatile("" ::: "memory");
+        __syncthreads();
+        if (it + 2 < it_end) dma_a(it + 2, buf);
+    };
+
+    if (it_begin < it_end) {
+        Raw r0, r1;
+        dma_a(it_begin, 0);
+        load_raw(it_begin, r0);
+        load_raw(min(it_begin + 1, it_end - 1), r1);
+        {
+            up.set_group(r0.z, r0.s);
+            u32x4* wbase = lds + A_SLOTS;
+            uint32_t cols[8][4];
+#pragma unroll
+            for (int rp = 0; rp < 4; ++rp) {
+                uint32_t o[8];
+                up.pair(r0.w[2 * rp], r0.w[2 * rp + 1], o);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) cols[c][rp] = o[c];
+            }
+#pragma unroll
+            for (int c = 0; c < 8; ++c) wbase[b_wr[c]] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
+        }
+        if (it_begin + 1 < it_end) dma_a(it_begin + 1, 1);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" ::: "memory");
+        __syncthreads();
+        for (int it = it_begin; it < it_end; it += 2) {
+            step(it, 0, r1, r0);
+            if (it + 1 < it_end) step(it + 1, 1, r0, r1);
+        }
+    }
+    gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, counters, &s_last, M, N, m0, n0, wm0, wn0, split,
+                                         splits);
+}
+
+}  // namespace
+
+hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
+                            const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
+                            void* workspace, int split_k, hipStream_t stream) {
+    const int tiles_m = (int)cdiv(M, 256), tiles_n = (int)cdiv(N, 256);
+    const int total_iters = K / kPBK;
+    const int ips = (int)cdiv(total_iters, split_k);
+    const int splits = (int)cdiv(total_iters, ips);
+    int* counters = reinterpret_cast<int*>(workspace);
+    float* partials =
+        workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes) : nullptr;
+    const size_t lds = (size_t)2 * (8 * 256 + 8 * 256) * 16;  // 128 KiB
+    const void* kern = dtype == AWQ_F16 ? reinterpret_cast<const void*>(gemm_pipe_kernel<F16>)
+                                        : reinterpret_cast<const void*>(gemm_pipe_kernel<BF16>);
+    static bool raised[2] = {false, false};
+    if (!raised[dtype]) {
+        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        raised[dtype] = true;
+    }
+    (void)hipGetLastError();
+    auto go = [&](auto k) {
+        hipLaunchKernelGGL(k, dim3(tiles_n, tiles_m, splits), dim3(256), lds, stream,
+                           reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
+                           reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
+                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials,
+                           counters, M, N, K, g, ips, splits);
+    };
+    if (dtype == AWQ_F16) go(gemm_pipe_kernel<F16>);
+    else go(gemm_pipe_kernel<BF16>);
+    return hipGetLastError();
+}
+
+}  // namespace awq
