@@ -31,6 +31,9 @@ EXTRA = {
     # keep MFMA results in VGPRs: the GEMV folds every accumulator into fp32 state right away,
     # AGPR destinations would cost a v_accvgpr_read per value and 4 more registers per wave
     "awq_gemv.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    # the SLP vectoriser pairs the two k rows of the unpack into <2 x i32> and/or, which then no
+    # longer select as one v_and_or_b32 each
+    "awq_gemm_pipe.hip": ["-fno-slp-vectorize"],
 }
 
 

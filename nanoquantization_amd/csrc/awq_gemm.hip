@@ -207,6 +207,7 @@ static const GemmVariant kGemmVariants[] = {
     {"64x256", 64, 256, 4},     {"32x256", 32, 256, 4},     {"64x128", 64, 128, 4},
     {"256x256", 256, 256, 4},   {"128x256", 128, 256, 4},   {"256x128w8", 256, 128, 8},
     {"256x256p", 256, 256, 4},  // the software-pipelined kernel of awq_gemm_pipe.hip
+    {"256x256pw8", 256, 256, 8},  // the same with two wavefronts per SIMD
 };
 constexpr int kPipeVariant = 9;
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
@@ -337,7 +338,8 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         AWQ_GEMM_CASE(7, 128, 256, 2, 2)
         AWQ_GEMM_CASE(8, 256, 128, 4, 2)
         case kPipeVariant:
-            e = launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+        case kPipeVariant + 1:
+            e = launch_gemm_pipe(dtype, variant == kPipeVariant ? 4 : 8, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
                                  workspace, split_k, s);
             break;
     }

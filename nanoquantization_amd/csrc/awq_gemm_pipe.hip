@@ -1,7 +1,12 @@
 // Kernel (c), large-M form: fused dequant + GEMM on the 32x32x16 MFMA with the unpack hidden
 // behind the matrix cores.
 //
-// A workgroup of 4 wavefronts (2 x 2) owns a 256 x 256 output tile and walks K in steps of 64.
+// A workgroup of 4 (2 x 2) or 8 (2 x 4) wavefronts owns a 256 x 256 output tile and walks K in
+// steps of 64.  A SIMD issues one instruction per wavefront every four cycles, and the unpack
+// adds some 240 vector-ALU instructions to the 64 MFMAs of a step: with one wavefront per SIMD
+// the issue slots, not the matrix core, set the pace.  With 8 wavefronts (two per SIMD, 128
+// accumulator registers each) one wavefront's MFMA issues beside the other's unpack and LDS
+// traffic.
 // LDS holds two buffers of { A tile, dequantised B tile }:
 //   A: x[m0.., k0..k0+63] lands straight from global memory (global_load_lds, no registers, no
 //      vector ALU), row-major, the eight 16-byte chunks of a row XOR-swizzled by the row number;
@@ -68,7 +73,8 @@ struct PipeUnpack<BF16> {
         return __builtin_bit_cast(float, (src & m) | magic);
     }
     __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
-        const uint32_t zl = zw << 8, zh = zw >> 12;
+        uint32_t zl = zw << 8, zh = zw >> 12;
+        asm("" : "+v"(zl), "+v"(zh));
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             const uint32_t pr = sv[c >> 1];
@@ -79,7 +85,8 @@ struct PipeUnpack<BF16> {
         }
     }
     __device__ __forceinline__ void pair(uint32_t w0, uint32_t w1, uint32_t out[8]) const {
-        const uint32_t l0 = w0 << 8, h0 = w0 >> 12, l1 = w1 << 8, h1 = w1 >> 12;
+        uint32_t l0 = w0 << 8, h0 = w0 >> 12, l1 = w1 << 8, h1 = w1 >> 12;
+        asm("" : "+v"(l0), "+v"(h0), "+v"(l1), "+v"(h1));  // keep the shifts: one per three nibbles
 #pragma unroll
         for (int c = 0; c < 8; ++c)
             out[c] = BF16::pack2(__builtin_fmaf(embed(w0, l0, h0, c), sc[c], off[c]),
@@ -87,26 +94,32 @@ struct PipeUnpack<BF16> {
     }
 };
 
+template <int UR>
 struct Raw {
-    uint32_t w[8];
+    uint32_t w[UR];
     uint32_t z;
     u32x4 s;
 };
 
-template <typename T>
-__global__ __launch_bounds__(256) void gemm_pipe_kernel(
+template <typename T, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
     const uint32_t* __restrict__ qzeros, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
     float* __restrict__ partials, int* __restrict__ counters, int M, int N, int K, int g, int iters_per_split,
     int splits) {
-    constexpr int BM = 256, BN = 256, TM = 4, TN = 4, NT = 256;
+    constexpr int BM = 256, BN = 256, NW = WM * WN, NT = 64 * NW;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int UR = kPBK * 32 / NT;   // k rows of one word column per lane and step: 8 or 4
+    constexpr int NP = UR / 2;           // row pairs per lane and step
+    constexpr int NDMA = 32 / NW;        // direct-to-LDS loads per wave and step
+    static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts");
     constexpr int A_SLOTS = 8 * BM, B_SLOTS = 8 * BN, BUF = A_SLOTS + B_SLOTS;
     extern __shared__ u32x4 lds[];  // [2][BUF]
     __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+    const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int split = blockIdx.z;
     const int words = N >> 3;
@@ -114,40 +127,60 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(
     const int it_begin = split * iters_per_split;
     const int it_end = min(it_begin + iters_per_split, total_iters);
 
-    // ---- A: 8 direct-to-LDS loads per wave and step; load i of wave w fills slots (8w+i)*64 + lane,
-    //      i.e. rows 8*(8w+i) + lane/8, whose chunk at position lane%8 is kc = lane%8 ^ swz(row).
-    //      Rows past M read the last row; their results are never stored.
-    const uint16_t* a_src[8];
+    // ---- A: NDMA direct-to-LDS loads per wave and step; load i of wave w fills slots
+    //      (NDMA*w + i)*64 + lane, i.e. rows 8*(NDMA*w + i) + lane/8, whose chunk at position lane%8
+    //      is kc = lane%8 ^ swz(row).  Rows past M read the last row; their results are never
+    //      stored.  Addresses are a wave-uniform base plus a 32-bit byte offset per lane.
+    const char* a_base = reinterpret_cast<const char*>(x + (size_t)m0 * K);
+    uint32_t a_off[NDMA];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int row = (wave * 8 + i) * 8 + (lane >> 3);
+    for (int i = 0; i < NDMA; ++i) {
+        const int row = (wave * NDMA + i) * 8 + (lane >> 3);
         const int kc = (lane & 7) ^ row_swz(row);
-        a_src[i] = x + (size_t)min(m0 + row, M - 1) * K + kc * 8;
+        a_off[i] = ((uint32_t)min(row, M - 1 - m0) * (uint32_t)K + (uint32_t)kc * 8u) * 2u;
     }
     auto dma_a = [&](int it, int buf) {
+        const char* base = a_base + (size_t)it * (kPBK * 2);  // uniform
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            __builtin_amdgcn_global_load_lds(AWQ_GPTR(a_src[i] + it * kPBK),
-                                             AWQ_LPTR(lds + buf * BUF + (wave * 8 + i) * 64), 16, 0, 0);
+        for (int i = 0; i < NDMA; ++i)
+            __builtin_amdgcn_global_load_lds(AWQ_GPTR(base + a_off[i]),
+                                             AWQ_LPTR(lds + buf * BUF + (wave * NDMA + i) * 64), 16, 0, 0);
     };
 
-    // ---- B: a lane owns word column wc for the 8 k rows of block rb ---------------------------------
+    // ---- B: a lane owns word column wc for the UR k rows of row block rb ----------------------------
     const int wc = tid & 31, rb = tid >> 5;
     const int gwc = min((n0 >> 3) + wc, words - 1);
-    const uint32_t w_off = (uint32_t)(rb * 8) * (uint32_t)words + (uint32_t)gwc;
-    const int g_lane = (rb * 8) / g;  // host guarantees g % 64 == 0 or 64 % g == 0
-    auto load_raw = [&](int it, Raw& r) {
+    const uint32_t w_off = ((uint32_t)(rb * UR) * (uint32_t)words + (uint32_t)gwc) * 4u;  // bytes
+    const int g_lane = (rb * UR) / g;  // host guarantees g % 64 == 0 or 64 % g == 0
+    const uint32_t z_off = ((uint32_t)g_lane * (uint32_t)words + (uint32_t)gwc) * 4u;   // bytes into qzeros
+    const uint32_t s_off = z_off * 4u;                                                    // bytes into scales
+    auto load_raw = [&](int it, Raw<UR>& r) {
         const int k0 = it * kPBK;
-        const uint32_t* wp = qweight + (size_t)k0 * words;  // uniform
+        const char* wp = reinterpret_cast<const char*>(qweight + (size_t)k0 * words);  // uniform
 #pragma unroll
-        for (int i = 0; i < 8; ++i) r.w[i] = (wp + (size_t)i * words)[w_off];
-        const int gi = k0 / g + g_lane;
-        r.z = qzeros[(size_t)gi * words + gwc];
-        r.s = *reinterpret_cast<const u32x4*>(scales + ((size_t)gi * words + gwc) * 8);
+        for (int i = 0; i < UR; ++i)
+            r.w[i] = *reinterpret_cast<const uint32_t*>(wp + (size_t)i * words * 4 + w_off);
+        const size_t grow = (size_t)(k0 / g) * words;  // uniform
+        r.z = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(qzeros + grow) + z_off);
+        r.s = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(scales + grow * 8) + s_off);
     };
+    // a lane's UR rows are the part `sub` of k-block `kblk`: it writes 2*UR bytes of each 16-byte slot
+    constexpr int PER_BLK = 8 / UR;
+    const int kblk = rb / PER_BLK, sub = rb % PER_BLK;
     int b_wr[8];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) b_wr[c] = b_slot_p(wc, c, rb);
+    for (int c = 0; c < 8; ++c) b_wr[c] = b_slot_p(wc, c, kblk) * PER_BLK + sub;
+    auto store_b = [&](int buf, const uint32_t (&cols)[8][NP]) {
+        u32x4* wbase = lds + buf * BUF + A_SLOTS;
+        if constexpr (UR == 8) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) wbase[b_wr[c]] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
+        } else {
+            u32x2* w2 = reinterpret_cast<u32x2*>(wbase);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) w2[b_wr[c]] = u32x2{cols[c][0], cols[c][1]};
+        }
+    };
 
     // ---- MFMA operand addresses ------------------------------------------------------------------
     const int li = lane & 31, kb2 = lane >> 5;
@@ -174,12 +207,12 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(
 
     // one K step: MFMAs of tile `it` (LDS buffer `buf`) interleaved with the unpack of tile it+1 (`cur`,
     // stored to the other buffer), while the packed words of tile it+2 travel to `nxt`
-    auto step = [&](int it, int buf, Raw& cur, Raw& nxt) {
+    auto step = [&](int it, int buf, Raw<UR>& cur, Raw<UR>& nxt) {
         load_raw(min(it + 2, it_end - 1), nxt);
         const u32x4* abase = lds + buf * BUF;
         const u32x4* bbase = abase + A_SLOTS;
         up.set_group(cur.z, cur.s);
-        uint32_t cols[8][4];
+        uint32_t cols[8][NP];
         u32x4 af[2][TM], bf[2][TN];
 #pragma unroll
         for (int a = 0; a < TM; ++a) af[0][a] = abase[a_rd[0] + a * 256];
@@ -194,28 +227,29 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(
 #pragma unroll
                 for (int b = 0; b < TN; ++b) bf[p ^ 1][b] = bbase[b_rd[b] + (ks + 1) * 512];
             }
-            uint32_t o[8];
-            up.pair(cur.w[2 * ks], cur.w[2 * ks + 1], o);
+            if (ks % (4 / NP) == 0) {   // one pair of rows per k-step (8 rows) or per two (4 rows)
+                constexpr int STRIDE = 4 / NP;
+                uint32_t o[8];
+                up.pair(cur.w[2 * (ks / STRIDE)], cur.w[2 * (ks / STRIDE) + 1], o);
 #pragma unroll
-            for (int c = 0; c < 8; ++c) cols[c][ks] = o[c];
+                for (int c = 0; c < 8; ++c) cols[c][ks / STRIDE] = o[c];
+            }
 #pragma unroll
             for (int a = 0; a < TM; ++a)
 #pragma unroll
                 for (int b = 0; b < TN; ++b) acc[a][b] = T::mfma32(af[p][a], bf[p][b], acc[a][b]);
         }
-        u32x4* wbase = lds + (buf ^ 1) * BUF + A_SLOTS;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) wbase[b_wr[c]] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
-        // pinned order: first the operands of k-step 0, then per MFMA a slice of the unpack, with the
-        // operand reads of the next k-step spread over the first half of each k-step
-        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // 8 LDS reads
+        store_b(buf ^ 1, cols);
+        // pinned order: the operands of k-step 0, then per MFMA a slice of the unpack, with the operand
+        // reads of the next k-step spread over the first MFMAs of each k-step
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int m = 0; m < 16; ++m) {
+            for (int m = 0; m < TM * TN; ++m) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
                 __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // 4 vector ALU
-                if (ks < 3 && m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if (ks < 3 && m < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
             }
         __builtin_amdgcn_sched_group_barrier(0x200, 8, 0);  // 8 LDS writes
         asm volatile("" ::: "memory");
@@ -226,23 +260,21 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(
     };
 
     if (it_begin < it_end) {
-        Raw r0, r1;
+        Raw<UR> r0, r1;
         dma_a(it_begin, 0);
         load_raw(it_begin, r0);
         load_raw(min(it_begin + 1, it_end - 1), r1);
         {
             up.set_group(r0.z, r0.s);
-            u32x4* wbase = lds + A_SLOTS;
-            uint32_t cols[8][4];
+            uint32_t cols[8][NP];
 #pragma unroll
-            for (int rp = 0; rp < 4; ++rp) {
+            for (int rp = 0; rp < NP; ++rp) {
                 uint32_t o[8];
                 up.pair(r0.w[2 * rp], r0.w[2 * rp + 1], o);
 #pragma unroll
                 for (int c = 0; c < 8; ++c) cols[c][rp] = o[c];
             }
-#pragma unroll
-            for (int c = 0; c < 8; ++c) wbase[b_wr[c]] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
+            store_b(0, cols);
         }
         if (it_begin + 1 < it_end) dma_a(it_begin + 1, 1);
         asm volatile("" ::: "memory");
@@ -254,15 +286,46 @@ __global__ __launch_bounds__(256) void gemm_pipe_kernel(
             if (it + 1 < it_end) step(it + 1, 1, r0, r1);
         }
     }
-    gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, counters, &s_last, M, N, m0, n0, wm0, wn0, split,
-                                         splits);
+    if (splits == 1) {
+        // Direct store through LDS: the MFMA layout gives a lane one column of a 32 x 32 tile, i.e.
+        // 2-byte stores; staged per wave as [32 rows][32*TN columns] the same data leaves as 16-byte
+        // stores, 4*TN lanes to a row segment.  The staging area is private to the wave and LDS
+        // operations of a wave execute in order, so no barrier is needed (the main loop ended with
+        // one, and no direct-to-LDS load is in flight).
+        constexpr int COLS = 32 * TN, PITCH = COLS + 8;  // halves per staged row, padded (bank spread)
+        constexpr int LPR = COLS / 8, RPP = 64 / LPR;    // lanes per row, rows per pass
+        uint16_t* stage = reinterpret_cast<uint16_t*>(lds) + wave * (32 * PITCH);
+        float bv[TN];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) {
+            const int n = n0 + wn0 + b * 32 + li;
+            bv[b] = (bias && n < N) ? T::to_f32(bias[n]) : 0.f;
+        }
+#pragma unroll
+        for (int a = 0; a < TM; ++a) {
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    stage[((v >> 2) * 8 + kb2 * 4 + (v & 3)) * PITCH + b * 32 + li] = T::from_f32(acc[a][b][v] + bv[b]);
+#pragma unroll
+            for (int j = 0; j < 32 / RPP; ++j) {
+                const int row = RPP * j + lane / LPR, chunk = lane % LPR;
+                const u32x4 val = *reinterpret_cast<const u32x4*>(stage + row * PITCH + chunk * 8);
+                const int m = m0 + wm0 + a * 32 + row, n = n0 + wn0 + chunk * 8;
+                if (m < M && n < N) *reinterpret_cast<u32x4*>(y + (size_t)m * N + n) = val;
+            }
+        }
+    } else {
+        gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, counters, &s_last, M, N, m0, n0, wm0, wn0,
+                                             split, splits);
+    }
 }
 
-}  // namespace
-
-hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
-                            const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
-                            void* workspace, int split_k, hipStream_t stream) {
+template <typename T, int WM, int WN>
+hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                       const void* bias, void* y, int M, int N, int K, int g, void* workspace, int split_k,
+                       hipStream_t stream) {
     const int tiles_m = (int)cdiv(M, 256), tiles_n = (int)cdiv(N, 256);
     const int total_iters = K / kPBK;
     const int ips = (int)cdiv(total_iters, split_k);
@@ -271,25 +334,35 @@ hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, co
     float* partials =
         workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes) : nullptr;
     const size_t lds = (size_t)2 * (8 * 256 + 8 * 256) * 16;  // 128 KiB
-    const void* kern = dtype == AWQ_F16 ? reinterpret_cast<const void*>(gemm_pipe_kernel<F16>)
-                                        : reinterpret_cast<const void*>(gemm_pipe_kernel<BF16>);
-    static bool raised[2] = {false, false};
-    if (!raised[dtype]) {
-        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    auto kern = gemm_pipe_kernel<T, WM, WN>;
+    static bool raised = false;  // once per process and instantiation
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        raised[dtype] = true;
+        raised = true;
     }
     (void)hipGetLastError();
-    auto go = [&](auto k) {
-        hipLaunchKernelGGL(k, dim3(tiles_n, tiles_m, splits), dim3(256), lds, stream,
-                           reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
-                           reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
-                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials,
-                           counters, M, N, K, g, ips, splits);
-    };
-    if (dtype == AWQ_F16) go(gemm_pipe_kernel<F16>);
-    else go(gemm_pipe_kernel<BF16>);
+    hipLaunchKernelGGL(kern, dim3(tiles_n, tiles_m, splits), dim3(64 * WM * WN), lds, stream,
+                       reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
+                       reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
+                       M, N, K, g, ips, splits);
     return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_gemm_pipe(int dtype, int waves, const void* x, const int32_t* qweight, const void* qscales,
+                            const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
+                            void* workspace, int split_k, hipStream_t stream) {
+    if (waves == 8)
+        return dtype == AWQ_F16
+                   ? launch_pipe<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
+                   : launch_pipe<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
+    return dtype == AWQ_F16
+               ? launch_pipe<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
+               : launch_pipe<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
 }
 
 }  // namespace awq
