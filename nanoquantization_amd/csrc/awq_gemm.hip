@@ -20,8 +20,8 @@
 // q*s - z*s whose exact result needs no more than fp32's significand, then
 // packs two rows with a single round-to-nearest-even conversion.
 //
-// Split-K: as in the GEMV, fp32 partials + an arrival counter per tile; the
-// last workgroup adds the partials in split order.
+// Split-K: every split stores fp32 partials with plain stores; a second kernel
+// adds them in split order (bit-stable) and applies the bias.
 #include "awq_common.hpp"
 #include "awq_gemm_parts.hpp"
 
@@ -44,7 +44,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
-    int* __restrict__ counters, int M, int N, int K, int g, int iters_per_split, int splits) {
+    int M, int N, int K, int g, int iters_per_split, int splits) {
     constexpr int NW = WM * WN, NT = 64 * NW;
     static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts per workgroup");
     static_assert(BN == 256 || BN == 128, "BN is 128 or 256");
@@ -58,7 +58,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
     constexpr int A_SLOTS = 8 * BM, B_SLOTS = 8 * BN;
 
     extern __shared__ u32x4 lds[];  // [2][A_SLOTS + B_SLOTS]
-    __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -194,7 +193,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(
         }
     }
 
-    gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, counters, &s_last, M, N, m0, n0, wm0, wn0, split, splits);
+    gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, M, N, m0, n0, wm0, wn0, split, splits);
 }
 
 // ---- host side -------------------------------------------------------------
@@ -220,7 +219,6 @@ static hipError_t launch_gemm(const void* x, const int32_t* qweight, const void*
     const int total_iters = K / kBK;
     const int ips = (int)cdiv(total_iters, split_k);
     const int splits = (int)cdiv(total_iters, ips);
-    int* counters = reinterpret_cast<int*>(workspace);
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
                                                             kCounterBytes)
                                 : nullptr;
@@ -242,8 +240,10 @@ static hipError_t launch_gemm(const void* x, const int32_t* qweight, const void*
                        reinterpret_cast<const uint16_t*>(qscales),
                        reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
-                       partials, counters, M, N, K, g, ips, splits);
-    return hipGetLastError();
+                       partials, M, N, K, g, ips, splits);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || splits == 1) return e;
+    return launch_splitk_reduce(T::id, partials, bias, y, M, N, splits, stream);
 }
 
 static int gemm_effective_splits(int64_t K, int split_k) {
@@ -259,21 +259,23 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
     return kCounterBytes + (size_t)splits * M * N * sizeof(float);
 }
 
-// Tile shape and split for the default entry point: the largest tile that still
-// yields at least one workgroup per CU, then split K until the chip is covered.
+// Tile shape and split for the default entry point.  Large M: the pipelined 256 x 256 kernel with two
+// wavefronts per SIMD, K split so that the tiles cover the CUs once (a split costs one more pass over
+// the fp32 partials, which is cheap next to an idle CU).  Small M: narrower tiles of the plain kernel.
 static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     const int kCUs = 256;
     // indices into kGemmVariants
-    constexpr int k256x256 = kPipeVariant, k128x128 = 2, k64x256 = 3, k32x256 = 4;
+    constexpr int kPipe8 = kPipeVariant + 1, k128x128 = 2, k64x256 = 3, k32x256 = 4;
     int v;
     if (M <= 32) v = k32x256;
     else if (M <= 64) v = k64x256;
-    else v = (cdiv(M, 256) * cdiv(N, 256) >= 2 * kCUs) ? k256x256 : k128x128;
+    else if (M <= 128) v = k128x128;
+    else v = kPipe8;
     const GemmVariant& gv = kGemmVariants[v];
     const int64_t tiles = cdiv(M, gv.BM) * cdiv(N, gv.BN);
     int64_t s = 1;
     if (tiles < kCUs) s = kCUs / tiles;
-    const int64_t max_s = K / kBK / 4 > 0 ? K / kBK / 4 : 1;  // at least 4 K-steps per split
+    const int64_t max_s = K / kBK / 8 > 0 ? K / kBK / 8 : 1;  // at least 8 K-steps per split
     if (s > max_s) s = max_s;
     if (s > 16) s = 16;
     if (s < 1) s = 1;
@@ -303,11 +305,6 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     const GemmVariant& gv = kGemmVariants[variant];
     if (cdiv(M, gv.BM) > 65535) {
         set_error("%s: M=%lld exceeds the launch grid for tile %s", fn, (long long)M, gv.name);
-        return AWQ_ERR_UNSUPPORTED;
-    }
-    if (gemm_effective_splits(K, split_k) > 1 && cdiv(M, gv.BM) * cdiv(N, gv.BN) > kMaxSplitTiles) {
-        set_error("%s: split-K supports at most %lld output tiles (M=%lld N=%lld tile %s)", fn,
-                  (long long)kMaxSplitTiles, (long long)M, (long long)N, gv.name);
         return AWQ_ERR_UNSUPPORTED;
     }
     const size_t need = gemm_ws_bytes(M, N, K, variant, split_k);

@@ -1,7 +1,6 @@
 // Pieces shared by the fused dequant+GEMM kernels: the register unpack of packed words into
 // k-pairs of dequantised values, and the epilogue: direct store (+ bias) of a workgroup's
-// BM x BN tile, or the split-K exchange (fp32 partials, arrival counter, in-order sum by the
-// last workgroup to arrive).
+// BM x BN tile, or fp32 partials of a K split that a second kernel adds in split order.
 #pragma once
 
 #include "awq_common.hpp"
@@ -68,13 +67,10 @@ struct UnpackRows<BF16> {
 // (a, b) of the wave's sub-tile at (wm0, wn0).
 template <typename T, int BM, int BN, int TM, int TN, int NT>
 __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const uint16_t* __restrict__ bias,
-                                              uint16_t* __restrict__ y, float* __restrict__ partials,
-                                              int* __restrict__ counters, int* s_last_p, int M, int N, int m0,
-                                              int n0, int wm0, int wn0, int split, int splits) {
-    constexpr int WCOLS = BN / 8;
-    const int tid = threadIdx.x, lane = tid & 63;
+                                              uint16_t* __restrict__ y, float* __restrict__ partials, int M,
+                                              int N, int m0, int n0, int wm0, int wn0, int split, int splits) {
+    const int lane = threadIdx.x & 63;
     const int li = lane & 31, kb2 = lane >> 5;
-    const int words = N >> 3;
     const bool direct = splits == 1;
 #pragma unroll
     for (int a = 0; a < TM; ++a)
@@ -91,47 +87,55 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const uint1
                 if (direct)
                     y[(size_t)m * N + n] = T::from_f32(acc[a][b][v] + bv);
                 else
-                    publish_f32(&partials[((size_t)split * M + m) * N + n], acc[a][b][v]);
+                    partials[((size_t)split * M + m) * N + n] = acc[a][b][v];   // 32 lanes = one 128-byte line
             }
         }
-    if (direct) return;
+}
 
-    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
-    if (!arrive_last(&counters[tile], splits, s_last_p)) return;
-    const int rows = min(BM, M - m0);
-    const int wcount = min(WCOLS, words - (n0 >> 3));
-    for (int idx = tid; idx < rows * wcount; idx += NT) {
-        const int m = m0 + idx / wcount;
-        const size_t nn = (size_t)n0 + (size_t)(idx % wcount) * 8;
-        float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int s0 = 0; s0 < splits; s0 += 8) {   // 8 splits in flight, added in split order
-            float v[8][8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int s = min(s0 + u, splits - 1);
-                const float* p = partials + ((size_t)s * M + m) * N + nn;
-#pragma unroll
-                for (int c = 0; c < 8; ++c) v[u][c] = fetch_f32(p + c);
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (s0 + u < splits) {
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) out[c] += v[u][c];
-                }
-        }
-        if (bias) {
-            const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-                out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
-        }
-        u32x4 o;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
-        *reinterpret_cast<u32x4*>(y + (size_t)m * N + nn) = o;
+// Second pass of a split-K product: y = dtype(sum over splits, in split order, of the fp32
+// partials [splits][M][N] (+ bias)).  A thread owns 8 consecutive columns of one row.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ partials,
+                                                                 const uint16_t* __restrict__ bias,
+                                                                 uint16_t* __restrict__ y, int64_t M, int N,
+                                                                 int splits) {
+    const int64_t vec = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int per_row = N >> 3;
+    if (vec >= M * per_row) return;
+    const int64_t m = vec / per_row;
+    const int nn = (int)(vec % per_row) * 8;
+    const size_t plane = (size_t)M * N;
+    const float* p = partials + (size_t)m * N + nn;
+    f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+    for (int s = 0; s < splits; ++s) {
+        lo += *reinterpret_cast<const f32x4*>(p + s * plane);
+        hi += *reinterpret_cast<const f32x4*>(p + s * plane + 4);
     }
-    if (tid == 0) __hip_atomic_store(&counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float out[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (bias) {
+        const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
+    }
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+    *reinterpret_cast<u32x4*>(y + (size_t)m * N + nn) = o;
+}
+
+// Launches the reduction pass on `stream` (after the product kernel that wrote `partials`).
+inline hipError_t launch_splitk_reduce(int dtype, const float* partials, const void* bias, void* y, int64_t M, int N,
+                                       int splits, hipStream_t stream) {
+    const int64_t vecs = M * (N >> 3);
+    const dim3 grid((unsigned)cdiv(vecs, 256)), block(256);
+    if (dtype == AWQ_F16)
+        gemm_splitk_reduce_kernel<F16><<<grid, block, 0, stream>>>(partials, reinterpret_cast<const uint16_t*>(bias),
+                                                                   reinterpret_cast<uint16_t*>(y), M, N, splits);
+    else
+        gemm_splitk_reduce_kernel<BF16><<<grid, block, 0, stream>>>(partials, reinterpret_cast<const uint16_t*>(bias),
+                                                                    reinterpret_cast<uint16_t*>(y), M, N, splits);
+    return hipGetLastError();
 }
 
 // awq_gemm_pipe.hip: the 256 x 256 software-pipelined kernel with 4 or 8 wavefronts (same

@@ -101,11 +101,11 @@ struct Raw {
     u32x4 s;
 };
 
-template <typename T, int WM, int WN>
+template <typename T, int WM, int WN, bool PIN = true>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
     const uint32_t* __restrict__ qzeros, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
-    float* __restrict__ partials, int* __restrict__ counters, int M, int N, int K, int g, int iters_per_split,
+    float* __restrict__ partials, int M, int N, int K, int g, int iters_per_split,
     int splits) {
     constexpr int BM = 256, BN = 256, NW = WM * WN, NT = 64 * NW;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -115,7 +115,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts");
     constexpr int A_SLOTS = 8 * BM, B_SLOTS = 8 * BN, BUF = A_SLOTS + B_SLOTS;
     extern __shared__ u32x4 lds[];  // [2][BUF]
-    __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -240,8 +239,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
                 for (int b = 0; b < TN; ++b) acc[a][b] = T::mfma32(af[p][a], bf[p][b], acc[a][b]);
         }
         store_b(buf ^ 1, cols);
-        // pinned order: the operands of k-step 0, then per MFMA a slice of the unpack, with the operand
-        // reads of the next k-step spread over the first MFMAs of each k-step
+        // With one wavefront per SIMD the order is pinned: the operands of k-step 0, then per MFMA a
+        // slice of the unpack, with the operand reads of the next k-step spread over the first MFMAs
+        // of each k-step.  With two per SIMD the hardware interleaves them and pinning only costs.
+        if constexpr (PIN) {
         __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
@@ -252,6 +253,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
                 if (ks < 3 && m < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
             }
         __builtin_amdgcn_sched_group_barrier(0x200, 8, 0);  // 8 LDS writes
+        }
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the A tile of step it+1 has landed
         asm volatile("" ::: "memory");
@@ -317,12 +319,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
             }
         }
     } else {
-        gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, counters, &s_last, M, N, m0, n0, wm0, wn0,
-                                             split, splits);
+        gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, M, N, m0, n0, wm0, wn0, split, splits);
     }
 }
 
-template <typename T, int WM, int WN>
+template <typename T, int WM, int WN, bool PIN = true>
 hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
                        const void* bias, void* y, int M, int N, int K, int g, void* workspace, int split_k,
                        hipStream_t stream) {
@@ -330,11 +331,10 @@ hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscale
     const int total_iters = K / kPBK;
     const int ips = (int)cdiv(total_iters, split_k);
     const int splits = (int)cdiv(total_iters, ips);
-    int* counters = reinterpret_cast<int*>(workspace);
     float* partials =
         workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes) : nullptr;
     const size_t lds = (size_t)2 * (8 * 256 + 8 * 256) * 16;  // 128 KiB
-    auto kern = gemm_pipe_kernel<T, WM, WN>;
+    auto kern = gemm_pipe_kernel<T, WM, WN, PIN>;
     static bool raised = false;  // once per process and instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -346,9 +346,11 @@ hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscale
     hipLaunchKernelGGL(kern, dim3(tiles_n, tiles_m, splits), dim3(64 * WM * WN), lds, stream,
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
-                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
-                       M, N, K, g, ips, splits);
-    return hipGetLastError();
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, M, N, K, g, ips,
+                       splits);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || splits == 1) return e;
+    return launch_splitk_reduce(T::id, partials, bias, y, M, N, splits, stream);
 }
 
 }  // namespace
@@ -358,8 +360,8 @@ hipError_t launch_gemm_pipe(int dtype, int waves, const void* x, const int32_t* 
                             void* workspace, int split_k, hipStream_t stream) {
     if (waves == 8)
         return dtype == AWQ_F16
-                   ? launch_pipe<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
-                   : launch_pipe<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
+                   ? launch_pipe<F16, 2, 4, false>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
+                   : launch_pipe<BF16, 2, 4, false>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
     return dtype == AWQ_F16
                ? launch_pipe<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
                : launch_pipe<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
