@@ -97,6 +97,20 @@ __device__ __forceinline__ void publish_f32x4(float* p, f32x4 v) {
 __device__ __forceinline__ float fetch_f32(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// 16-byte form of fetch_f32 that does not wait: the load is invisible to the compiler's wait-count
+// bookkeeping, so the values may only be used after fetch_wait() has been given every one of them.
+__device__ __forceinline__ f32x4 fetch_f32x4_nowait(const float* p) {
+    f32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void fetch_wait(f32x4 (&a)[8], f32x4 (&b)[8]) {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
+                   "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(b[4]), "+v"(b[5]), "+v"(b[6]), "+v"(b[7])
+                 :
+                 : "memory");
+}
 // All of this workgroup's publish_f32 stores have been acknowledged (vmcnt = 0
 // in every wave, then the barrier) before one thread bumps the tile's arrival
 // counter; returns true in the workgroup that arrived last.

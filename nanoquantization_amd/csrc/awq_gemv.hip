@@ -256,21 +256,25 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
         const int m = idx / w_count, wc = idx - m * w_count;
         const size_t n0 = (size_t)(w_begin + wc) * 8;
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        // fetch 8 splits at a time so that their loads overlap; add in split order
+        // fetch 8 splits at a time (two 16-byte loads each) so that their loads overlap; add in split order
         for (int s0 = 0; s0 < splits; s0 += 8) {
-            float v[8][8];
+            f32x4 lo[8], hi[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const int s = min(s0 + u, splits - 1);
                 const float* p = partials + ((size_t)s * M + m) * N + n0;
-#pragma unroll
-                for (int c = 0; c < 8; ++c) v[u][c] = fetch_f32(p + c);
+                lo[u] = fetch_f32x4_nowait(p);
+                hi[u] = fetch_f32x4_nowait(p + 4);
             }
+            fetch_wait(lo, hi);
 #pragma unroll
             for (int u = 0; u < 8; ++u)
                 if (s0 + u < splits) {
 #pragma unroll
-                    for (int c = 0; c < 8; ++c) out[c] += v[u][c];
+                    for (int c = 0; c < 4; ++c) {
+                        out[c] += lo[u][c];
+                        out[4 + c] += hi[u][c];
+                    }
                 }
         }
         if (bias) {
@@ -677,14 +681,20 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
     if (N % 128 == 0 && g % 128 == 0) {
         // From sweeps on MI355X (HBM-streaming): short K runs best as one workgroup of 8 waves per
         // column tile; otherwise 4-wave workgroups, split over K for M <= 4 until ~3000 waves exist
-        // (the split's serial tail grows with M, so larger M splits only to cover the CUs).
+        // (the split's tail grows with M, so larger M splits only to cover the CUs).
         const int64_t tiles = N / 128;
         int v = 10 /* dma1x4d1 */;
         int64_t s = 1;
-        if (M > 32) {
-            v = 22 /* dma1x4d1m4 */;   // 17..64 rows: never split K, the tail grows with M
-        } else if (M > 16) {
-            v = chunks >= 8 ? 21 /* dma1x8d1m2 */ : 20 /* dma1x4d1m2 */;
+        if (M > 16) {
+            // 17..64 rows: with 32 column tiles or more one 8-wave workgroup per tile covers the chip
+            // well enough; with fewer, split K until some 48 workgroups exist (4 chunks per split at least)
+            if (M <= 32 && tiles >= 32 && chunks >= 8) {
+                v = 21 /* dma1x8d1m2 */;
+            } else {
+                v = M > 32 ? 22 /* dma1x4d1m4 */ : 20 /* dma1x4d1m2 */;
+                if (tiles < 48) s = cdiv(48, tiles);
+                if (s > chunks / 4) s = chunks / 4;
+            }
         } else if (chunks <= 8) {
             v = 11 /* dma1x8d1 */;
         } else if (M <= 4) {
