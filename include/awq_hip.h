@@ -48,6 +48,17 @@ const char* awq_hip_last_error(void);
 int awq_dequantize(const int32_t* qweight, const void* qscales, const int32_t* qzeros, void* out,
                    int64_t K, int64_t N, int64_t group_size, int dtype, void* stream);
 
+/* Offline path: weight f32 [N, K] (the nn.Linear layout) -> packed AWQ buffers in one pass:
+ * per group of `group_size` input features s = max(max - min, 1e-5) / 15,
+ * z = clamp(-round(min / s), 0, 15), q = clamp(round(w / s) + z, 0, 15); qweight [K, N/8] and
+ * qzeros [K/g, N/8] hold q and z in the nibble order above, qscales [K/g, N] holds s in `dtype`.
+ * fp32 arithmetic with true divisions and round-half-to-even, word for word what
+ * pseudo_quantize(w, g, 4, zero_point=True) (nanoquantization/utils/quantization.py:5-58), the
+ * transposes of awq/quantizer.py:156-158 and WQLinear_GEMM.from_linear
+ * (nanoquantization/layers/gemm.py:447-550) produce for an fp32 weight.  The weight must hold no NaN. */
+int awq_quantize_pack(const float* weight, int32_t* qweight, void* qscales, int32_t* qzeros,
+                      int64_t N, int64_t K, int64_t group_size, int dtype, void* stream);
+
 /* Bytes of device workspace awq_gemv / awq_gemm / awq_linear need for this
  * problem (0 is possible).  The workspace must be zero-filled ONCE when it is
  * allocated; every call leaves it in that state (its counters are reset by

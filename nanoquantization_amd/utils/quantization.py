@@ -38,3 +38,28 @@ def pseudo_quantize(
         deq = torch.clamp(torch.round(groups / scales), q_lo, q_hi) * scales
         zeros_out = None
     return deq.reshape(shape), scales.reshape(shape[0], -1), zeros_out
+
+
+def quantize_pack(weight: torch.Tensor, group_size: int, output_dtype: torch.dtype = torch.bfloat16):
+    """weight fp32 [N, K] on a HIP device -> (qweight int32 [K, N/8], qscales [K/g, N], qzeros int32
+    [K/g, N/8]) in one kernel: the words that pseudo_quantize(weight, g, 4, True) followed by
+    WQLinear_GEMM.from_linear would produce (utils/quantization.py:5-58, layers/gemm.py:447-550 of the
+    reference), without the [N, K] temporaries."""
+    from .. import _lib
+    if weight.device.type != "cuda":
+        raise _lib.AwqHipError(f"quantize_pack runs on a HIP device only (tensor is on {weight.device})")
+    assert weight.dim() == 2 and weight.dtype == torch.float32, "an fp32 [out_features, in_features] weight"
+    assert not bool(torch.isnan(weight).any()), "weight should not contain nan"
+    weight = weight.contiguous()
+    N, K = weight.shape
+    g = K if group_size <= 0 else group_size
+    assert K % g == 0 and N % 8 == 0
+    dev = weight.device
+    qweight = torch.empty(K, N // 8, dtype=torch.int32, device=dev)
+    qzeros = torch.empty(K // g, N // 8, dtype=torch.int32, device=dev)
+    qscales = torch.empty(K // g, N, dtype=output_dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().awq_quantize_pack(weight.data_ptr(), qweight.data_ptr(), qscales.data_ptr(),
+                                                qzeros.data_ptr(), N, K, g, _lib.dtype_id(output_dtype),
+                                                torch.cuda.current_stream().cuda_stream))
+    return qweight, qscales, qzeros
