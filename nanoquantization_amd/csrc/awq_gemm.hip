@@ -205,8 +205,7 @@ static const GemmVariant kGemmVariants[] = {
     {"256x256w8", 256, 256, 8}, {"128x256w8", 128, 256, 8}, {"128x128", 128, 128, 4},
     {"64x256", 64, 256, 4},     {"32x256", 32, 256, 4},     {"64x128", 64, 128, 4},
     {"256x256", 256, 256, 4},   {"128x256", 128, 256, 4},   {"256x128w8", 256, 128, 8},
-    {"256x256p", 256, 256, 4},  // the software-pipelined kernel of awq_gemm_pipe.hip
-    {"256x256pw8", 256, 256, 8},  // the same with two wavefronts per SIMD
+    {"256x256p", 256, 256, 8},  // the software-pipelined kernel of awq_gemm_pipe.hip
 };
 constexpr int kPipeVariant = 9;
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
@@ -265,7 +264,7 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
 static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     const int kCUs = 256;
     // indices into kGemmVariants
-    constexpr int kPipe8 = kPipeVariant + 1, k128x128 = 2, k64x256 = 3, k32x256 = 4;
+    constexpr int kPipe8 = kPipeVariant, k128x128 = 2, k64x256 = 3, k32x256 = 4;
     int v;
     if (M <= 32) v = k32x256;
     else if (M <= 64) v = k64x256;
@@ -335,8 +334,7 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         AWQ_GEMM_CASE(7, 128, 256, 2, 2)
         AWQ_GEMM_CASE(8, 256, 128, 4, 2)
         case kPipeVariant:
-        case kPipeVariant + 1:
-            e = launch_gemm_pipe(dtype, variant == kPipeVariant ? 4 : 8, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+            e = launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
                                  workspace, split_k, s);
             break;
     }

@@ -138,9 +138,8 @@ inline hipError_t launch_splitk_reduce(int dtype, const float* partials, const v
     return hipGetLastError();
 }
 
-// awq_gemm_pipe.hip: the 256 x 256 software-pipelined kernel with 4 or 8 wavefronts (same
-// arguments as the tiled launcher).
-hipError_t launch_gemm_pipe(int dtype, int waves, const void* x, const int32_t* qweight, const void* qscales,
+// awq_gemm_pipe.hip: the 256 x 256 software-pipelined kernel (same arguments as the tiled launcher).
+hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
                             void* workspace, int split_k, hipStream_t stream);
 

@@ -1,21 +1,19 @@
 // Kernel (c), large-M form: fused dequant + GEMM on the 32x32x16 MFMA with the unpack hidden
 // behind the matrix cores.
 //
-// A workgroup of 4 (2 x 2) or 8 (2 x 4) wavefronts owns a 256 x 256 output tile and walks K in
-// steps of 64.  A SIMD issues one instruction per wavefront every four cycles, and the unpack
-// adds some 240 vector-ALU instructions to the 64 MFMAs of a step: with one wavefront per SIMD
-// the issue slots, not the matrix core, set the pace.  With 8 wavefronts (two per SIMD, 128
-// accumulator registers each) one wavefront's MFMA issues beside the other's unpack and LDS
-// traffic.
+// A workgroup of 8 wavefronts (2 x 4, a 128 x 64 sub-tile and 128 accumulator registers each) owns a
+// 256 x 256 output tile and walks K in steps of 64.  Two wavefronts share a SIMD on purpose: a SIMD
+// issues one instruction per wavefront every four cycles, and the unpack adds some 240 vector-ALU
+// instructions to the 64 MFMAs of a step, so with a single wavefront per SIMD the issue slots, not
+// the matrix core, set the pace (measured: 0.98 vs 1.10 PFLOP/s at M = 8192); with two, one
+// wavefront's MFMAs issue beside the other's unpack and LDS traffic.
+//
 // LDS holds two buffers of { A tile, dequantised B tile }:
 //   A: x[m0.., k0..k0+63] lands straight from global memory (global_load_lds, no registers, no
 //      vector ALU), row-major, the eight 16-byte chunks of a row XOR-swizzled by the row number;
 //   B: packed words go global -> registers one step ahead; while the MFMAs of step i run, the
-//      same wave turns the words of step i+1 into RN_dtype((q - z) * s) -- two k rows at a time,
-//      one pair of rows per quarter of the MFMAs -- and stores them k-contiguous for step i+1.
-// The instruction order of a step is pinned with scheduling-group barriers: one MFMA, a few
-// vector-ALU instructions, an LDS read of the next operands, and so on, so that the matrix core
-// never waits for the unpack.
+//      same wave turns the words of step i+1 into RN_dtype((q - z) * s), two k rows at a time, and
+//      stores them k-contiguous for step i+1.
 //
 // bf16 unpack: a nibble is masked in place at mantissa bit 8, 12 or 16 of the fp32 pattern
 // 0x4B000000 (value 2^23 + q * 2^e), so  fma(f, s * 2^-e, -(2^(23-e) + z) * s) = (q - z) * s
@@ -101,7 +99,7 @@ struct Raw {
     u32x4 s;
 };
 
-template <typename T, int WM, int WN, bool PIN = true>
+template <typename T, int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
     const uint32_t* __restrict__ qzeros, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
@@ -239,21 +237,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
                 for (int b = 0; b < TN; ++b) acc[a][b] = T::mfma32(af[p][a], bf[p][b], acc[a][b]);
         }
         store_b(buf ^ 1, cols);
-        // With one wavefront per SIMD the order is pinned: the operands of k-step 0, then per MFMA a
-        // slice of the unpack, with the operand reads of the next k-step spread over the first MFMAs
-        // of each k-step.  With two per SIMD the hardware interleaves them and pinning only costs.
-        if constexpr (PIN) {
-        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int m = 0; m < TM * TN; ++m) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // 4 vector ALU
-                if (ks < 3 && m < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
-            }
-        __builtin_amdgcn_sched_group_barrier(0x200, 8, 0);  // 8 LDS writes
-        }
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the A tile of step it+1 has landed
         asm volatile("" ::: "memory");
@@ -323,7 +306,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     }
 }
 
-template <typename T, int WM, int WN, bool PIN = true>
+template <typename T, int WM, int WN>
 hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
                        const void* bias, void* y, int M, int N, int K, int g, void* workspace, int split_k,
                        hipStream_t stream) {
@@ -334,7 +317,7 @@ hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscale
     float* partials =
         workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes) : nullptr;
     const size_t lds = (size_t)2 * (8 * 256 + 8 * 256) * 16;  // 128 KiB
-    auto kern = gemm_pipe_kernel<T, WM, WN, PIN>;
+    auto kern = gemm_pipe_kernel<T, WM, WN>;
     static bool raised = false;  // once per process and instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -355,16 +338,12 @@ hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscale
 
 }  // namespace
 
-hipError_t launch_gemm_pipe(int dtype, int waves, const void* x, const int32_t* qweight, const void* qscales,
+hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
                             void* workspace, int split_k, hipStream_t stream) {
-    if (waves == 8)
-        return dtype == AWQ_F16
-                   ? launch_pipe<F16, 2, 4, false>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
-                   : launch_pipe<BF16, 2, 4, false>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
     return dtype == AWQ_F16
-               ? launch_pipe<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
-               : launch_pipe<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
+               ? launch_pipe<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
+               : launch_pipe<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
 }
 
 }  // namespace awq
