@@ -27,6 +27,13 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# HBM bytes per GEMV launch of the headline sweep, from two `rocprofv3 --pmc` runs of this file
+# (FETCH_SIZE, then WRITE_SIZE; profiles/gemv_cfg2_sweep_hbm_traffic.txt).  Each counter is scaled by
+# what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,014 -> 2047 B per count,
+# WRITE_SIZE 64,000 -> 1024 B per count.
+MEASURED_FETCH_BYTES_PER_LAUNCH = 1065.4 * 2047.1
+MEASURED_WRITE_BYTES_PER_LAUNCH = 108.9 * 1024.0
+
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16, published
 QWEN3_0P6B = [("q", 1024, 2048), ("k", 1024, 1024), ("v", 1024, 1024), ("o", 2048, 1024),
@@ -130,9 +137,15 @@ def main():
     avg_launch_us = ms_graph * 1e3 / launches_per_step
     avg_bytes = bytes_per_step / launches_per_step
     roofline = {
-        "kernel": "awq::gemv_dma_kernel<F16,1,4|8>", "bound": "hbm",
+        "kernel": "awq::gemv_dma_kernel<F16, WN=1, WK=4|8, DEPTH=1, MT=1>", "bound": "hbm",
         "achieved": avg_bytes / (avg_launch_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+        "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+        "traffic": MEASURED_FETCH_BYTES_PER_LAUNCH + MEASURED_WRITE_BYTES_PER_LAUNCH,
+        "traffic_note": "HBM bytes per launch (fetch 2.18 MB + write 0.11 MB) from rocprofv3 FETCH_SIZE / WRITE_SIZE, "
+                        "copy-calibrated; above the 1.17 MB of packed weights because a workgroup reads 64-byte row "
+                        "pieces and, with only 8-24 column tiles, the other half of a 128-byte line is often fetched "
+                        "again by another XCD's L2; the writes are split-K partials.  These launches are latency-bound "
+                        "(the variant without the re-fetch is 15-25 % slower); at the 68 MB shapes fetch = 1.05 x algorithmic",
         "avg_launch_us": avg_launch_us, "algorithmic_bytes_per_launch": avg_bytes,
         "note": "packed-weight bytes (0.5195 B/weight) / HIP-event time per launch over the timed graph replays; "
                 "0.5-1.6 MB per launch: latency-bound, see roofline_large for the HBM-bound regime",
@@ -198,7 +211,7 @@ def main():
                                              "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4)}
             del w
         bestp = max(v["TFLOPs"] for v in prefill.values())
-        out["roofline_prefill"] = {"kernel": "awq::gemm_kernel<BF16,...>", "bound": "mfma", "achieved": bestp,
+        out["roofline_prefill"] = {"kernel": "awq::gemm_pipe_kernel<BF16,2,4>", "bound": "mfma", "achieved": bestp,
                                    "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": bestp / MFMA_PEAK_TFLOPS,
                                    "workload": "cfg3: Qwen3-8B MLP shapes, bf16, M in {512,2048,8192}", "cases": prefill}
 

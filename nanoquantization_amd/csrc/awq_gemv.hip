@@ -701,8 +701,8 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             s = cdiv(3072, tiles * 4);
             const int64_t cap = chunks / 2 < 10 ? chunks / 2 : 10;
             if (s > cap) s = cap;
-        } else if (tiles * 4 < 512) {
-            s = cdiv(512, tiles * 4);
+        } else if (tiles < 200) {
+            s = cdiv(200, tiles);   // about 200 workgroups
             if (s > chunks / 4) s = chunks / 4;
         }
         if (s < 1) s = 1;
