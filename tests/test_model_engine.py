@@ -146,3 +146,33 @@ def test_model_forward_matches_dequantised_torch_model():
     h_ref = ref(ids, pos).float()
     err = (h - h_ref).abs().max().item() / h_ref.abs().max().item()
     assert err <= 3e-2, err
+
+
+@pytest.mark.gpu
+def test_engine_at_qwen3_32b_widths():
+    """Two blocks of the Qwen3-32B architecture at its real widths (hidden 5120, 64 q / 8 kv heads,
+    intermediate 25600, vocabulary 151936): batch-64 decode shapes (idle rows included), 8 query heads per kv
+    head in the paged attention, the pipelined GEMM in the recompute.  Same check as the small model: the
+    engine's own continuation, teacher-forced through the full-recompute forward, must be that forward's
+    argmax wherever the logits are not near-tied."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+    print("engine at Qwen3-32B widths, 2 layers", flush=True)
+    cfg = dict(QWEN3_32B, num_hidden_layers=2, max_position_embeddings=512)
+    model = random_awq_qwen3(cfg, seed=5, std=0.02)
+    torch.manual_seed(6)
+    plen, new = 37, 6
+    prompts = torch.randint(0, cfg["vocab_size"], (3, plen)).tolist()
+    eng = LLMEngine(model, max_batch=64, max_seq_len=128, block_size=64, use_graph=True)
+    got = eng.generate(prompts, new)
+    seqs = torch.tensor([p + g for p, g in zip(prompts, got)], device="cuda")
+    pos = torch.arange(seqs.shape[1], device="cuda").unsqueeze(0)
+    logits = model.lm_head(model(seqs, pos)).float()[:, plen - 1:-1]
+    chosen = torch.tensor(got, device="cuda")
+    gap = logits.max(-1).values - logits.gather(-1, chosen.unsqueeze(-1)).squeeze(-1)
+    scale = logits.abs().max().item()
+    assert gap.max().item() <= 2e-2 * scale, (gap.max().item(), scale)
+    top2 = logits.topk(2, dim=-1).values
+    clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
+    assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
+    assert eng.generate(prompts, new) == got
