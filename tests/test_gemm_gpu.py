@@ -96,3 +96,29 @@ def test_gemm_prefill_full_size_bf16():
     xb = make_x(M, K, "bf16", seed=91)
     y = nq.awq_gemm(to_dev(xb, "bf16"), to_dev(p["qweight"]), to_dev(p["qscales"], "bf16"), to_dev(p["qzeros"]), 8)
     _check(y, xb, p, "bf16")
+
+
+@pytest.mark.parametrize("M,K,N", [(8192, 4096, 12288), (8192, 12288, 4096), (4096, 8192, 5120), (300, 5120, 25600)])
+def test_gemm_largest_shapes_properties(M, K, N):
+    """The largest prefill shapes (Qwen3-8B MLP at M = 8192, Qwen3-32B o_proj at a 4096-token prefill and gate/up
+    at a ragged M), too big for the CPU oracle: checked through size-independent properties.  (1) rows sampled
+    across every workgroup tile equal the same rows pushed through the kernel alone (a row's result does not
+    depend on M or on its tile) -- and those small calls are checked against the fp32 matmul of the dequantised,
+    bit-exact weight; (2) the kernel is run-to-run bit-stable; (3) zero rows give exact zeros."""
+    print(f"gemm properties M={M} K={K} N={N} bf16", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(M + K)
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    sc = (torch.rand(K // 128, N, device="cuda", generator=g) * 0.01 + 0.002).to(torch.bfloat16)
+    x = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    x[5] = 0
+    y = nq.awq_gemm(x, qw, sc, qz, 8)
+    assert torch.equal(y, nq.awq_gemm(x, qw, sc, qz, 8))
+    assert torch.count_nonzero(y[5]) == 0
+    rows = torch.arange(3, M, max(1, M // 61), device="cuda")[:64]          # one or two rows of every 256-row tile
+    w = nq.awq_dequantize(qw, sc, qz).float()
+    ref = x[rows].float() @ w
+    err = ((y[rows].float() - ref).abs().max() / ref.abs().max()).item()
+    assert err <= TIGHT["bf16"], err
+    sub = nq.awq_gemm(x[rows].contiguous(), qw, sc, qz, 8).float()          # another kernel / tile shape
+    assert ((sub - ref).abs().max() / ref.abs().max()).item() <= TIGHT["bf16"]
