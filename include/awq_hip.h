@@ -78,6 +78,16 @@ int awq_gemv(const void* x, const int32_t* qweight, const void* qscales, const i
              const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
              int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* awq_gemv with the gate/up epilogue of the MLP fused in.  The packed buffers hold the gate and the up
+ * projection interleaved word by word along N: packed word column 2t = the 8 gate columns 8t..8t+7,
+ * word column 2t+1 = the up columns of the same outputs (qzeros and qscales alike), N = 2 * intermediate.
+ * y [M, N/2] = dtype(SiLU(dtype(x @ Wgate))) * dtype(x @ Wup), the rounding points of the reference's
+ * F.silu(self.gate_proj(x)) * self.up_proj(x), nanoquantization/models/qwen3_quantized.py:147-152.
+ * M <= 64, N % 128 == 0, group_size % 128 == 0; workspace as for awq_gemv(M, N, K). */
+int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                    void* y, int64_t M, int64_t N, int64_t K, int64_t group_size, int dtype,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
 /* Prefill regime, any M >= 1 (meant for M > 16): fused dequant + MFMA GEMM,
  * y = x @ dequant(W) (+ bias), W rounded to dtype exactly as the reference
  * does before the product, fp32 accumulation.

@@ -173,12 +173,39 @@ __device__ __forceinline__ void compute_chunk(const Chunk<V, CH, MT>& d, f32x4 (
 // (fixed order), then either store y (splits == 1) or publish this split's
 // partial and let the last workgroup of the tile group add the partials in
 // split order.  `group` is the workgroup's index along N.
+// Gated epilogue: the N columns are word-interleaved (word 2t = 8 gate columns, word 2t+1 = the 8 up
+// columns of the same outputs), a lane holds one word of a row, its neighbour (lane ^ 1) the partner
+// word.  out = dtype(SiLU(dtype(gate))) * dtype(up), written to y [M, N/2] by the gate lanes.  Every lane
+// of a pair must call this (the exchange is a cross-lane read).
+template <typename T>
+__device__ __forceinline__ void swiglu_store(const float (&out)[8], uint16_t* __restrict__ y, int m, int N,
+                                             size_t n0) {
+    float other[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) other[c] = __shfl_xor(out[c], 1);
+    if (((n0 >> 3) & 1) == 0) {
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float r[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const float g = T::to_f32(T::from_f32(out[2 * i + h]));
+                const float u = T::to_f32(T::from_f32(other[2 * i + h]));
+                r[h] = T::to_f32(T::from_f32(g / (1.f + __expf(-g)))) * u;
+            }
+            o[i] = T::pack2(r[0], r[1]);
+        }
+        *reinterpret_cast<u32x4*>(y + (size_t)m * (N >> 1) + (n0 >> 1)) = o;
+    }
+}
+
 template <typename T, int V, int WN, int WK>
 __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_base, float* red, int lane,
                                                   int wave, int group, int split, int splits,
                                                   const uint16_t* __restrict__ bias,
                                                   uint16_t* __restrict__ y, float* __restrict__ partials,
-                                                  int M, int N) {
+                                                  int M, int N, int act) {
     constexpr int NF = 8 * V, NQ = 4 * V;
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
@@ -221,7 +248,9 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
         }
         if (m < M && col_ok) {
             const size_t n0 = ((size_t)wv_col * V + v) * 8;
-            if (splits == 1) {
+            if (splits == 1 && act) {
+                swiglu_store<T>(out, y, m, N, n0);
+            } else if (splits == 1) {
                 if (bias) {
                     const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
 #pragma unroll
@@ -245,7 +274,7 @@ template <typename T, int V, int WN, int WK>
 __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int splits,
                                                 const uint16_t* __restrict__ bias,
                                                 uint16_t* __restrict__ y, float* __restrict__ partials,
-                                                int* __restrict__ counters, int M, int N) {
+                                                int* __restrict__ counters, int M, int N, int act) {
     constexpr int WAVES = WN * WK;
     const int words = N >> 3;
     if (!arrive_last(&counters[group], splits, s_last)) return;
@@ -277,6 +306,10 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
                     }
                 }
         }
+        if (act) {   // w_count is even here: a gate word and its up word sit in neighbouring lanes
+            swiglu_store<T>(out, y, m, N, n0);
+            continue;
+        }
         if (bias) {
             const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
 #pragma unroll
@@ -301,7 +334,7 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* re
                                               int wave, int group, int split, int splits,
                                               const uint16_t* __restrict__ bias,
                                               uint16_t* __restrict__ y, float* __restrict__ partials,
-                                              int* __restrict__ counters, int M, int N) {
+                                              int* __restrict__ counters, int M, int N, int act = 0) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (mt > 0) {
@@ -309,10 +342,10 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* re
             __syncthreads();          // the reduction buffer is reused per m-tile
         }
         gemv_reduce_store<T, V, WN, WK>(acc[mt], 16 * mt, red, lane, wave, group, split, splits, bias, y,
-                                        partials, M, N);
+                                        partials, M, N, act);
     }
     if (splits == 1) return;
-    gemv_split_tail<T, V, WN, WK>(s_last, group, splits, bias, y, partials, counters, M, N);
+    gemv_split_tail<T, V, WN, WK>(s_last, group, splits, bias, y, partials, counters, M, N, act);
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
@@ -427,7 +460,7 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
-    int splits) {
+    int splits, int act) {
     constexpr int CH = 4;
     extern __shared__ float red[];  // staging while streaming, [WAVES][32][64] floats afterwards
     __shared__ int s_last;
@@ -555,7 +588,7 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     }
     __syncthreads();  // staging area becomes the reduction buffer
     gemv_epilogue<T, 1, WN, WK, MT>(acc, red, &s_last, lane, wave, group, split, splits, bias, y, partials,
-                                counters, M, N);
+                                counters, M, N, act);
 }
 
 // ---- host side -------------------------------------------------------------
@@ -624,7 +657,7 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
 template <typename T, int WN, int WK, int DEPTH, int MT>
 static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
-                                  int g, void* workspace, int split_k, hipStream_t stream) {
+                                  int g, void* workspace, int split_k, hipStream_t stream, int act) {
     constexpr int WAVES = WN * WK;
     const int groups = N / (128 * WN);
     const int total_chunks = K / 128;
@@ -658,7 +691,7 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
                        reinterpret_cast<const uint16_t*>(qscales),
                        reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
-                       partials, counters, M, N, K, g / 128, cps, splits);
+                       partials, counters, M, N, K, g / 128, cps, splits, act);
     return hipGetLastError();
 }
 
@@ -726,9 +759,14 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
 static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, const void* qscales,
                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
-                         void* stream, int variant, int split_k) {
+                         void* stream, int variant, int split_k, int act = 0) {
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
+    if (act && (variant < kFirstDmaVariant || bias)) {
+        set_error("%s: the gated epilogue runs on the staged path only (N %% 128 == 0, group_size %% 128 == 0) "
+                  "and takes no bias", fn);
+        return AWQ_ERR_UNSUPPORTED;
+    }
     if (M > 64) {
         set_error("%s: M=%lld is outside the decode regime (1..64); use awq_gemm", fn, (long long)M);
         return AWQ_ERR_UNSUPPORTED;
@@ -782,9 +820,9 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     if (gv.wn == NN && gv.waves == NN * KK && gv.depth == DD && gv.mt == MM)                        \
         e = dtype == AWQ_F16                                                                        \
                 ? launch_gemv_dma<F16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                       (int)N, (int)K, (int)g, workspace, split_k, s) \
+                                                       (int)N, (int)K, (int)g, workspace, split_k, s, act) \
                 : launch_gemv_dma<BF16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                        (int)N, (int)K, (int)g, workspace, split_k, s);
+                                                        (int)N, (int)K, (int)g, workspace, split_k, s, act);
         AWQ_DMA_CASE(1, 4, 1, 1)
         AWQ_DMA_CASE(1, 8, 1, 1)
         AWQ_DMA_CASE(1, 16, 1, 1)
@@ -853,6 +891,16 @@ extern "C" size_t awq_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     awq::pick_gemv(M, N, K, 32, &v, &s);
     const size_t b = awq::gemv_ws_bytes(M, N, K, v, s);
     return a > b ? a : b;
+}
+
+extern "C" int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void* qscales,
+                               const int32_t* qzeros, void* y, int64_t M, int64_t N, int64_t K,
+                               int64_t group_size, int dtype, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+    int v = 0, s = 1;
+    if (K >= 32 && N >= 8 && group_size > 0) awq::pick_gemv(M, N, K, group_size, &v, &s);
+    return awq::gemv_dispatch("awq_gemv_swiglu", x, qweight, qscales, qzeros, nullptr, y, M, N, K, group_size,
+                              dtype, workspace, workspace_bytes, stream, v, s, 1);
 }
 
 extern "C" int awq_gemv_ex(const void* x, const int32_t* qweight, const void* qscales,

@@ -80,6 +80,12 @@ class LLMEngine:
         self.cache = PagedKVCache(len(layers), num_blocks, block_size, self.nkv, self.hd, self.dtype, self.device)
         self.qkv = [_FusedLinear([l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj]) for l in layers]
         self.gate_up = [_FusedLinear([l.mlp.gate_proj, l.mlp.up_proj]) for l in layers]
+        # decode: gate and up interleaved word by word, SiLU(gate) * up applied in the GEMV's epilogue
+        g0 = layers[0].mlp.gate_proj
+        self.swiglu_ok = (max_batch <= 64 and (2 * self.inter) % 128 == 0 and g0.group_size % 128 == 0)
+        self.gate_up_il = [ops.interleave_gate_up((l.mlp.gate_proj.qweight, l.mlp.gate_proj.qscales, l.mlp.gate_proj.qzeros),
+                                                  (l.mlp.up_proj.qweight, l.mlp.up_proj.qscales, l.mlp.up_proj.qzeros))
+                           for l in layers] if self.swiglu_ok else None
         self.use_graph = use_graph
         self._graph = None
         B, dev = max_batch, self.device
@@ -155,7 +161,9 @@ class LLMEngine:
                                        self.nh, self.nkv, self.hd, attn.q_norm.eps)
             o = ops.paged_attention_decode(q, self.cache.k[li], self.cache.v[li], self.s_table, ctx, self.scale)
             h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
-            delta = layer.mlp.down_proj(ops.silu_mul(self.gate_up[li](h)))
+            act = (ops.awq_gemv_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
+                   else ops.silu_mul(self.gate_up[li](h)))
+            delta = layer.mlp.down_proj(act)
         h = ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps)
         nxt = self.model.lm_head(h).argmax(dim=-1)
         self.s_out.index_copy_(0, self.s_step, nxt.unsqueeze(0))

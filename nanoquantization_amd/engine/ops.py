@@ -99,3 +99,35 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
         _lib.check(_lib.lib().nq_silu_mul(gate_up.data_ptr(), out.data_ptr(), rows, inter,
                                           _lib.dtype_id(gate_up.dtype), _stream()))
     return out
+
+
+def interleave_gate_up(gate, up):
+    """Packed buffers (qweight, qscales, qzeros) of the gate and the up projection -> one set with the word
+    columns interleaved (word 2t = gate word t, word 2t+1 = up word t), the layout awq_gemv_swiglu takes."""
+    gq, gs, gz = gate
+    uq, us, uz = up
+    K, W = gq.shape
+    G = gz.shape[0]
+    qweight = torch.stack([gq, uq], dim=2).reshape(K, 2 * W).contiguous()
+    qzeros = torch.stack([gz, uz], dim=2).reshape(G, 2 * W).contiguous()
+    qscales = torch.stack([gs.view(G, W, 8), us.view(G, W, 8)], dim=2).reshape(G, 16 * W).contiguous()
+    return qweight, qscales, qzeros
+
+
+def awq_gemv_swiglu(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor) -> torch.Tensor:
+    """x [M <= 64, K] and interleaved gate|up buffers [K, 2*inter/8] -> SiLU(x @ Wgate) * (x @ Wup) [M, inter]."""
+    dev = _dev(x, qweight, qscales, qzeros)
+    M, K = x.shape
+    N = qscales.shape[1]
+    g = K // qscales.shape[0]
+    assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    out = torch.empty(M, N // 2, dtype=x.dtype, device=dev)
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        stream = _stream()
+        nbytes = L.awq_gemv_workspace_bytes(M, N, K)
+        ws = _lib.workspace(dev, stream, nbytes)
+        _lib.check(L.awq_gemv_swiglu(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(),
+                                     out.data_ptr(), M, N, K, g, _lib.dtype_id(x.dtype),
+                                     None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), stream))
+    return out

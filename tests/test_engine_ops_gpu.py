@@ -145,3 +145,25 @@ def test_silu_mul(dtype, rows, inter):
     g = torch.Generator().manual_seed(rows + inter)
     gu = (2 * torch.randn(rows, 2 * inter, generator=g)).to(dtype).cuda()
     _close(ops.silu_mul(gu), F.silu(gu[:, :inter]) * gu[:, inter:], dtype, what="silu*up")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,inter", [(1, 1024, 3072), (32, 1024, 3072), (16, 2048, 1024), (64, 5120, 1280), (3, 4096, 64)])
+def test_gemv_swiglu_equals_unfused(dtype, M, K, inter):
+    """Gate and up interleaved + gated epilogue must give, bit for bit, what the plain GEMV over gate|up side by
+    side followed by the SiLU*up kernel gives (a column's sum does not depend on where the column sits)."""
+    import nanoquantization_amd as nq
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(M * 31 + K + inter)
+    def packed(n):
+        return (torch.randint(-2 ** 31, 2 ** 31 - 1, (K, n // 8), dtype=torch.int32, device="cuda", generator=g),
+                (torch.rand(K // 128, n, device="cuda", generator=g) * 0.02 + 0.001).to(dtype),
+                torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, n // 8), dtype=torch.int32, device="cuda", generator=g))
+    gate, up = packed(inter), packed(inter)
+    x = torch.randn(M, K, device="cuda", generator=g).to(dtype)
+    print(f"gemv_swiglu M={M} K={K} inter={inter} {dtype}", flush=True)
+    fused = ops.awq_gemv_swiglu(x, *ops.interleave_gate_up(gate, up))
+    side = [torch.cat([a, b], dim=1).contiguous() for a, b in zip(gate, up)]
+    ref = ops.silu_mul(nq.awq_gemm(x, side[0], side[1], side[2], 8))
+    assert fused.shape == (M, inter)
+    assert torch.equal(fused, ref)
