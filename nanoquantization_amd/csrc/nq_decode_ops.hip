@@ -49,11 +49,13 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
     __shared__ float s_part[kNormThreads / kWave];
     const int64_t base = (int64_t)blockIdx.x * hidden;
     float v[kNormPasses][8];
+    u32x4 wraw[kNormPasses];   // the weight does not depend on the reduction: fetched up front
     float ss = 0.f;
 #pragma unroll
     for (int p = 0; p < kNormPasses; ++p) {
         const int i = (p * kNormThreads + threadIdx.x) * 8;
         if (i < hidden) {
+            wraw[p] = *reinterpret_cast<const u32x4*>(weight + i);
             unpack8<T>(*reinterpret_cast<const u32x4*>(residual + base + i), v[p]);
             if (delta) {
                 float d[8];
@@ -78,7 +80,7 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
         const int i = (p * kNormThreads + threadIdx.x) * 8;
         if (i < hidden) {
             float w[8], o[8];
-            unpack8<T>(*reinterpret_cast<const u32x4*>(weight + i), w);
+            unpack8<T>(wraw[p], w);
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = round_to<T>(v[p][e] * r) * w[e];
             *reinterpret_cast<u32x4*>(y + base + i) = pack8<T>(o);
@@ -138,20 +140,32 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
         }
         return;
     }
-    const float r = rsqrtf(wave_sum(ss) / (float)hd + eps);
+    // norm weight and angles do not depend on the reduction: fetched before it
     const uint16_t* w = h < nh ? q_weight : k_weight;
     int64_t pos = positions[row];
     pos = pos < 0 ? 0 : (pos >= max_positions ? max_positions - 1 : pos);
     const float* cs = cos_sin + pos * hd;
+    float w1[kMaxPairs], w2[kMaxPairs], cc[kMaxPairs], sn[kMaxPairs];
+#pragma unroll
+    for (int p = 0; p < kMaxPairs; ++p) {
+        const int i = p * 64 + lane;
+        w1[p] = w2[p] = cc[p] = sn[p] = 0.f;
+        if (i < half) {
+            w1[p] = T::to_f32(w[i]);
+            w2[p] = T::to_f32(w[i + half]);
+            cc[p] = cs[i];
+            sn[p] = cs[i + half];
+        }
+    }
+    const float r = rsqrtf(wave_sum(ss) / (float)hd + eps);
 #pragma unroll
     for (int p = 0; p < kMaxPairs; ++p) {
         const int i = p * 64 + lane;
         if (i < half) {
-            const float x1 = round_to<T>(round_to<T>(a[p] * r) * T::to_f32(w[i]));
-            const float x2 = round_to<T>(round_to<T>(b[p] * r) * T::to_f32(w[i + half]));
-            const float c = cs[i], s = cs[i + half];
-            dst[i] = T::from_f32(__fsub_rn(__fmul_rn(x1, c), __fmul_rn(x2, s)));
-            dst[i + half] = T::from_f32(__fadd_rn(__fmul_rn(x1, s), __fmul_rn(x2, c)));
+            const float x1 = round_to<T>(round_to<T>(a[p] * r) * w1[p]);
+            const float x2 = round_to<T>(round_to<T>(b[p] * r) * w2[p]);
+            dst[i] = T::from_f32(__fsub_rn(__fmul_rn(x1, cc[p]), __fmul_rn(x2, sn[p])));
+            dst[i + half] = T::from_f32(__fadd_rn(__fmul_rn(x1, sn[p]), __fmul_rn(x2, cc[p])));
         }
     }
 }
