@@ -709,6 +709,25 @@ static size_t gemv_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
 // workgroup with WK waves over K.  Splitting K across workgroups costs a
 // serial tail (publish, arrival counter, fetch: a few microseconds), so it is
 // used only while one workgroup per column tile leaves most SIMDs empty.
+// A workgroup gives each of its `wk` waves ceil(chunks_per_split / wk) chunks and lasts as long as the
+// busiest one (40 chunks in 4 splits over 4 waves: 3, 3, 3, 1 -- a quarter of the time wasted).  Among the
+// split counts from `s` to twice that (capped), take the one that wastes the fewest wave slots.
+static int64_t balance_splits(int64_t chunks, int64_t s, int64_t wk, int64_t cap) {
+    if (s <= 1) return 1;
+    int64_t best = s;
+    double best_eff = 0.0;
+    const int64_t hi = 2 * s < cap ? 2 * s : cap;
+    for (int64_t c = s; c <= hi; ++c) {
+        const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
+        const double eff = (double)chunks / (double)(splits * wk * cdiv(cps, wk));
+        if (eff > best_eff + 1e-9) {
+            best_eff = eff;
+            best = c;
+        }
+    }
+    return best;
+}
+
 static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, int* split_k) {
     const int64_t chunks = K / 128 > 0 ? K / 128 : 1;
     if (N % 128 == 0 && g % 128 == 0) {
@@ -732,11 +751,14 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             v = 11 /* dma1x8d1 */;
         } else if (M <= 4) {
             s = cdiv(3072, tiles * 4);
-            const int64_t cap = chunks / 2 < 10 ? chunks / 2 : 10;
+            // short K: at most 10 splits (the tail is a larger share of a 6 us launch); long K: up to 32
+            const int64_t cap = chunks < 64 ? (chunks / 2 < 10 ? chunks / 2 : 10) : 32;
             if (s > cap) s = cap;
+            s = balance_splits(chunks, s, 4, cap);
         } else if (tiles < 200) {
             s = cdiv(200, tiles);   // about 200 workgroups
             if (s > chunks / 4) s = chunks / 4;
+            s = balance_splits(chunks, s, 4, chunks / 4);
         }
         if (s < 1) s = 1;
         *variant = v;
