@@ -31,7 +31,8 @@ int nq_add_rmsnorm(void* residual, const void* delta, const void* weight, void* 
  * side by side.  Every q and k head is RMS-normalised (q_weight / k_weight, [head_dim]) and rotated
  * (half-split rotary, angle table cos_sin f32 [max_positions, head_dim] = cos | sin) at
  * positions[row]; q goes to q_out [rows, num_heads, head_dim], k and the untouched v go to
- * k_cache / v_cache [num_slots, num_kv_heads, head_dim] at slots[row] (a row whose slot is outside
+ * k_cache / v_cache [num_slots / block_size, num_kv_heads, block_size, head_dim] (a head's tokens of one
+ * block are contiguous) at slot slots[row] = block * block_size + offset (a row whose slot is outside
  * [0, num_slots) writes no k/v).  head_dim even, <= 256.
  * Qwen3QuantizedAttention.forward, nanoquantization/models/qwen3_quantized.py:79-93;
  * RoPE.apply_rope / forward, nanoquantization/layers/rope.py:24-45. */
@@ -39,7 +40,7 @@ int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, const void* k_w
                           const float* cos_sin, const int64_t* positions, const int64_t* slots,
                           void* q_out, void* k_cache, void* v_cache, int64_t rows, int64_t num_heads,
                           int64_t num_kv_heads, int64_t head_dim, int64_t max_positions,
-                          int64_t num_slots, float eps, int dtype, void* stream);
+                          int64_t num_slots, int64_t block_size, float eps, int dtype, void* stream);
 
 /* Bytes of device workspace nq_paged_attention_decode needs (0 is possible); no initialisation
  * needed.  max_context = block_size * max_blocks_per_seq. */
@@ -47,9 +48,9 @@ size_t nq_paged_attention_workspace_bytes(int64_t batch, int64_t num_heads, int6
                                           int64_t head_dim, int64_t max_context);
 
 /* out[b, h, :] = softmax(scale * q[b, h, :] . K_b^T) V_b over the first context_lens[b] tokens of
- * sequence b (the new token's k/v already written).  Token t of sequence b lives in cache slot
- * block_table[b, t / block_size] * block_size + t % block_size of k_cache / v_cache
- * [num_blocks * block_size, num_kv_heads, head_dim]; query head h reads kv head
+ * sequence b (the new token's k/v already written).  Token t of sequence b is token t % block_size
+ * of block block_table[b, t / block_size] in k_cache / v_cache
+ * [num_blocks, num_kv_heads, block_size, head_dim]; query head h reads kv head
  * h / (num_heads / num_kv_heads).  q, out: [batch, num_heads, head_dim].  head_dim 64 or 128,
  * num_heads / num_kv_heads in {1, 2, 4, 8}; block indices are clamped to the cache.
  * F.scaled_dot_product_attention(..., enable_gqa) of Qwen3QuantizedAttention.forward,

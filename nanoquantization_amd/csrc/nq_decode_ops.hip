@@ -92,6 +92,7 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
 // One wave per (token row, head) of the fused q|k|v projection output.  q and k heads: RMSNorm over
 // the head, then the half-split rotary at the row's position; q goes to q_out, k to its cache
 // slot; v heads are copied to their cache slot.  A lane owns the rotary pairs (i, i + hd/2).
+// Cache layout [blocks][kv heads][block_size][head_dim]: slot s is token s % block_size of block s / block_size.
 constexpr int kMaxPairs = 2;  // head_dim <= 256
 
 template <typename T>
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ q_weight, const uint16_t* __restrict__ k_weight,
     const float* __restrict__ cos_sin, const int64_t* __restrict__ positions, const int64_t* __restrict__ slots,
     uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache, int rows, int nh,
-    int nkv, int hd, int max_positions, int64_t num_slots, float eps) {
+    int nkv, int hd, int max_positions, int64_t num_slots, int block_size, float eps) {
     const int heads = nh + 2 * nkv;
     const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (item >= (int64_t)rows * heads) return;
@@ -112,10 +113,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
         dst = q_out + ((int64_t)row * nh + h) * hd;
     } else if (h < nh + nkv) {
         if (!slot_ok) return;
-        dst = k_cache + (slot * nkv + (h - nh)) * hd;
+        dst = k_cache + (((slot / block_size) * nkv + (h - nh)) * block_size + slot % block_size) * hd;
     } else {
         if (!slot_ok) return;
-        dst = v_cache + (slot * nkv + (h - nh - nkv)) * hd;
+        dst = v_cache + (((slot / block_size) * nkv + (h - nh - nkv)) * block_size + slot % block_size) * hd;
     }
     float a[kMaxPairs], b[kMaxPairs];
     float ss = 0.f;
@@ -230,7 +231,7 @@ __global__ __launch_bounds__(256) void paged_attn_decode_kernel(
             const int tc = ok[u] ? tt : t0;
             int blk = table[tc / block_size];
             blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);
-            const int64_t off = (((int64_t)blk * block_size + tc % block_size) * nkv + kvh) * HD + dc * 8;
+            const int64_t off = (((int64_t)blk * nkv + kvh) * block_size + tc % block_size) * HD + dc * 8;
             kr[u] = *reinterpret_cast<const u32x4*>(k_cache + off);
             vr[u] = *reinterpret_cast<const u32x4*>(v_cache + off);
         }
@@ -422,14 +423,15 @@ extern "C" int nq_add_rmsnorm(void* residual, const void* delta, const void* wei
 extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, const void* k_weight, const float* cos_sin,
                                      const int64_t* positions, const int64_t* slots, void* q_out, void* k_cache,
                                      void* v_cache, int64_t rows, int64_t num_heads, int64_t num_kv_heads,
-                                     int64_t head_dim, int64_t max_positions, int64_t num_slots, float eps, int dtype,
-                                     void* stream) {
+                                     int64_t head_dim, int64_t max_positions, int64_t num_slots, int64_t block_size,
+                                     float eps, int dtype, void* stream) {
     const char* fn = "nq_qk_norm_rope_store";
     if (!qkv || !q_weight || !k_weight || !cos_sin || !positions || !slots || !q_out || !k_cache || !v_cache)
         return bad(fn, "null pointer argument");
     if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
-    if (rows <= 0 || num_heads <= 0 || num_kv_heads <= 0 || max_positions <= 0 || num_slots <= 0)
-        return bad(fn, "rows, head counts, max_positions and num_slots must be positive");
+    if (rows <= 0 || num_heads <= 0 || num_kv_heads <= 0 || max_positions <= 0 || num_slots <= 0 || block_size <= 0 ||
+        block_size > 0x7fffffff || num_slots % block_size != 0)
+        return bad(fn, "rows, head counts, max_positions, block_size must be positive and num_slots a multiple of block_size");
     if (head_dim <= 0 || head_dim % 2 != 0 || head_dim > 128 * kMaxPairs) {
         set_error("%s: head_dim must be even and at most %d, got %lld", fn, 128 * kMaxPairs, (long long)head_dim);
         return AWQ_ERR_UNSUPPORTED;
@@ -443,12 +445,12 @@ extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, cons
         qk_norm_rope_store_kernel<F16><<<grid, block, 0, st>>>(
             (const uint16_t*)qkv, (const uint16_t*)q_weight, (const uint16_t*)k_weight, cos_sin, positions, slots,
             (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads, (int)num_kv_heads,
-            (int)head_dim, (int)max_positions, num_slots, eps);
+            (int)head_dim, (int)max_positions, num_slots, (int)block_size, eps);
     else
         qk_norm_rope_store_kernel<BF16><<<grid, block, 0, st>>>(
             (const uint16_t*)qkv, (const uint16_t*)q_weight, (const uint16_t*)k_weight, cos_sin, positions, slots,
             (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads, (int)num_kv_heads,
-            (int)head_dim, (int)max_positions, num_slots, eps);
+            (int)head_dim, (int)max_positions, num_slots, (int)block_size, eps);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }

@@ -1,7 +1,7 @@
 """Paged-KV greedy generation for Qwen3QuantizedForCausalLM on one MI355X.
 
-Layout.  One K and one V tensor per model: [layers, blocks, block_size, kv_heads, head_dim] in the
-model dtype; a sequence owns a list of blocks (its row of the block table); token t of a sequence
+Layout.  One K and one V tensor per model: [layers, blocks, kv_heads, block_size, head_dim] in the
+model dtype (a head's tokens of one block are contiguous: 16 KiB runs for the attention kernel); a sequence owns a list of blocks (its row of the block table); token t of a sequence
 lives in slot block_table[t // block_size] * block_size + t % block_size.
 
 Weights.  q/k/v (same input) and gate/up (same input) are concatenated along N into one packed AWQ
@@ -33,7 +33,7 @@ class PagedKVCache:
                  dtype: torch.dtype, device: torch.device):
         self.block_size = block_size
         self.num_blocks = num_blocks
-        shape = (num_layers, num_blocks, block_size, num_kv_heads, head_dim)
+        shape = (num_layers, num_blocks, num_kv_heads, block_size, head_dim)
         self.k = torch.zeros(shape, dtype=dtype, device=device)
         self.v = torch.zeros(shape, dtype=dtype, device=device)
         self.free: List[int] = list(range(num_blocks - 1, -1, -1))
@@ -113,8 +113,9 @@ class LLMEngine:
         k = k.view(b, s, self.nkv, self.hd)
         v = v.view(b, s, self.nkv, self.hd)
         q, k = attn.rope(attn.q_norm(q), attn.k_norm(k), pos)
-        self.cache.k[li].view(-1, self.nkv, self.hd).index_copy_(0, slots, k.reshape(b * s, self.nkv, self.hd))
-        self.cache.v[li].view(-1, self.nkv, self.hd).index_copy_(0, slots, v.reshape(b * s, self.nkv, self.hd))
+        blk, off = slots // self.block_size, slots % self.block_size
+        self.cache.k[li][blk, :, off] = k.reshape(b * s, self.nkv, self.hd)
+        self.cache.v[li][blk, :, off] = v.reshape(b * s, self.nkv, self.hd)
         o = attend(q, k, v, li)
         x = x + attn.o_proj(o).view(b, s, -1)
         h = layer.post_attention_layernorm(x)

@@ -44,14 +44,15 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
 def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, cos_sin: torch.Tensor,
                        positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                        num_heads: int, num_kv_heads: int, head_dim: int, eps: float) -> torch.Tensor:
-    """qkv [rows, (nh + 2 nkv) * hd]; caches [..., nkv, hd] viewed as slots; returns q [rows, nh, hd]."""
+    """qkv [rows, (nh + 2 nkv) * hd]; caches [blocks, nkv, block_size, hd]; returns q [rows, nh, hd]."""
     dev = _dev(qkv, q_weight, k_weight, cos_sin, positions, slots, k_cache, v_cache)
     rows = qkv.shape[0]
     assert qkv.shape[1] == (num_heads + 2 * num_kv_heads) * head_dim
     assert q_weight.shape == (head_dim,) and k_weight.shape == (head_dim,)
     assert q_weight.dtype == qkv.dtype and k_weight.dtype == qkv.dtype
     assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and k_cache.shape == v_cache.shape
-    assert k_cache.shape[-2:] == (num_kv_heads, head_dim)
+    assert k_cache.dim() == 4 and k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim
+    block_size = k_cache.shape[2]
     assert cos_sin.dtype == torch.float32 and cos_sin.numel() % head_dim == 0
     assert positions.dtype == torch.int64 and slots.dtype == torch.int64
     assert positions.numel() == rows and slots.numel() == rows
@@ -61,17 +62,17 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torc
         _lib.check(_lib.lib().nq_qk_norm_rope_store(
             qkv.data_ptr(), q_weight.data_ptr(), k_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(),
             slots.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), rows, num_heads, num_kv_heads,
-            head_dim, cos_sin.numel() // head_dim, num_slots, eps, _lib.dtype_id(qkv.dtype), _stream()))
+            head_dim, cos_sin.numel() // head_dim, num_slots, block_size, eps, _lib.dtype_id(qkv.dtype), _stream()))
     return q
 
 
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                            context_lens: torch.Tensor, scale: float) -> torch.Tensor:
-    """q [batch, nh, hd]; caches [num_blocks, block_size, nkv, hd]; block_table int32 [batch, max_blocks];
+    """q [batch, nh, hd]; caches [num_blocks, nkv, block_size, hd]; block_table int32 [batch, max_blocks];
     context_lens int32 [batch].  Returns [batch, nh * hd]."""
     dev = _dev(q, k_cache, v_cache, block_table, context_lens)
     batch, nh, hd = q.shape
-    num_blocks, block_size, nkv, hd2 = k_cache.shape
+    num_blocks, nkv, block_size, hd2 = k_cache.shape
     assert hd2 == hd and v_cache.shape == k_cache.shape and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype
     assert block_table.dtype == torch.int32 and context_lens.dtype == torch.int32
     assert block_table.shape[0] == batch and context_lens.shape == (batch,)

@@ -66,7 +66,8 @@ def test_qk_norm_rope_store(dtype, nh, nkv, hd):
     slots = torch.randperm(num_slots, generator=g)[:rows].cuda()
     slots[5] = -1            # a row that owns no cache slot
     rope = RoPE(hd, max_pos).cuda()
-    kc = torch.zeros(num_slots, nkv, hd, dtype=dtype, device="cuda")
+    bs = 16
+    kc = torch.zeros(num_slots // bs, nkv, bs, hd, dtype=dtype, device="cuda")   # [blocks, kv heads, block, hd]
     vc = torch.zeros_like(kc)
     q = ops.qk_norm_rope_store(qkv, qw, kw, rope.cos_sin_cache, pos, slots, kc, vc, nh, nkv, hd, 1e-6)
 
@@ -76,24 +77,25 @@ def test_qk_norm_rope_store(dtype, nh, nkv, hd):
     qr, kr = rope(qr, kr, pos.view(rows, 1))
     _close(q, qr.view(rows, nh, hd), dtype, what="q")
     keep = slots >= 0
-    _close(kc[slots[keep]], kr.view(rows, nkv, hd)[keep], dtype, what="k cache")
-    assert torch.equal(vc[slots[keep]], vr.reshape(rows, nkv, hd)[keep]), "v is copied bit for bit"
+    by_slot = lambda c: c.permute(0, 2, 1, 3).reshape(num_slots, nkv, hd)      # slot = block * bs + offset
+    _close(by_slot(kc)[slots[keep]], kr.view(rows, nkv, hd)[keep], dtype, what="k cache")
+    assert torch.equal(by_slot(vc)[slots[keep]], vr.reshape(rows, nkv, hd)[keep]), "v is copied bit for bit"
     untouched = torch.ones(num_slots, dtype=torch.bool, device="cuda")
     untouched[slots[keep]] = False
-    assert not kc[untouched].any() and not vc[untouched].any(), "slots of other tokens must stay untouched"
+    assert not by_slot(kc)[untouched].any() and not by_slot(vc)[untouched].any(), "other slots must stay untouched"
 
 
 def _attn_ref(q, kc, vc, table, ctx, scale):
     B, nh, hd = q.shape
-    nb, bs, nkv, _ = kc.shape
+    nb, nkv, bs, _ = kc.shape
     G = nh // nkv
     out = torch.empty(B, nh, hd, dtype=torch.float32, device=q.device)
     for b in range(B):
         n = int(ctx[b])
         t = torch.arange(n, device=q.device)
-        sl = table[b, t // bs].long() * bs + t % bs
-        k = kc.view(-1, nkv, hd)[sl].float().repeat_interleave(G, dim=1)      # [n, nh, hd]
-        v = vc.view(-1, nkv, hd)[sl].float().repeat_interleave(G, dim=1)
+        blk, off = table[b, t // bs].long(), t % bs
+        k = kc[blk, :, off].float().repeat_interleave(G, dim=1)               # [n, nh, hd]
+        v = vc[blk, :, off].float().repeat_interleave(G, dim=1)
         s = torch.einsum("hd,nhd->hn", q[b].float(), k) * scale
         out[b] = torch.einsum("hn,nhd->hd", torch.softmax(s, dim=-1), v)
     return out.view(B, nh * hd)
@@ -112,8 +114,8 @@ def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
     from nanoquantization_amd.engine import ops
     g = torch.Generator().manual_seed(B * 1000 + nh)
     nb = B * max_blocks + 3
-    kc = torch.randn(nb, bs, nkv, hd, generator=g).to(dtype).cuda()
-    vc = torch.randn(nb, bs, nkv, hd, generator=g).to(dtype).cuda()
+    kc = torch.randn(nb, nkv, bs, hd, generator=g).to(dtype).cuda()
+    vc = torch.randn(nb, nkv, bs, hd, generator=g).to(dtype).cuda()
     q = torch.randn(B, nh, hd, generator=g).to(dtype).cuda()
     table = torch.randperm(nb, generator=g)[: B * max_blocks].view(B, max_blocks).to(torch.int32).cuda()
     ctx = torch.randint(1, bs * max_blocks + 1, (B,), generator=g).to(torch.int32)
@@ -129,7 +131,7 @@ def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
 def test_paged_attention_rejects_unsupported():
     from nanoquantization_amd import _lib
     from nanoquantization_amd.engine import ops
-    kc = torch.zeros(4, 16, 1, 128, dtype=torch.bfloat16, device="cuda")
+    kc = torch.zeros(4, 1, 16, 128, dtype=torch.bfloat16, device="cuda")
     q = torch.zeros(1, 3, 128, dtype=torch.bfloat16, device="cuda")
     tb = torch.zeros(1, 2, dtype=torch.int32, device="cuda")
     cx = torch.ones(1, dtype=torch.int32, device="cuda")
