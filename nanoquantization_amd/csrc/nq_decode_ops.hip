@@ -173,7 +173,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
 
 // ---------------------------------------------------------------------------------------------
 // Attention of one new token per sequence over its paged KV cache (flash-decoding).
-// Workgroup = (sequence, kv head, context split), 4 waves.  A wave covers TPW = 64 / (HD/8) tokens
+// Workgroup = (sequence, kv head, context split), WAVES waves (16 for up to 2 query heads per kv head, 8 for
+// 4, 4 for 8: the wave merge buffer grows with G); with enough waves per workgroup a batch of sequences
+// needs no context split and no second kernel.  A wave covers TPW = 64 / (HD/8) tokens
 // per step: a lane holds 8 head dims of one token's K and V rows (one 16-byte load each), the G
 // query heads of the kv group share those loads.  Every lane group keeps its own online-softmax
 // state (running max, sum, 8 accumulators per query head); the states are merged across lane
@@ -184,8 +186,8 @@ struct SoftState {
     float m, l;
 };
 
-template <typename T, int G, int HD>
-__global__ __launch_bounds__(256) void paged_attn_decode_kernel(
+template <typename T, int G, int HD, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, const int32_t* __restrict__ context_lens, uint16_t* __restrict__ out,
     float* __restrict__ partial, int nkv, int block_size, int max_blocks, int num_blocks, int nsplit, float scale) {
@@ -221,12 +223,12 @@ __global__ __launch_bounds__(256) void paged_attn_decode_kernel(
     }
 
     const int32_t* table = block_table + (int64_t)b * max_blocks;
-    for (int t = t0 + wave * TPW + ts; t - ts < t1; t += 4 * TPW * U) {
+    for (int t = t0 + wave * TPW + ts; t - ts < t1; t += WAVES * TPW * U) {
         u32x4 kr[U], vr[U];
         bool ok[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int tt = t + u * 4 * TPW;
+            const int tt = t + u * WAVES * TPW;
             ok[u] = tt < t1;
             const int tc = ok[u] ? tt : t0;
             int blk = table[tc / block_size];
@@ -273,8 +275,8 @@ __global__ __launch_bounds__(256) void paged_attn_decode_kernel(
             m[g] = mn;
         }
     }
-    // merge the 4 waves through LDS: [wave][g][HD + 2]
-    __shared__ float s_acc[4][G][HD + 2];
+    // merge the waves through LDS: [wave][g][HD + 2]
+    __shared__ float s_acc[WAVES][G][HD + 2];
     if (ts == 0) {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
@@ -287,14 +289,14 @@ __global__ __launch_bounds__(256) void paged_attn_decode_kernel(
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
+    for (int idx = threadIdx.x; idx < G * HD; idx += 64 * WAVES) {
         const int g = idx / HD, d = idx % HD;
         float mn = kNegBig;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) mn = fmaxf(mn, s_acc[w][g][HD]);
+        for (int w = 0; w < WAVES; ++w) mn = fmaxf(mn, s_acc[w][g][HD]);
         float lt = 0.f, at = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < WAVES; ++w) {
             const float c = exp2f(s_acc[w][g][HD] - mn);
             lt += s_acc[w][g][HD + 1] * c;
             at += s_acc[w][g][d] * c;
@@ -354,8 +356,10 @@ int bad(const char* fn, const char* what) {
 }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int pick_splits(int64_t batch, int64_t nkv, int64_t max_context) {
-    int64_t s = cdiv(1024, batch * nkv);
+int attn_waves(int G) { return G <= 2 ? 16 : (G <= 4 ? 8 : 4); }
+
+int pick_splits(int64_t batch, int64_t nkv, int64_t max_context, int G) {
+    int64_t s = cdiv(4096, batch * nkv * attn_waves(G));   // about 4096 waves on the chip
     const int64_t cap = max_context / 64 > 1 ? max_context / 64 : 1;
     s = s > cap ? cap : s;
     s = s > 16 ? 16 : s;
@@ -366,7 +370,8 @@ template <typename T, int G, int HD>
 void launch_attn(const void* q, const void* kc, const void* vc, const int32_t* table, const int32_t* ctx, void* out,
                  float* partial, int64_t batch, int nkv, int bs, int max_blocks, int num_blocks, int nsplit,
                  float scale, hipStream_t st) {
-    paged_attn_decode_kernel<T, G, HD><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(256), 0, st>>>(
+    constexpr int WAVES = G <= 2 ? 16 : (G <= 4 ? 8 : 4);
+    paged_attn_decode_kernel<T, G, HD, WAVES><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(64 * WAVES), 0, st>>>(
         (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, table, ctx, (uint16_t*)out, partial, nkv, bs,
         max_blocks, num_blocks, nsplit, scale);
     if (nsplit > 1)
@@ -458,7 +463,7 @@ extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, cons
 extern "C" size_t nq_paged_attention_workspace_bytes(int64_t batch, int64_t num_heads, int64_t num_kv_heads,
                                                      int64_t head_dim, int64_t max_context) {
     if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || max_context <= 0) return 0;
-    const int s = pick_splits(batch, num_kv_heads, max_context);
+    const int s = pick_splits(batch, num_kv_heads, max_context, (int)(num_heads / num_kv_heads));
     return s > 1 ? (size_t)(batch * num_heads * s * (head_dim + 2)) * sizeof(float) : 0;
 }
 
@@ -482,7 +487,7 @@ extern "C" int nq_paged_attention_decode(const void* q, const void* k_cache, con
     const int64_t max_context = block_size * max_blocks_per_seq;
     if (max_context > 0x7fffffff || num_blocks * block_size > 0x7fffffff || batch * num_kv_heads * 16 > 0x7fffffff)
         return bad(fn, "problem too large");
-    const int nsplit = pick_splits(batch, num_kv_heads, max_context);
+    const int nsplit = pick_splits(batch, num_kv_heads, max_context, (int)(num_heads / num_kv_heads));
     const size_t need = nq_paged_attention_workspace_bytes(batch, num_heads, num_kv_heads, head_dim, max_context);
     if (need && (!workspace || workspace_bytes < need || !aligned16(workspace))) {
         set_error("%s: workspace of %zu bytes needed, %zu given", fn, need, workspace ? workspace_bytes : (size_t)0);
