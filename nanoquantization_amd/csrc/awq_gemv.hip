@@ -738,14 +738,15 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int v = 10 /* dma1x4d1 */;
         int64_t s = 1;
         if (M > 16) {
-            // 17..64 rows: with 32 column tiles or more one 8-wave workgroup per tile covers the chip
-            // well enough; with fewer, split K until some 48 workgroups exist (4 chunks per split at least)
-            if (M <= 32 && tiles >= 32 && chunks >= 8) {
+            // 17..64 rows: short K with 32 column tiles or more runs as one 8-wave workgroup per tile;
+            // otherwise 4-wave workgroups, K split until about 200 of them exist (4 chunks per split at least)
+            if (M <= 32 && tiles >= 32 && chunks <= 8) {
                 v = 21 /* dma1x8d1m2 */;
             } else {
                 v = M > 32 ? 22 /* dma1x4d1m4 */ : 20 /* dma1x4d1m2 */;
-                if (tiles < 48) s = cdiv(48, tiles);
+                if (tiles < 200) s = cdiv(200, tiles);
                 if (s > chunks / 4) s = chunks / 4;
+                s = balance_splits(chunks, s, 4, chunks / 4);
             }
         } else if (chunks <= 8) {
             v = 11 /* dma1x8d1 */;
