@@ -15,6 +15,11 @@ decoding over the block table), o_proj GEMV, add+RMSNorm, fused gate|up GEMV, Si
 (include/nq_engine_ops.h + include/awq_hip.h).  All per-step state lives in fixed device buffers (token
 ids, positions, active mask, block table, step counter, output tokens) and the step advances that
 state itself, so it is captured once in a HIP graph and replayed with no host work between steps.
+
+Scheduling.  `generate` runs one static batch of equal-length prompts.  `serve` is continuous batching over
+the same decode graph: requests of any length wait in a queue, are admitted whenever a batch row and enough
+cache blocks are free (their prompt is prefilled on its own), decode together with whatever else is running,
+and give their row and blocks back when they reach their token budget or the end-of-sequence token.
 """
 from __future__ import annotations
 
@@ -169,7 +174,7 @@ class LLMEngine:
         nxt = self.model.lm_head(h).argmax(dim=-1)
         self.s_out.index_copy_(0, self.s_step, nxt.unsqueeze(0))
         self.s_ids.copy_(nxt)
-        self.s_pos.add_(1)
+        self.s_pos.add_(self.s_active.to(torch.long))               # idle rows stay where they are
         self.s_step.add_(1)
 
     def _state(self):
@@ -240,3 +245,107 @@ class LLMEngine:
         finally:
             for t in tables:
                 self.cache.release(t)
+
+    # ---- continuous batching ---------------------------------------------------------------------------
+    @torch.no_grad()
+    def serve(self, requests, eos_token_id: Optional[int] = None, stats: Optional[dict] = None) -> List[List[int]]:
+        """requests: sequence of (prompt token ids, max_new_tokens), any lengths.  Returns the greedy continuation
+        of each request, in request order (cut after `eos_token_id` if one is given).  Without an end-of-sequence
+        token the host reads tokens back only when the output buffer fills up or at the end; with one it reads
+        them after every step."""
+        import time
+        from collections import deque
+        bs = self.block_size
+        for prompt, max_new in requests:
+            if len(prompt) < 1 or max_new < 1:
+                raise ValueError("every request needs a non-empty prompt and max_new_tokens >= 1")
+            if len(prompt) + max_new > self.max_ctx:
+                raise ValueError("prompt + max_new_tokens exceeds max_seq_len")
+        out: List[List[int]] = [[] for _ in requests]
+        waiting = deque(range(len(requests)))
+        free_rows = list(range(self.max_batch - 1, -1, -1))
+        running = {}                      # row -> [request index, tokens still to decode, blocks]
+        step_log = []                     # per decode step since the last read-back: [(row, request index)]
+        self.s_active.zero_(); self.s_pos.zero_(); self.s_ids.zero_(); self.s_table.zero_(); self.s_step.zero_()
+        torch.cuda.synchronize()
+        t_start, n_steps, n_prefill = time.perf_counter(), 0, 0
+
+        def retire(row):
+            _, _, blocks = running.pop(row)
+            self.cache.release(blocks)
+            free_rows.append(row)
+            self.s_active[row] = False
+            self.s_pos[row] = 0
+
+        def read_back():
+            """Tokens of the logged steps -> their requests; returns the rows whose request ended with eos."""
+            ended = []
+            if step_log:
+                toks = self.s_out[:len(step_log)].tolist()
+                for i, entries in enumerate(step_log):
+                    for row, ri in entries:
+                        if out[ri] and eos_token_id is not None and out[ri][-1] == eos_token_id:
+                            continue            # already ended on an earlier step of this batch of steps
+                        out[ri].append(toks[i][row])
+                        if eos_token_id is not None and toks[i][row] == eos_token_id and row in running \
+                                and running[row][0] == ri:
+                            ended.append(row)
+                step_log.clear()
+                self.s_step.zero_()
+            return ended
+
+        try:
+            while waiting or running:
+                # admit while a row and the blocks for the whole request are free
+                while waiting and free_rows:
+                    ri = waiting[0]
+                    prompt, max_new = requests[ri]
+                    need = (len(prompt) + max_new + bs - 1) // bs
+                    if need > len(self.cache.free):
+                        if not running:
+                            raise RuntimeError(f"KV cache too small for request {ri}: {need} blocks wanted, "
+                                               f"{len(self.cache.free)} exist free with nothing running")
+                        break
+                    waiting.popleft()
+                    blocks = self.cache.allocate(need)
+                    try:
+                        ids = torch.tensor([prompt], dtype=torch.long, device=self.device)
+                        tok = int(self._prefill(ids, [blocks])[0])
+                    except Exception:
+                        self.cache.release(blocks)
+                        raise
+                    n_prefill += 1
+                    out[ri].append(tok)
+                    if max_new == 1 or tok == eos_token_id:
+                        self.cache.release(blocks)
+                        continue
+                    row = free_rows.pop()
+                    running[row] = [ri, max_new - 1, blocks]
+                    self.s_table[row] = torch.tensor(blocks + [0] * (self.max_blocks - need), dtype=torch.int32)
+                    self.s_ids[row] = tok
+                    self.s_pos[row] = len(prompt)
+                    self.s_active[row] = True
+                if not running:
+                    continue
+                self._run_decode()
+                n_steps += 1
+                step_log.append([(row, r[0]) for row, r in running.items()])
+                done = []
+                for row, r in running.items():
+                    r[1] -= 1
+                    if r[1] == 0:
+                        done.append(row)
+                if eos_token_id is not None or len(step_log) == self.s_out.shape[0]:
+                    done.extend(row for row in read_back() if row not in done)
+                for row in done:
+                    retire(row)
+            read_back()
+        finally:
+            for row in list(running):
+                retire(row)
+        if stats is not None:
+            torch.cuda.synchronize()
+            stats.update(wall_s=time.perf_counter() - t_start, decode_steps=n_steps, prefills=n_prefill,
+                         tokens=sum(len(o) for o in out))
+        return out
+

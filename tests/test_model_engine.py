@@ -176,3 +176,50 @@ def test_engine_at_qwen3_32b_widths():
     clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
     assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
     assert eng.generate(prompts, new) == got
+
+
+@pytest.mark.gpu
+def test_engine_continuous_batching():
+    """serve(): ragged prompts, more requests than batch rows, different token budgets.  Every request's
+    continuation, teacher-forced through the full-recompute forward, must be that forward's argmax wherever the
+    logits are not near-tied; rows and cache blocks are all given back; an end-of-sequence token cuts a request."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import random_awq_qwen3
+    print("engine continuous batching", flush=True)
+    model = random_awq_qwen3(TINY, seed=7, std=0.05)
+    g = torch.Generator().manual_seed(8)
+    lens = [5, 19, 33, 7, 12, 40, 3, 26, 9]
+    budgets = [6, 3, 9, 1, 12, 4, 8, 5, 7]
+    reqs = [(torch.randint(0, 512, (n,), generator=g).tolist(), m) for n, m in zip(lens, budgets)]
+    eng = LLMEngine(model, max_batch=4, max_seq_len=64, block_size=16, use_graph=True)
+    total_blocks = len(eng.cache.free)
+    st = {}
+    got = eng.serve(reqs, stats=st)
+    assert [len(o) for o in got] == budgets
+    assert len(eng.cache.free) == total_blocks and st["prefills"] == len(reqs)
+    assert st["decode_steps"] < sum(b - 1 for b in budgets), "requests must share decode steps"
+    for (prompt, _), cont in zip(reqs, got):
+        seq = torch.tensor([prompt + cont], device="cuda")
+        pos = torch.arange(seq.shape[1], device="cuda").unsqueeze(0)
+        logits = model.lm_head(model(seq, pos)).float()[0, len(prompt) - 1:-1]
+        chosen = torch.tensor(cont, device="cuda")
+        gap = logits.max(-1).values - logits.gather(-1, chosen.unsqueeze(-1)).squeeze(-1)
+        scale = logits.abs().max().item()
+        assert gap.max().item() <= 2e-2 * scale
+        top2 = logits.topk(2, dim=-1).values
+        clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
+        assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
+    # the same requests again (the captured graph and the freed blocks are reused) give the same tokens
+    assert eng.serve(reqs) == got
+    # end-of-sequence: pick a token that some request emits mid-way and check the cut
+    ri = max(range(len(got)), key=lambda i: len(got[i]))
+    eos = got[ri][len(got[ri]) // 2]
+    cut = eng.serve(reqs, eos_token_id=eos)
+    for a, b in zip(cut, got):
+        want = b[: b.index(eos) + 1] if eos in b else b
+        assert a == want
+    assert len(eng.cache.free) == total_blocks
+    # a request that can never fit is refused, not queued forever
+    small = LLMEngine(model, max_batch=2, max_seq_len=64, block_size=16, num_blocks=2, use_graph=False)
+    with pytest.raises(RuntimeError, match="KV cache too small"):
+        small.serve([(list(range(40)), 8)])
