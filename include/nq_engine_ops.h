@@ -33,12 +33,14 @@ int nq_add_rmsnorm(void* residual, const void* delta, const void* weight, void* 
  * positions[row]; q goes to q_out [rows, num_heads, head_dim], k and the untouched v go to
  * k_cache / v_cache [num_slots / block_size, num_kv_heads, block_size, head_dim] (a head's tokens of one
  * block are contiguous) at slot slots[row] = block * block_size + offset (a row whose slot is outside
- * [0, num_slots) writes no k/v).  head_dim even, <= 256.
+ * [0, num_slots) writes no k/v).  If k_out is not NULL the normalised, rotated k heads are also written
+ * densely to k_out [rows, num_kv_heads, head_dim] (what a causal prefill attention over the same rows
+ * reads).  head_dim even, <= 256.
  * Qwen3QuantizedAttention.forward, nanoquantization/models/qwen3_quantized.py:79-93;
  * RoPE.apply_rope / forward, nanoquantization/layers/rope.py:24-45. */
 int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, const void* k_weight,
                           const float* cos_sin, const int64_t* positions, const int64_t* slots,
-                          void* q_out, void* k_cache, void* v_cache, int64_t rows, int64_t num_heads,
+                          void* q_out, void* k_out, void* k_cache, void* v_cache, int64_t rows, int64_t num_heads,
                           int64_t num_kv_heads, int64_t head_dim, int64_t max_positions,
                           int64_t num_slots, int64_t block_size, float eps, int dtype, void* stream);
 

@@ -99,8 +99,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ q_weight, const uint16_t* __restrict__ k_weight,
     const float* __restrict__ cos_sin, const int64_t* __restrict__ positions, const int64_t* __restrict__ slots,
-    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache, int rows, int nh,
-    int nkv, int hd, int max_positions, int64_t num_slots, int block_size, float eps) {
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_out, uint16_t* __restrict__ k_cache,
+    uint16_t* __restrict__ v_cache, int rows, int nh, int nkv, int hd, int max_positions, int64_t num_slots,
+    int block_size, float eps) {
     const int heads = nh + 2 * nkv;
     const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (item >= (int64_t)rows * heads) return;
@@ -109,11 +110,18 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     const int64_t slot = slots[row];
     const bool slot_ok = slot >= 0 && slot < num_slots;
     uint16_t* dst;
+    uint16_t* dst2 = nullptr;   // dense copy of a normalised, rotated k head (prefill attention reads it)
     if (h < nh) {
         dst = q_out + ((int64_t)row * nh + h) * hd;
     } else if (h < nh + nkv) {
-        if (!slot_ok) return;
-        dst = k_cache + (((slot / block_size) * nkv + (h - nh)) * block_size + slot % block_size) * hd;
+        if (k_out) dst2 = k_out + ((int64_t)row * nkv + (h - nh)) * hd;
+        if (!slot_ok) {
+            if (!dst2) return;
+            dst = dst2;
+            dst2 = nullptr;
+        } else {
+            dst = k_cache + (((slot / block_size) * nkv + (h - nh)) * block_size + slot % block_size) * hd;
+        }
     } else {
         if (!slot_ok) return;
         dst = v_cache + (((slot / block_size) * nkv + (h - nh - nkv)) * block_size + slot % block_size) * hd;
@@ -165,8 +173,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
         if (i < half) {
             const float x1 = round_to<T>(round_to<T>(a[p] * r) * w1[p]);
             const float x2 = round_to<T>(round_to<T>(b[p] * r) * w2[p]);
-            dst[i] = T::from_f32(__fsub_rn(__fmul_rn(x1, cc[p]), __fmul_rn(x2, sn[p])));
-            dst[i + half] = T::from_f32(__fadd_rn(__fmul_rn(x1, sn[p]), __fmul_rn(x2, cc[p])));
+            const uint16_t y1 = T::from_f32(__fsub_rn(__fmul_rn(x1, cc[p]), __fmul_rn(x2, sn[p])));
+            const uint16_t y2 = T::from_f32(__fadd_rn(__fmul_rn(x1, sn[p]), __fmul_rn(x2, cc[p])));
+            dst[i] = y1;
+            dst[i + half] = y2;
+            if (dst2) {
+                dst2[i] = y1;
+                dst2[i + half] = y2;
+            }
         }
     }
 }
@@ -426,8 +440,8 @@ extern "C" int nq_add_rmsnorm(void* residual, const void* delta, const void* wei
 }
 
 extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, const void* k_weight, const float* cos_sin,
-                                     const int64_t* positions, const int64_t* slots, void* q_out, void* k_cache,
-                                     void* v_cache, int64_t rows, int64_t num_heads, int64_t num_kv_heads,
+                                     const int64_t* positions, const int64_t* slots, void* q_out, void* k_out,
+                                     void* k_cache, void* v_cache, int64_t rows, int64_t num_heads, int64_t num_kv_heads,
                                      int64_t head_dim, int64_t max_positions, int64_t num_slots, int64_t block_size,
                                      float eps, int dtype, void* stream) {
     const char* fn = "nq_qk_norm_rope_store";
@@ -449,12 +463,14 @@ extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, cons
     if (dtype == AWQ_F16)
         qk_norm_rope_store_kernel<F16><<<grid, block, 0, st>>>(
             (const uint16_t*)qkv, (const uint16_t*)q_weight, (const uint16_t*)k_weight, cos_sin, positions, slots,
-            (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads, (int)num_kv_heads,
+            (uint16_t*)q_out, (uint16_t*)k_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads,
+            (int)num_kv_heads,
             (int)head_dim, (int)max_positions, num_slots, (int)block_size, eps);
     else
         qk_norm_rope_store_kernel<BF16><<<grid, block, 0, st>>>(
             (const uint16_t*)qkv, (const uint16_t*)q_weight, (const uint16_t*)k_weight, cos_sin, positions, slots,
-            (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads, (int)num_kv_heads,
+            (uint16_t*)q_out, (uint16_t*)k_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads,
+            (int)num_kv_heads,
             (int)head_dim, (int)max_positions, num_slots, (int)block_size, eps);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);

@@ -104,50 +104,40 @@ class LLMEngine:
         self.eps = layers[0].input_layernorm.eps
         self.scale = float(self.hd) ** -0.5
 
-    # ---- one transformer block on the cache --------------------------------------------------------
-    def _block(self, li: int, x: torch.Tensor, pos: torch.Tensor, slots: torch.Tensor, attend):
-        """x: [b, s, hidden]; pos: [b, s]; slots: [b*s] flat cache slots of these tokens;
-        attend(q, k, v, li) -> [b, s, heads*head_dim] given this call's q [b,s,h,d], k, v [b,s,kv,d]."""
-        layer = self.model.model.layers[li]
-        attn = layer.self_attn
-        b, s, _ = x.shape
-        h = layer.input_layernorm(x)
-        qkv = self.qkv[li](h.reshape(b * s, -1))
-        q, k, v = torch.split(qkv, [self.nh * self.hd, self.nkv * self.hd, self.nkv * self.hd], dim=-1)
-        q = q.view(b, s, self.nh, self.hd)
-        k = k.view(b, s, self.nkv, self.hd)
-        v = v.view(b, s, self.nkv, self.hd)
-        q, k = attn.rope(attn.q_norm(q), attn.k_norm(k), pos)
-        blk, off = slots // self.block_size, slots % self.block_size
-        self.cache.k[li][blk, :, off] = k.reshape(b * s, self.nkv, self.hd)
-        self.cache.v[li][blk, :, off] = v.reshape(b * s, self.nkv, self.hd)
-        o = attend(q, k, v, li)
-        x = x + attn.o_proj(o).view(b, s, -1)
-        h = layer.post_attention_layernorm(x)
-        gu = self.gate_up[li](h.reshape(b * s, -1))
-        act = F.silu(gu[:, : self.inter]) * gu[:, self.inter:]
-        return x + layer.mlp.down_proj(act).view(b, s, -1)
-
     # ---- prefill: full causal attention over the prompt itself ------------------------------------
     @torch.no_grad()
     def _prefill(self, ids: torch.Tensor, tables: List[List[int]]) -> torch.Tensor:
-        """ids: [b, s] (equal-length prompts). Returns the next token of every sequence [b]."""
+        """ids: [b, s] (equal-length prompts). Returns the next token of every sequence [b].  Same kernels as
+        the decode step around the AWQ linears (which take the MFMA GEMM at these row counts); the causal
+        attention over the prompt is torch's scaled_dot_product_attention."""
         b, s = ids.shape
+        m, bs, eps = self.model.model, self.block_size, self.eps
         pos = torch.arange(s, device=self.device).unsqueeze(0).expand(b, s)
-        tbl = torch.tensor([t[: (s + self.block_size - 1) // self.block_size] for t in tables], device=self.device)
-        slots = (tbl[:, pos[0] // self.block_size] * self.block_size + pos % self.block_size).reshape(-1)
+        tbl = torch.tensor([t[: (s + bs - 1) // bs] for t in tables], device=self.device)
+        slots = (tbl[:, pos[0] // bs] * bs + pos % bs).reshape(-1).contiguous()
+        pos_flat = pos.reshape(-1).contiguous()
         gqa = self.nh != self.nkv
-
-        def attend(q, k, v, li):
-            o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
+        kvw = self.nkv * self.hd
+        x = m.embed_tokens(ids).reshape(b * s, -1)                       # residual stream [b*s, hidden]
+        delta = None
+        for li, layer in enumerate(m.layers):
+            attn = layer.self_attn
+            h = ops.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps)
+            qkv = self.qkv[li](h)
+            q, k = ops.qk_norm_rope_store(qkv, attn.q_norm.weight, attn.k_norm.weight, attn.rope.cos_sin_cache,
+                                          pos_flat, slots, self.cache.k[li], self.cache.v[li], self.nh, self.nkv,
+                                          self.hd, attn.q_norm.eps, dense_k=True)
+            v = qkv[:, -kvw:].view(b, s, self.nkv, self.hd)
+            o = F.scaled_dot_product_attention(q.view(b, s, self.nh, self.hd).transpose(1, 2),
+                                               k.view(b, s, self.nkv, self.hd).transpose(1, 2), v.transpose(1, 2),
                                                is_causal=True, enable_gqa=gqa)
-            return o.transpose(1, 2).reshape(b * s, self.nh * self.hd)
-
-        x = self.model.model.embed_tokens(ids)
-        for li in range(len(self.model.model.layers)):
-            x = self._block(li, x, pos, slots, attend)
-        x = self.model.model.norm(x[:, -1])
-        return self.model.lm_head(x).argmax(dim=-1)
+            o = o.transpose(1, 2).reshape(b * s, self.nh * self.hd)
+            h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
+            delta = layer.mlp.down_proj(ops.silu_mul(self.gate_up[li](h)))
+        last = x.view(b, s, -1)[:, -1].contiguous()
+        dlast = delta.view(b, s, -1)[:, -1].contiguous()
+        h = ops.add_rmsnorm(last, dlast, m.norm.weight, m.norm.eps)
+        return self.model.lm_head(h).argmax(dim=-1)
 
     # ---- decode: one token per sequence, attention over the paged cache --------------------------
     def _decode_step(self) -> None:

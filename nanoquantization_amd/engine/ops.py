@@ -43,8 +43,9 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
 
 def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, cos_sin: torch.Tensor,
                        positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                       num_heads: int, num_kv_heads: int, head_dim: int, eps: float) -> torch.Tensor:
-    """qkv [rows, (nh + 2 nkv) * hd]; caches [blocks, nkv, block_size, hd]; returns q [rows, nh, hd]."""
+                       num_heads: int, num_kv_heads: int, head_dim: int, eps: float, dense_k: bool = False):
+    """qkv [rows, (nh + 2 nkv) * hd]; caches [blocks, nkv, block_size, hd]; returns q [rows, nh, hd], or
+    (q, k [rows, nkv, hd]) with dense_k."""
     dev = _dev(qkv, q_weight, k_weight, cos_sin, positions, slots, k_cache, v_cache)
     rows = qkv.shape[0]
     assert qkv.shape[1] == (num_heads + 2 * num_kv_heads) * head_dim
@@ -58,12 +59,14 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torc
     assert positions.numel() == rows and slots.numel() == rows
     num_slots = k_cache.numel() // (num_kv_heads * head_dim)
     q = torch.empty(rows, num_heads, head_dim, dtype=qkv.dtype, device=dev)
+    k = torch.empty(rows, num_kv_heads, head_dim, dtype=qkv.dtype, device=dev) if dense_k else None
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().nq_qk_norm_rope_store(
             qkv.data_ptr(), q_weight.data_ptr(), k_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(),
-            slots.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), rows, num_heads, num_kv_heads,
+            slots.data_ptr(), q.data_ptr(), None if k is None else k.data_ptr(), k_cache.data_ptr(),
+            v_cache.data_ptr(), rows, num_heads, num_kv_heads,
             head_dim, cos_sin.numel() // head_dim, num_slots, block_size, eps, _lib.dtype_id(qkv.dtype), _stream()))
-    return q
+    return (q, k) if dense_k else q
 
 
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,

@@ -70,12 +70,17 @@ def test_qk_norm_rope_store(dtype, nh, nkv, hd):
     kc = torch.zeros(num_slots // bs, nkv, bs, hd, dtype=dtype, device="cuda")   # [blocks, kv heads, block, hd]
     vc = torch.zeros_like(kc)
     q = ops.qk_norm_rope_store(qkv, qw, kw, rope.cos_sin_cache, pos, slots, kc, vc, nh, nkv, hd, 1e-6)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    q2, kd = ops.qk_norm_rope_store(qkv, qw, kw, rope.cos_sin_cache, pos, slots, kc2, vc2, nh, nkv, hd, 1e-6,
+                                    dense_k=True)
+    assert torch.equal(q2, q) and torch.equal(kc2, kc) and torch.equal(vc2, vc)
 
     qr, kr, vr = torch.split(qkv, [nh * hd, nkv * hd, nkv * hd], dim=-1)
     qr = _rmsnorm_ref(qr.view(rows, 1, nh, hd), qw, 1e-6)
     kr = _rmsnorm_ref(kr.view(rows, 1, nkv, hd), kw, 1e-6)
     qr, kr = rope(qr, kr, pos.view(rows, 1))
     _close(q, qr.view(rows, nh, hd), dtype, what="q")
+    _close(kd, kr.view(rows, nkv, hd), dtype, what="dense k (every row, also the one without a slot)")
     keep = slots >= 0
     by_slot = lambda c: c.permute(0, 2, 1, 3).reshape(num_slots, nkv, hd)      # slot = block * bs + offset
     _close(by_slot(kc)[slots[keep]], kr.view(rows, nkv, hd)[keep], dtype, what="k cache")
