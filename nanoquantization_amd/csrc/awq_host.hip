@@ -58,7 +58,27 @@ int check_linear_args(const char* fn, const void* x, const int32_t* qweight, con
     return AWQ_OK;
 }
 
+static thread_local const char* g_pf_ptr = nullptr;
+static thread_local long long g_pf_bytes = 0;
+
+void take_prefetch_hint(const char** ptr, long long* bytes) {
+    *ptr = g_pf_ptr;
+    *bytes = g_pf_bytes;
+    g_pf_ptr = nullptr;
+    g_pf_bytes = 0;
+}
+
 }  // namespace awq
+
+extern "C" int awq_prefetch_hint(const void* ptr, size_t bytes) {
+    if ((reinterpret_cast<uintptr_t>(ptr) & 127u) != 0) {
+        awq::set_error("awq_prefetch_hint: the region must start on a 128-byte boundary");
+        return AWQ_ERR_INVALID_ARG;
+    }
+    awq::g_pf_ptr = static_cast<const char*>(ptr);
+    awq::g_pf_bytes = ptr ? (long long)bytes : 0;
+    return AWQ_OK;
+}
 
 extern "C" int awq_hip_version(void) { return 100; }
 

@@ -28,7 +28,7 @@ from typing import List, Optional
 import torch
 import torch.nn.functional as F
 
-from ..layers.gemm import _linear
+from ..layers.gemm import _linear, prefetch_hint
 from . import ops
 from ..models.qwen3_quantized import Qwen3QuantizedForCausalLM
 
@@ -149,16 +149,24 @@ class LLMEngine:
         ctx = (pos + 1).to(torch.int32)
         x = m.embed_tokens(self.s_ids)                                   # residual stream [B, hidden]
         delta = None
+        nl = len(m.layers)
         for li, layer in enumerate(m.layers):
             attn = layer.self_attn
+            gu_w = self.gate_up_il[li][0] if self.swiglu_ok else self.gate_up[li].qweight
             h = ops.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps)
+            # every AWQ launch also pulls the next launch's packed weights towards the Infinity Cache
+            prefetch_hint(attn.o_proj.qweight)
             q = ops.qk_norm_rope_store(self.qkv[li](h), attn.q_norm.weight, attn.k_norm.weight,
                                        attn.rope.cos_sin_cache, pos, slots, self.cache.k[li], self.cache.v[li],
                                        self.nh, self.nkv, self.hd, attn.q_norm.eps)
             o = ops.paged_attention_decode(q, self.cache.k[li], self.cache.v[li], self.s_table, ctx, self.scale)
+            prefetch_hint(gu_w)
             h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
+            prefetch_hint(layer.mlp.down_proj.qweight)
             act = (ops.awq_gemv_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
                    else ops.silu_mul(self.gate_up[li](h)))
+            if li + 1 < nl:
+                prefetch_hint(self.qkv[li + 1].qweight)
             delta = layer.mlp.down_proj(act)
         h = ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps)
         nxt = self.model.lm_head(h).argmax(dim=-1)

@@ -144,3 +144,24 @@ def test_gemv_errors():
         nq.awq_gemm(x[:, :128], *dev, 8)
     with pytest.raises(AssertionError):
         nq.awq_gemm(x, *dev, 6)       # split_k_iters must be a power of two, as in the reference
+
+
+def test_prefetch_hint_never_changes_results():
+    """A pending hint adds workgroups that only read the hinted region; y must stay bit-identical, with and
+    without K splits, and the hint must be gone after one launch."""
+    import ctypes
+    L = _lib.lib()
+    for (M, K, N) in ((1, 1024, 1024), (16, 1024, 3072), (4, 2048, 1024), (32, 3072, 1024), (1, 5120, 25600)):
+        p = random_packed(K, N, 128, "f16", seed=K + N)
+        dev = [to_dev(p["qweight"]), to_dev(p["qscales"], "f16"), to_dev(p["qzeros"])]
+        xd = to_dev(make_x(M, K, "f16", seed=M), "f16")
+        other = torch.randint(-2 ** 31, 2 ** 31 - 1, (2048, 384), dtype=torch.int32, device="cuda")
+        print(f"prefetch hint M={M} K={K} N={N}", flush=True)
+        ref = nq.awq_gemm(xd, *dev, 8)
+        nq.prefetch_hint(other)
+        got = nq.awq_gemm(xd, *dev, 8)
+        again = nq.awq_gemm(xd, *dev, 8)           # the hint was consumed
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref) and torch.equal(again, ref)
+    assert L.awq_prefetch_hint(ctypes.c_void_p(64), 1024) == 1      # not 128-byte aligned
+    assert L.awq_prefetch_hint(None, 0) == 0
