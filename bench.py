@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 # (FETCH_SIZE, then WRITE_SIZE; profiles/gemv_cfg2_sweep_hbm_traffic.txt).  Each counter is scaled by
 # what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,014 -> 2047 B per count,
 # WRITE_SIZE 64,000 -> 1024 B per count.
-MEASURED_FETCH_BYTES_PER_LAUNCH = 1065.4 * 2047.1
+MEASURED_FETCH_BYTES_PER_LAUNCH = 1492.2 * 2047.1
 MEASURED_WRITE_BYTES_PER_LAUNCH = 108.9 * 1024.0
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
@@ -145,11 +145,15 @@ def main():
         "achieved": avg_bytes / (avg_launch_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "traffic": MEASURED_FETCH_BYTES_PER_LAUNCH + MEASURED_WRITE_BYTES_PER_LAUNCH,
-        "traffic_note": "HBM bytes per launch (fetch 2.18 MB + write 0.11 MB) from rocprofv3 FETCH_SIZE / WRITE_SIZE, "
-                        "copy-calibrated; above the 1.17 MB of packed weights because a workgroup reads 64-byte row "
-                        "pieces and, with only 8-24 column tiles, the other half of a 128-byte line is often fetched "
-                        "again by another XCD's L2; the writes are split-K partials.  These launches are latency-bound "
-                        "(the variant without the re-fetch is 15-25 % slower); at the 68 MB shapes fetch = 1.05 x algorithmic",
+        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 3.05 MB + write 0.11 MB) from rocprofv3 "
+                        "FETCH_SIZE / WRITE_SIZE, copy-calibrated.  The counters sit between the L2s and the fabric "
+                        "and cannot tell Infinity Cache hits from HBM reads: 0.87 MB of the fetch is the prefetch "
+                        "(spare workgroups read the next launch's weights once to park them in the Infinity Cache, "
+                        "the consumer reads them again from there); without the prefetch the fetch is 2.18 MB "
+                        "against 1.17 MB of packed weights, because a workgroup reads 64-byte row pieces and, with "
+                        "only 8-24 column tiles, the other half of a 128-byte line is often fetched again by another "
+                        "XCD's L2; the writes are split-K partials.  These launches are latency-bound (variants "
+                        "without the re-fetch are 15-25 % slower); at the 68 MB shapes fetch = 1.05 x algorithmic",
         "avg_launch_us": avg_launch_us, "algorithmic_bytes_per_launch": avg_bytes,
         "note": "packed-weight bytes (0.5195 B/weight) / HIP-event time per launch over the timed graph replays; "
                 "0.5-1.6 MB per launch: latency-bound, see roofline_large for the HBM-bound regime",
