@@ -132,7 +132,7 @@ def main():
         # of the (small) GEMV grid pull it into the Infinity Cache (awq_prefetch_hint)
         for M in DECODE_MS:
             for i, ((qw, sc, qz), K) in enumerate(flat):
-                nq.prefetch_hint(flat[(i + 1) % len(flat)][0][0])
+                nq.prefetch_hint(*flat[(i + 1) % len(flat)][0][:2])        # qweight, qscales
                 nq.awq_gemm(xs[(M, K)], qw, sc, qz, 8)
 
     ms_graph = time_graph(sweep_step, args.steps, args.warmup)

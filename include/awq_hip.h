@@ -91,9 +91,9 @@ int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void* qscales, 
 /* Optional hint for latency-bound decode loops: the next awq_gemv / awq_linear / awq_gemv_swiglu call of
  * the calling thread that takes the staged GEMV path and leaves compute units idle also launches a few
  * spare workgroups that read [ptr, ptr + bytes) -- meant to be the packed qweight of the launch AFTER it --
- * so that that launch finds its weights in the 256 MB Infinity Cache instead of HBM.  The hint is consumed
- * (or dropped) by that one call; it never changes results.  ptr must be 128-byte aligned, NULL clears a
- * pending hint.  No reference counterpart (the reference launches each linear on its own). */
+ * so that that launch finds its weights in the 256 MB Infinity Cache instead of HBM.  Up to four regions
+ * (qweight, qscales, qzeros ...) can be pending; all are consumed (or dropped) by that one call; they never
+ * change results.  ptr must be 128-byte aligned, NULL clears the pending hints.  No reference counterpart (the reference launches each linear on its own). */
 int awq_prefetch_hint(const void* ptr, size_t bytes);
 
 /* Prefill regime, any M >= 1 (meant for M > 16): fused dequant + MFMA GEMM,

@@ -135,8 +135,14 @@ int hip_fail(const char* fn, hipError_t e);
 
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// Prefetch hint of the calling thread (awq_prefetch_hint): taken, and cleared, by the next GEMV launch.
-void take_prefetch_hint(const char** ptr, long long* bytes);
+// Prefetch hints of the calling thread (awq_prefetch_hint): taken, and cleared, by the next GEMV launch.
+constexpr int kMaxPrefetchRegions = 4;
+struct PrefetchRegions {
+    const char* ptr[kMaxPrefetchRegions];
+    long long bytes[kMaxPrefetchRegions];
+    int count;
+};
+void take_prefetch_hint(PrefetchRegions* out);
 
 // Split-K bookkeeping shared by the GEMV and GEMM kernels.  The workspace is
 //   [ kMaxSplitTiles int32 arrival counters | fp32 partials [splits][M][N] ]

@@ -460,21 +460,32 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
-    int splits, int act, int groups, const char* __restrict__ pf_ptr, long long pf_bytes) {
+    int splits, int act, int groups, PrefetchRegions pf) {
     constexpr int CH = 4;
     extern __shared__ float red[];  // staging while streaming, [WAVES][32][64] floats afterwards
     __shared__ int s_last;
     if ((int)blockIdx.x >= groups) {
         if (blockIdx.y != 0) return;   // with K splits the extra workgroups exist once per split; one set works
         // Prefetch workgroups (launched beside the compute grid on CUs a small GEMV leaves idle): touch one
-        // dword of every 128-byte line of [pf_ptr, pf_ptr + pf_bytes) -- the packed weights of the NEXT
-        // launch -- so that it finds them in the Infinity Cache instead of HBM.
-        const long long lines = pf_bytes >> 7;
+        // dword of every 128-byte line of the hinted regions -- the packed weights, scales and zeros of the
+        // NEXT launch -- so that it finds them in the Infinity Cache instead of HBM.
         const long long nthreads = (long long)(gridDim.x - groups) * blockDim.x;
+        const long long tid = (long long)(blockIdx.x - groups) * blockDim.x + threadIdx.x;
         uint32_t sink = 0;
-        for (long long l = (long long)(blockIdx.x - groups) * blockDim.x + threadIdx.x; l < lines; l += nthreads)
-            sink ^= *reinterpret_cast<const volatile uint32_t*>(pf_ptr + (l << 7));
-        if (sink == 0x9e3779b9u && pf_bytes < 0) counters[0] = 0;   // never true: keeps the loads alive
+        for (int r = 0; r < pf.count; ++r) {
+            const long long lines = pf.bytes[r] >> 7;
+            // four independent loads in flight per thread and round
+            for (long long l = tid; l < lines; l += 4 * nthreads) {
+                uint32_t v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const long long lu = l + u * nthreads;
+                    v[u] = *reinterpret_cast<const volatile uint32_t*>(pf.ptr[r] + ((lu < lines ? lu : l) << 7));
+                }
+                sink ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+            }
+        }
+        if (sink == 0x9e3779b9u && pf.count < 0) counters[0] = 0;   // never true: keeps the loads alive
         return;
     }
 
@@ -698,16 +709,19 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
         }
     }
     (void)hipGetLastError();  // do not report an earlier, unrelated failure as this launch's
-    // a pending prefetch hint rides on this launch when the compute grid leaves CUs idle
-    const char* pf_ptr = nullptr;
+    // pending prefetch hints ride on this launch when the compute grid leaves CUs idle
+    PrefetchRegions pf;
+    take_prefetch_hint(&pf);
     long long pf_bytes = 0;
+    for (int r = 0; r < pf.count; ++r) pf_bytes += pf.bytes[r];
     int pf_wgs = 0;
-    take_prefetch_hint(&pf_ptr, &pf_bytes);
-    if (pf_ptr && pf_bytes >= 128 && (long long)groups * splits < 192) {
-        const long long want = cdiv(pf_bytes >> 7, 64 * WAVES * 4);   // about 4 lines per thread
+    if (pf_bytes >= 128 && (long long)groups * splits < 192) {
+        const long long want = cdiv(pf_bytes >> 7, 64 * WAVES * 2);   // about 2 lines per thread
         const long long room = (256 - (long long)groups * splits) / splits;   // stay within one wave of workgroups
         pf_wgs = (int)(want < room ? want : room);
         if (pf_wgs < 1) pf_wgs = 1;
+    } else {
+        pf.count = 0;
     }
     hipLaunchKernelGGL(kern, dim3(groups + pf_wgs, splits), dim3(64 * WAVES), lds, stream,
                        reinterpret_cast<const uint16_t*>(x),
@@ -715,8 +729,7 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
                        reinterpret_cast<const uint16_t*>(qscales),
                        reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
-                       partials, counters, M, N, K, g / 128, cps, splits, act, groups, pf_ptr,
-                       pf_wgs ? pf_bytes : 0);
+                       partials, counters, M, N, K, g / 128, cps, splits, act, groups, pf);
     return hipGetLastError();
 }
 

@@ -58,25 +58,32 @@ int check_linear_args(const char* fn, const void* x, const int32_t* qweight, con
     return AWQ_OK;
 }
 
-static thread_local const char* g_pf_ptr = nullptr;
-static thread_local long long g_pf_bytes = 0;
+// up to kMaxPrefetchRegions pending regions per thread
+static thread_local PrefetchRegions g_pf = {};
 
-void take_prefetch_hint(const char** ptr, long long* bytes) {
-    *ptr = g_pf_ptr;
-    *bytes = g_pf_bytes;
-    g_pf_ptr = nullptr;
-    g_pf_bytes = 0;
+void take_prefetch_hint(PrefetchRegions* out) {
+    *out = g_pf;
+    g_pf.count = 0;
 }
 
 }  // namespace awq
 
 extern "C" int awq_prefetch_hint(const void* ptr, size_t bytes) {
+    if (!ptr) {
+        awq::g_pf.count = 0;
+        return AWQ_OK;
+    }
     if ((reinterpret_cast<uintptr_t>(ptr) & 127u) != 0) {
         awq::set_error("awq_prefetch_hint: the region must start on a 128-byte boundary");
         return AWQ_ERR_INVALID_ARG;
     }
-    awq::g_pf_ptr = static_cast<const char*>(ptr);
-    awq::g_pf_bytes = ptr ? (long long)bytes : 0;
+    if (awq::g_pf.count == awq::kMaxPrefetchRegions) {
+        awq::set_error("awq_prefetch_hint: at most %d regions can be pending", awq::kMaxPrefetchRegions);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    awq::g_pf.ptr[awq::g_pf.count] = static_cast<const char*>(ptr);
+    awq::g_pf.bytes[awq::g_pf.count] = (long long)bytes;
+    ++awq::g_pf.count;
     return AWQ_OK;
 }
 

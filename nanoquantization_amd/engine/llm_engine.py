@@ -152,21 +152,23 @@ class LLMEngine:
         nl = len(m.layers)
         for li, layer in enumerate(m.layers):
             attn = layer.self_attn
-            gu_w = self.gate_up_il[li][0] if self.swiglu_ok else self.gate_up[li].qweight
+            gu = self.gate_up_il[li][:2] if self.swiglu_ok else (self.gate_up[li].qweight, self.gate_up[li].qscales)
             h = ops.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps)
-            # every AWQ launch also pulls the next launch's packed weights towards the Infinity Cache
-            prefetch_hint(attn.o_proj.qweight)
+            # every AWQ launch also pulls the next launch's packed weights and scales towards the Infinity Cache
+            # (the small zero-point tensor measured as a net loss)
+            prefetch_hint(attn.o_proj.qweight, attn.o_proj.qscales)
             q = ops.qk_norm_rope_store(self.qkv[li](h), attn.q_norm.weight, attn.k_norm.weight,
                                        attn.rope.cos_sin_cache, pos, slots, self.cache.k[li], self.cache.v[li],
                                        self.nh, self.nkv, self.hd, attn.q_norm.eps)
             o = ops.paged_attention_decode(q, self.cache.k[li], self.cache.v[li], self.s_table, ctx, self.scale)
-            prefetch_hint(gu_w)
+            prefetch_hint(*gu)
             h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
-            prefetch_hint(layer.mlp.down_proj.qweight)
+            prefetch_hint(layer.mlp.down_proj.qweight, layer.mlp.down_proj.qscales)
             act = (ops.awq_gemv_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
                    else ops.silu_mul(self.gate_up[li](h)))
             if li + 1 < nl:
-                prefetch_hint(self.qkv[li + 1].qweight)
+                nq_ = self.qkv[li + 1]
+                prefetch_hint(nq_.qweight, nq_.qscales)
             delta = layer.mlp.down_proj(act)
         h = ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps)
         nxt = self.model.lm_head(h).argmax(dim=-1)

@@ -97,12 +97,15 @@ def _linear(entry: str, x, qweight, qscales, qzeros, bias, extra=()):
     return out
 
 
-def prefetch_hint(next_qweight: torch.Tensor) -> None:
-    """Tell the next decode-regime AWQ launch of this thread to also pull `next_qweight` (the packed weight of the
-    launch after it) into the Infinity Cache with workgroups it would leave idle.  Results never change."""
-    if next_qweight.device.type != "cuda" or next_qweight.data_ptr() % 128 != 0:
-        return
-    _lib.check(_lib.lib().awq_prefetch_hint(next_qweight.data_ptr(), next_qweight.numel() * next_qweight.element_size()))
+def prefetch_hint(*next_buffers: torch.Tensor) -> None:
+    """Tell the next decode-regime AWQ launch of this thread to also pull the given tensors (the packed qweight,
+    qscales, qzeros of the launch after it; at most four) into the Infinity Cache with workgroups it would leave
+    idle.  Results never change."""
+    L = _lib.lib()
+    for t in next_buffers:
+        if t.device.type != "cuda" or t.data_ptr() % 128 != 0:
+            continue
+        _lib.check(L.awq_prefetch_hint(t.data_ptr(), t.numel() * t.element_size()))
 
 
 def awq_gemm(

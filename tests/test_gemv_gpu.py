@@ -158,10 +158,15 @@ def test_prefetch_hint_never_changes_results():
         other = torch.randint(-2 ** 31, 2 ** 31 - 1, (2048, 384), dtype=torch.int32, device="cuda")
         print(f"prefetch hint M={M} K={K} N={N}", flush=True)
         ref = nq.awq_gemm(xd, *dev, 8)
-        nq.prefetch_hint(other)
+        nq.prefetch_hint(other, dev[1], dev[2])
         got = nq.awq_gemm(xd, *dev, 8)
         again = nq.awq_gemm(xd, *dev, 8)           # the hint was consumed
         torch.cuda.synchronize()
         assert torch.equal(got, ref) and torch.equal(again, ref)
     assert L.awq_prefetch_hint(ctypes.c_void_p(64), 1024) == 1      # not 128-byte aligned
+    assert L.awq_prefetch_hint(None, 0) == 0
+    buf = torch.zeros(1024, dtype=torch.uint8, device="cuda")
+    for _ in range(4):
+        assert L.awq_prefetch_hint(buf.data_ptr(), 1024) == 0
+    assert L.awq_prefetch_hint(buf.data_ptr(), 1024) == 1           # a fifth pending region is refused
     assert L.awq_prefetch_hint(None, 0) == 0
