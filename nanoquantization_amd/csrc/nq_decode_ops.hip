@@ -196,10 +196,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
 // groups, then waves (LDS), then splits (fp32 partials + a second kernel).
 constexpr float kNegBig = -3.0e38f;
 
-struct SoftState {
-    float m, l;
-};
-
 template <typename T, int G, int HD, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
