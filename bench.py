@@ -97,6 +97,8 @@ def main():
     ap.add_argument("--layers", type=int, default=64, help="distinct weight copies of one block per step")
     ap.add_argument("--quick", action="store_true", help="skip the extra (non-headline) measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cfg5", action="store_true",
+                    help="also run the Qwen3-32B-architecture section (about 75 GB of device memory, a minute)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the AWQ linear path has no multi-GPU part); "
@@ -267,6 +269,40 @@ def main():
             torch.cuda.empty_cache()
         except Exception as e:  # the headline must still be printed
             out["e2e_qwen3_0p6b"] = {"error": repr(e)}
+
+    if args.cfg5:
+        # ---------------- extra: cfg5, Qwen3-32B architecture: batch-64 decode at 2048 context, 4096-token prefill
+        try:
+            from nanoquantization_amd.engine import LLMEngine
+            from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+            cfg = dict(QWEN3_32B, max_position_embeddings=8192)
+            model = random_awq_qwen3(cfg, seed=0, device=dev, dtype=torch.bfloat16)
+            B, P, NEW = 64, 2048, 17
+            eng = LLMEngine(model, max_batch=B, max_seq_len=P + 64, block_size=64, use_graph=True)
+            prompts = torch.randint(0, cfg["vocab_size"], (B, P), generator=torch.Generator().manual_seed(1)).tolist()
+            eng.generate(prompts, 4)
+            st = {}
+            eng.generate(prompts, NEW, stats=st)
+            del eng
+            torch.cuda.empty_cache()
+            eng1 = LLMEngine(model, max_batch=1, max_seq_len=4096 + 64, block_size=64, use_graph=False)
+            one = torch.randint(0, cfg["vocab_size"], (1, 4096), generator=torch.Generator().manual_seed(2)).tolist()
+            eng1.generate(one, 2)
+            st1 = {}
+            eng1.generate(one, 2, stats=st1)
+            out["cfg5_qwen3_32b"] = {
+                "workload": "Qwen3-32B architecture (64 layers, hidden 5120, 64 q / 8 kv heads, intermediate 25600), random AWQ "
+                            "g=128 weights, bf16: batch 64 decode at 2048 context; one 4096-token prefill",
+                "decode_tok_per_s": round(B * st["decode_steps"] / st["decode_s"], 1),
+                "decode_ms_per_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 2),
+                "batch_prefill_tok_per_s": round(B * P / st["prefill_s"], 1),
+                "prefill_4096_s": round(st1["prefill_s"], 4),
+                "prefill_4096_tok_per_s": round(4096 / st1["prefill_s"], 1),
+            }
+            del eng1, model
+            torch.cuda.empty_cache()
+        except Exception as e:
+            out["cfg5_qwen3_32b"] = {"error": repr(e)}
 
     # ---------------- CPU baseline: the reference's path restated on host tensors (bounded sample) ----------
     if not args.no_cpu:
