@@ -205,9 +205,10 @@ static const GemmVariant kGemmVariants[] = {
     {"256x256w8", 256, 256, 8}, {"128x256w8", 128, 256, 8}, {"128x128", 128, 128, 4},
     {"64x256", 64, 256, 4},     {"32x256", 32, 256, 4},     {"64x128", 64, 128, 4},
     {"256x256", 256, 256, 4},   {"128x256", 128, 256, 4},   {"256x128w8", 256, 128, 8},
-    {"256x256p", 256, 256, 8},  // the software-pipelined kernel of awq_gemm_pipe.hip
+    {"256x256p", 256, 256, 8},   // the software-pipelined kernel of awq_gemm_pipe.hip, every tile cut split_k ways
+    {"256x256pt", 256, 256, 8},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
 };
-constexpr int kPipeVariant = 9;
+constexpr int kPipeVariant = 9, kPipeTailVariant = 10;
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 template <typename T, int BM, int BN, int WM, int WN>
@@ -252,7 +253,8 @@ static int gemm_effective_splits(int64_t K, int split_k) {
 }
 
 static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k) {
-    const GemmVariant& gv = kGemmVariants[variant];
+    if (variant == kPipeVariant || variant == kPipeTailVariant)
+        return pipe_ws_bytes(make_pipe_plan(M, N, K, split_k, variant == kPipeTailVariant));
     const int splits = gemm_effective_splits(K, split_k);
     if (splits <= 1) return 0;
     return kCounterBytes + (size_t)splits * M * N * sizeof(float);
@@ -275,6 +277,18 @@ static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_
     int64_t s = 1;
     if (tiles < kCUs) s = kCUs / tiles;
     const int64_t max_s = K / kBK / 8 > 0 ? K / kBK / 8 : 1;  // at least 8 K-steps per split
+    if (v == kPipe8 && tiles > kCUs && tiles % kCUs != 0) {
+        // The last round would leave CUs idle: cut only its R tiles into s pieces each.  The pieces take
+        // ceil(R*s / CUs) rounds of (steps/s + a fixed cost of about 5 steps for prologue and partial store);
+        // take the s that minimises it, if that saves a tenth of a round at least.
+        const int64_t R = tiles % kCUs, steps = K / kBK;
+        int64_t best_s = 1, best_t = steps;
+        for (int64_t c = 2; c <= 16 && c <= max_s; ++c) {
+            const int64_t t = cdiv(R * c, kCUs) * (cdiv(steps, c) + 5);
+            if (t < best_t) best_t = t, best_s = c;
+        }
+        if (best_s > 1 && best_t * 10 <= steps * 9) v = kPipeTailVariant, s = best_s;
+    }
     if (s > max_s) s = max_s;
     if (s > 16) s = 16;
     if (s < 1) s = 1;
@@ -334,8 +348,9 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         AWQ_GEMM_CASE(7, 128, 256, 2, 2)
         AWQ_GEMM_CASE(8, 256, 128, 4, 2)
         case kPipeVariant:
+        case kPipeTailVariant:
             e = launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
-                                 workspace, split_k, s);
+                                 workspace, split_k, variant == kPipeTailVariant, s);
             break;
     }
 #undef AWQ_GEMM_CASE

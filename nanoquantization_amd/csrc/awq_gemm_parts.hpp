@@ -138,9 +138,35 @@ inline hipError_t launch_splitk_reduce(int dtype, const float* partials, const v
     return hipGetLastError();
 }
 
+// Work split of the 256 x 256 pipelined kernel: `full_tiles` output tiles are computed whole by one
+// workgroup each; the `tail_tiles` after them (tile index = m-tile * tiles_n + n-tile) are cut into `splits`
+// K slices of `iters_per_split` 64-row steps whose fp32 partials a second kernel adds.
+struct PipePlan {
+    int tiles_n, full_tiles, tail_tiles, splits, iters_per_split;
+};
+
+// tail_only = false: every tile is cut `split_k` ways (none if that leaves one slice).
+// tail_only = true: only the tiles beyond the last full round of 256 workgroups are cut.
+inline PipePlan make_pipe_plan(int64_t M, int64_t N, int64_t K, int split_k, bool tail_only) {
+    PipePlan p;
+    p.tiles_n = (int)cdiv(N, 256);
+    const int tiles = (int)(cdiv(M, 256) * p.tiles_n);
+    const int total_iters = (int)(K / 64);
+    p.iters_per_split = (int)cdiv(total_iters, split_k);
+    p.splits = (int)cdiv(total_iters, p.iters_per_split);
+    p.tail_tiles = p.splits <= 1 ? 0 : (tail_only ? tiles % 256 : tiles);
+    p.full_tiles = tiles - p.tail_tiles;
+    if (p.tail_tiles == 0) p.splits = 1;
+    return p;
+}
+
+inline size_t pipe_ws_bytes(const PipePlan& p) {
+    return p.tail_tiles == 0 ? 0 : kCounterBytes + ((size_t)p.splits * p.tail_tiles << 18);
+}
+
 // awq_gemm_pipe.hip: the 256 x 256 software-pipelined kernel (same arguments as the tiled launcher).
 hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
-                            void* workspace, int split_k, hipStream_t stream);
+                            void* workspace, int split_k, bool tail_only, hipStream_t stream);
 
 }  // namespace awq

@@ -103,8 +103,7 @@ template <typename T, int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
     const uint32_t* __restrict__ qzeros, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
-    float* __restrict__ partials, int M, int N, int K, int g, int iters_per_split,
-    int splits) {
+    float* __restrict__ partials, int M, int N, int K, int g, PipePlan plan) {
     constexpr int BM = 256, BN = 256, NW = WM * WN, NT = 64 * NW;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int UR = kPBK * 32 / NT;   // k rows of one word column per lane and step: 8 or 4
@@ -117,12 +116,21 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const int split = blockIdx.z;
+    // Workgroups [0, full_tiles) own a whole output tile each; the rest share the tail tiles, `splits`
+    // K slices per tile, slice-major.  The hardware hands workgroups out in index order, so the short
+    // tail pieces fill the CUs that the last full round would leave idle.
+    int tile = blockIdx.x, split = 0;
+    const bool whole = (int)blockIdx.x < plan.full_tiles;
+    if (!whole) {
+        const int r = blockIdx.x - plan.full_tiles;
+        split = r / plan.tail_tiles;
+        tile = plan.full_tiles + (r - split * plan.tail_tiles);
+    }
+    const int m0 = (tile / plan.tiles_n) * BM, n0 = (tile % plan.tiles_n) * BN;
     const int words = N >> 3;
     const int total_iters = K / kPBK;
-    const int it_begin = split * iters_per_split;
-    const int it_end = min(it_begin + iters_per_split, total_iters);
+    const int it_begin = whole ? 0 : split * plan.iters_per_split;
+    const int it_end = whole ? total_iters : min(it_begin + plan.iters_per_split, total_iters);
 
     // ---- A: NDMA direct-to-LDS loads per wave and step; load i of wave w fills slots
     //      (NDMA*w + i)*64 + lane, i.e. rows 8*(NDMA*w + i) + lane/8, whose chunk at position lane%8
@@ -271,7 +279,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
             if (it + 1 < it_end) step(it + 1, 1, r0, r1);
         }
     }
-    if (splits == 1) {
+    if (whole) {
         // Direct store through LDS: the MFMA layout gives a lane one column of a 32 x 32 tile, i.e.
         // 2-byte stores; staged per wave as [32 rows][32*TN columns] the same data leaves as 16-byte
         // stores, 4*TN lanes to a row segment.  The staging area is private to the wave and LDS
@@ -302,18 +310,58 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
             }
         }
     } else {
-        gemm_epilogue<T, BM, BN, TM, TN, NT>(acc, bias, y, partials, M, N, m0, n0, wm0, wn0, split, splits);
+        // fp32 partial of this K slice, tile-compact: [slice][tail tile][256][256].  Rows and columns past
+        // M and N are stored too (they stay inside the tile's slot); the reduction pass masks them.
+        float* slot = partials + ((size_t)(split * plan.tail_tiles + (tile - plan.full_tiles)) << 16);
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = wm0 + a * 32 + (v >> 2) * 8 + kb2 * 4 + (v & 3);
+                    slot[row * BN + wn0 + b * 32 + li] = acc[a][b][v];   // 32 lanes = one 128-byte line
+                }
     }
+}
+
+// Second pass over the tail tiles: y = dtype(sum over K slices, in slice order, of the fp32 partials (+ bias)).
+// 32 workgroups per tile; a thread owns 8 consecutive columns of one row.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __restrict__ partials,
+                                                               const uint16_t* __restrict__ bias,
+                                                               uint16_t* __restrict__ y, int M, int N, PipePlan plan) {
+    const int r = blockIdx.x >> 5;
+    const int vec = ((blockIdx.x & 31) << 8) + threadIdx.x;
+    const int row = vec >> 5, col = (vec & 31) << 3;
+    const int tile = plan.full_tiles + r;
+    const int m = (tile / plan.tiles_n) * 256 + row, n = (tile % plan.tiles_n) * 256 + col;
+    if (m >= M || n >= N) return;
+    const float* p = partials + ((size_t)r << 16) + row * 256 + col;
+    const size_t plane = (size_t)plan.tail_tiles << 16;
+    f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+    for (int s = 0; s < plan.splits; ++s) {
+        lo += *reinterpret_cast<const f32x4*>(p + s * plane);
+        hi += *reinterpret_cast<const f32x4*>(p + s * plane + 4);
+    }
+    float out[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (bias) {
+        const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + n);
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
+    }
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+    *reinterpret_cast<u32x4*>(y + (size_t)m * N + n) = o;
 }
 
 template <typename T, int WM, int WN>
 hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
                        const void* bias, void* y, int M, int N, int K, int g, void* workspace, int split_k,
-                       hipStream_t stream) {
-    const int tiles_m = (int)cdiv(M, 256), tiles_n = (int)cdiv(N, 256);
-    const int total_iters = K / kPBK;
-    const int ips = (int)cdiv(total_iters, split_k);
-    const int splits = (int)cdiv(total_iters, ips);
+                       bool tail_only, hipStream_t stream) {
+    const PipePlan plan = make_pipe_plan(M, N, K, split_k, tail_only);
     float* partials =
         workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes) : nullptr;
     const size_t lds = (size_t)2 * (8 * 256 + 8 * 256) * 16;  // 128 KiB
@@ -326,24 +374,27 @@ hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscale
         raised = true;
     }
     (void)hipGetLastError();
-    hipLaunchKernelGGL(kern, dim3(tiles_n, tiles_m, splits), dim3(64 * WM * WN), lds, stream,
+    hipLaunchKernelGGL(kern, dim3(plan.full_tiles + plan.tail_tiles * plan.splits), dim3(64 * WM * WN), lds, stream,
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
-                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, M, N, K, g, ips,
-                       splits);
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, M, N, K, g, plan);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || splits == 1) return e;
-    return launch_splitk_reduce(T::id, partials, bias, y, M, N, splits, stream);
+    if (e != hipSuccess || plan.tail_tiles == 0) return e;
+    hipLaunchKernelGGL(gemm_tail_reduce_kernel<T>, dim3(plan.tail_tiles * 32), dim3(256), 0, stream, partials,
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, plan);
+    return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
-                            void* workspace, int split_k, hipStream_t stream) {
+                            void* workspace, int split_k, bool tail_only, hipStream_t stream) {
     return dtype == AWQ_F16
-               ? launch_pipe<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream)
-               : launch_pipe<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, stream);
+               ? launch_pipe<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, tail_only,
+                                        stream)
+               : launch_pipe<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, tail_only,
+                                         stream);
 }
 
 }  // namespace awq

@@ -88,6 +88,34 @@ def test_gemm_bias_and_determinism(dtype):
     assert torch.count_nonzero(awq_gemm_variant(torch.zeros_like(xd), *dev, 2, 4)) == 0
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_tail_tiles_split(dtype):
+    # 9 x 30 = 270 tiles of 256 x 256 (ragged in M and N): 256 whole tiles and a tail of 14 whose K range is cut;
+    # the mixed launch must agree with the oracle, with the uncut launch bit for bit where no cut applies,
+    # and be bit-stable
+    L = _lib.lib()
+    names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
+    tail, whole = names.index("256x256pt"), names.index("256x256p")
+    M, K, N = 2300, 256, 7672
+    p = random_packed(K, N, 128, dtype, seed=95)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    xb = make_x(M, K, dtype, seed=96)
+    xd = to_dev(xb, dtype)
+    bias = np.linspace(-1, 1, N).astype(np.float32)
+    bd = to_dev(o.to_bits16(bias, dtype), dtype)
+    y1 = awq_gemm_variant(xd, *dev, whole, 1, bias=bd)
+    _check(y1, xb, p, dtype, o.to_dtype_f32(bias, dtype))
+    for split in (2, 4):
+        print(f"gemm tail split={split} {dtype}", flush=True)
+        y = awq_gemm_variant(xd, *dev, tail, split, bias=bd)
+        torch.cuda.synchronize()
+        _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
+        assert torch.equal(y, awq_gemm_variant(xd, *dev, tail, split, bias=bd))
+        # tiles 0..255 in n-fastest order: tile rows 0..7 entirely (8 x 30 = 240) and 16 tiles of row 8
+        assert torch.equal(y[:2048], y1[:2048])
+        assert torch.equal(y[2048:, :16 * 256], y1[2048:, :16 * 256])
+
+
 def test_gemm_prefill_full_size_bf16():
     # Qwen3-8B MLP gate/up at M=512, its real size (oracle: numpy float64 matmul, a few seconds)
     print("gemm full size M=512 4096x12288 bf16", flush=True)
