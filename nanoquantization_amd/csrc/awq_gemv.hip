@@ -40,6 +40,8 @@
 // through LDS in a fixed order; workgroups of different K-splits publish fp32
 // partials and the last one to arrive (an arrival counter per tile) adds them
 // in split order, so results are bit-stable run to run.
+#include <type_traits>
+
 #include "awq_common.hpp"
 
 namespace awq {
@@ -168,6 +170,63 @@ __device__ __forceinline__ void compute_chunk(const Chunk<V, CH, MT>& d, f32x4 (
     }
 }
 
+// The same for two of the four bytes of every word (bytes 2*BH and 2*BH + 1, i.e. the even output columns of
+// a word for BH = 0 and the odd ones for BH = 1): acc[mt][2*bi + h][r] is output row 16*mt + 4*kb + r,
+// column {0,2,4,6}[2*bi + h] + BH of the lane's word.  Two waves, one per half, split a column tile without
+// unpacking anything twice.
+template <typename T, int CH, int MT, int BH>
+__device__ __forceinline__ void compute_chunk_bytes(const Chunk<1, CH, MT>& d, f32x4 (&acc)[MT][4]) {
+    const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
+    const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+    const AndOr emb_lo(Embed<T>::kMaskLo, Embed<T>::kMagicLo), emb_hi(Embed<T>::kMaskHi, Embed<T>::kMagicHi);
+    f32x4 dones[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        dones[mt] = zero4;
+#pragma unroll
+        for (int s = 0; s < CH; ++s) dones[mt] = T::mfma16(d.xa[s][mt], ones, dones[mt]);
+    }
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi) {
+        constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
+        const int b = 2 * BH + bi;
+        f32x4 dlo[MT], dhi[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) dlo[mt] = dhi[mt] = zero4;
+#pragma unroll
+        for (int s = 0; s < CH; ++s) {
+            u32x4 flo, fhi;
+#pragma unroll
+            for (int rp = 0; rp < 4; ++rp) {
+                const uint32_t p = __builtin_amdgcn_perm(d.w[s][2 * rp + 1], d.w[s][2 * rp],
+                                                         0x0c000c00u | (uint32_t)b | ((4u + b) << 16));
+                flo[rp] = emb_lo(Embed<T>::pre_lo(p));
+                fhi[rp] = emb_hi(Embed<T>::pre_hi(p));
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                dlo[mt] = T::mfma16(d.xa[s][mt], flo, dlo[mt]);
+                dhi[mt] = T::mfma16(d.xa[s][mt], fhi, dhi[mt]);
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int c = h ? kHiCol[b] : kLoCol[b];
+            const float mul = h ? Embed<T>::kMulHi : Embed<T>::kMulLo;
+            const float off = h ? Embed<T>::kOffHi : Embed<T>::kOffLo;
+            const float zf = (float)((d.zw >> nibble_shift(c)) & 0xFu) * mul + off;
+            const uint32_t pair = d.sv[0][c >> 1];
+            const float sc = T::to_f32((uint16_t)((c & 1) ? (pair >> 16) : (pair & 0xFFFFu))) * (1.f / mul);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const f32x4 dq = h ? dhi[mt] : dlo[mt];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[mt][2 * bi + h][r] += sc * (dq[r] - zf * dones[mt][r]);
+            }
+        }
+    }
+}
+
 // A workgroup is WN x WK waves: wave w works on column tile (group*WN + w % WN)
 // and K sub-slice w / WN.  Sum the WK waves of each column tile through LDS
 // (fixed order), then either store y (splits == 1) or publish this split's
@@ -200,7 +259,8 @@ __device__ __forceinline__ void swiglu_store(const float (&out)[8], uint16_t* __
     }
 }
 
-template <typename T, int V, int WN, int WK>
+// kPlain: the partials are read by a later kernel, not by a concurrent workgroup: ordinary stores do.
+template <typename T, int V, int WN, int WK, bool kPlain = false>
 __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_base, float* red, int lane,
                                                   int wave, int group, int split, int splits,
                                                   const uint16_t* __restrict__ bias,
@@ -263,8 +323,13 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
                 *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
             } else {
                 float* p = partials + ((size_t)split * M + m) * N + n0;
-                publish_f32x4(p, f32x4{out[0], out[1], out[2], out[3]});
-                publish_f32x4(p + 4, f32x4{out[4], out[5], out[6], out[7]});
+                if constexpr (kPlain) {
+                    *reinterpret_cast<f32x4*>(p) = f32x4{out[0], out[1], out[2], out[3]};
+                    *reinterpret_cast<f32x4*>(p + 4) = f32x4{out[4], out[5], out[6], out[7]};
+                } else {
+                    publish_f32x4(p, f32x4{out[0], out[1], out[2], out[3]});
+                    publish_f32x4(p + 4, f32x4{out[4], out[5], out[6], out[7]});
+                }
             }
         }
     }
@@ -615,6 +680,213 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
                                 counters, M, N, act);
 }
 
+// ---- data path 3: a workgroup of eight waves shares one staged chunk --------------------------
+// For 17..64 rows the activation chunk (MT*16 rows x 128 k = 4*MT KiB) is as large as the weights of a
+// column tile; staged once per workgroup instead of once per wave it leaves room for DEPTH buffers, i.e.
+// DEPTH-1 chunks (4 x 8 KiB of weights each) in flight while one is multiplied.  A workgroup owns 512
+// columns (four column tiles) and a K range; nothing is reduced inside it.
+//   buffer = [x: 4 steps x (MT*16 rows x 64 B)] [tile 0..3: 8 KiB weights + 512 B zeros/scales]
+// Waves wn and wn + 4 work on the same column tile and the same rows, one on bytes 0-1 of every word
+// (even output columns), the other on bytes 2-3 (odd columns).  Nothing is unpacked or scaled twice, each
+// wave holds half the accumulators, and every SIMD has two waves.  What bounds this regime is the vector
+// ALU port (one instruction per SIMD every four cycles: about 270 unpack, 140 scale/zero and 2 x 144 MFMA
+// issue slots per 128 x 128 weights at 64 rows), not the memory.
+// At the end the two halves exchange fragments through LDS so that each stores whole words of half the rows.
+__host__ __device__ constexpr int wide_buf_bytes(int MT) { return 4096 * MT + 4 * 8704; }
+
+template <typename T, int DEPTH, int MT>
+__global__ __launch_bounds__(512) void gemv_wide_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
+    const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
+    int M, int N, int K, int chunks_per_group, int chunks_per_split, int splits, int act) {
+    constexpr int CH = 4, WN = 4, HMT = MT / 2;
+    static_assert(DEPTH >= 2 && DEPTH <= 3, "two or three staging buffers");
+    static_assert(MT == 2 || MT == 4, "m-tiles per workgroup");
+    extern __shared__ float red[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave & 3, bh = wave >> 2;
+    const int j = lane & 15, kb = lane >> 4;
+    const int words = N >> 3;
+    const int group = blockIdx.x, split = blockIdx.y;
+    const int tile = group * WN + wn;   // host guarantees N % 512 == 0
+
+    const int total_chunks = K / 128;
+    const int c0 = split * chunks_per_split;
+    const int c1 = min(c0 + chunks_per_split, total_chunks);
+
+    constexpr int buf_bytes = wide_buf_bytes(MT);
+    constexpr int x_step = 1024 * MT;
+    char* stage = reinterpret_cast<char*>(red);
+    const int w_off = 4096 * MT + wn * 8704, zs_off = w_off + 8192;
+
+    const int dq = lane & 3, dsl = lane >> 2;
+    uint32_t wsrc[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int slot = h * 16 + dsl;
+        wsrc[h] = (uint32_t)((slot & 3) * 8 + (slot >> 2)) * (uint32_t)words + (uint32_t)(tile * 16 + dq * 4);
+    }
+    // x: the 4*MT (step, m-tile) pieces of 16 rows x 64 B are dealt to the 8 waves, HMT each
+    int x_s[HMT], x_mt[HMT];
+    uint32_t xsrc[HMT];
+#pragma unroll
+    for (int i = 0; i < HMT; ++i) {
+        const int o = wave * HMT + i;
+        x_s[i] = o / MT;
+        x_mt[i] = o % MT;
+        xsrc[i] = (uint32_t)min(16 * x_mt[i] + (lane >> 2), M - 1) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
+    }
+    const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
+    const bool zs_lane = lane < 16;
+
+    constexpr int kDmaOps = CH + HMT + 1;   // per wave and chunk
+    auto issue_dma = [&](int c, int buf) {
+        const int row0 = c * 128;
+        char* base = stage + buf * buf_bytes;
+        uint32_t* w_lds = reinterpret_cast<uint32_t*>(base + w_off);
+#pragma unroll
+        for (int i = 0; i < CH / 2; ++i) {
+            const int s = bh * (CH / 2) + i;
+            const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
+                                                 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < HMT; ++i)
+            __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + x_s[i] * 32) + xsrc[i]),
+                                             AWQ_LPTR(base + x_s[i] * x_step + x_mt[i] * 1024), 16, 0, 0);
+        if (zs_lane) {
+            const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
+            if (bh == 0)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(qzeros + (size_t)gi * words + zsrc),
+                                                 AWQ_LPTR(base + zs_off), 4, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(scales + ((size_t)gi * words + zsrc) * 8),
+                                                 AWQ_LPTR(base + zs_off + 64), 16, 0, 0);
+        }
+    };
+
+    const int w_rd_off = w_off + (kb * 16 + j) * 4;
+    int x_rd_off[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) x_rd_off[mt] = ((16 * mt + j) * 4 + kb) * 16;
+    const int z_rd_off = zs_off + j * 4;
+    const int s_rd_off = zs_off + 64 + j * 16;
+
+    auto run = [&](auto half) {
+        constexpr int BH = decltype(half)::value;
+        f32x4 acc[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int f = 0; f < 4; ++f) acc[mt][f] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (c0 + d < c1) issue_dma(c0 + d, d);
+        int buf = 0;
+        for (int c = c0; c < c1; ++c) {
+            const int newer = min(c1 - 1 - c, DEPTH - 2);
+            if (newer == 0) __builtin_amdgcn_s_waitcnt(0x0F70);                                   // vmcnt(0)
+            else __builtin_amdgcn_s_waitcnt(0x0F70 | (kDmaOps & 15) | ((kDmaOps >> 4) << 14));    // vmcnt(kDmaOps)
+            asm volatile("" ::: "memory");
+            // every wave's share of the chunk is in LDS, and every wave is done reading the buffer of chunk c-1.
+            // A bare barrier: __syncthreads() would first wait for every outstanding load, i.e. for the chunks
+            // in flight too; the LDS itself needs no fence (DMA data is there once vmcnt has counted it).
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if (c + DEPTH - 1 < c1) issue_dma(c + DEPTH - 1, buf == 0 ? DEPTH - 1 : buf - 1);
+            const char* base = stage + buf * buf_bytes;
+            const uint32_t* w_rd = reinterpret_cast<const uint32_t*>(base + w_rd_off);
+            Chunk<1, CH, MT> d;
+#pragma unroll
+            for (int s = 0; s < CH; ++s) {
+#pragma unroll
+                for (int r = 0; r < 8; ++r) d.w[s][r] = w_rd[s * 512 + r * 64];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    d.xa[s][mt] = *reinterpret_cast<const u32x4*>(base + x_rd_off[mt] + s * x_step);
+            }
+            d.zw = *reinterpret_cast<const uint32_t*>(base + z_rd_off);
+            d.sv[0] = *reinterpret_cast<const u32x4*>(base + s_rd_off);
+            // no wait here: this buffer is overwritten only after the next barrier, which a wave reaches
+            // with every read consumed
+            buf = (buf + 1 == DEPTH) ? 0 : buf + 1;
+            compute_chunk_bytes<T, CH, MT, BH>(d, acc);
+        }
+        // Exchange: this wave stores m-tiles BH*HMT .. and sends its fragments of the other m-tiles to its
+        // partner (wave ^ 4).  xch[wave][(ml*4 + f)*4 + r][lane]
+        __syncthreads();   // staging is free
+        float* xch = red;
+        constexpr int PER_WAVE = HMT * 16 * 64;
+#pragma unroll
+        for (int ml = 0; ml < HMT; ++ml)
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    xch[wave * PER_WAVE + ((ml * 4 + f) * 4 + r) * 64 + lane] = acc[(1 - BH) * HMT + ml][f][r];
+        __syncthreads();
+#pragma unroll
+        for (int ml = 0; ml < HMT; ++ml) {
+            const int mt = BH * HMT + ml;
+            f32x4 acc8[8];
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+                acc8[2 * f + BH] = acc[mt][f];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc8[2 * f + 1 - BH][r] = xch[(wave ^ 4) * PER_WAVE + ((ml * 4 + f) * 4 + r) * 64 + lane];
+            }
+            if (16 * mt < M)
+                gemv_reduce_store<T, 1, WN, 1, true>(acc8, 16 * mt, red, lane, wn, group, split, splits, bias, y,
+                                                     partials, M, N, act);
+        }
+    };
+    if (bh == 0) run(std::integral_constant<int, 0>{});
+    else run(std::integral_constant<int, 1>{});
+}
+
+// Second pass of a K-split wide GEMV: y = epilogue(sum over splits, in split order, of partials [splits][M][N]).
+// A thread owns one word (8 columns) of one row; with the gated epilogue neighbouring threads hold a gate word
+// and its up word.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_wide_reduce_kernel(const float* __restrict__ partials,
+                                                               const uint16_t* __restrict__ bias,
+                                                               uint16_t* __restrict__ y, int M, int N, int splits,
+                                                               int act) {
+    const int words = N >> 3;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= M * words) return;   // words is even: a gate word and its up word leave together
+    const int m = idx / words, wc = idx - m * words;
+    const size_t n0 = (size_t)wc * 8;
+    const size_t plane = (size_t)M * N;
+    const float* p = partials + (size_t)m * N + n0;
+    f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+    for (int s = 0; s < splits; ++s) {
+        lo += *reinterpret_cast<const f32x4*>(p + s * plane);
+        hi += *reinterpret_cast<const f32x4*>(p + s * plane + 4);
+    }
+    float out[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (act) {
+        swiglu_store<T>(out, y, m, N, n0);
+        return;
+    }
+    if (bias) {
+        const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
+    }
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+    *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
+}
+
 // ---- host side -------------------------------------------------------------
 struct GemvVariant {
     const char* name;
@@ -623,6 +895,7 @@ struct GemvVariant {
     int wn;     // waves side by side along N (DMA variants), 1 otherwise
     int depth;  // DMA staging buffers per wave (DMA variants), 0 otherwise
     int mt;     // tiles of 16 activation rows: M <= 16 * mt
+    bool wide;  // a workgroup of eight waves shares one staged chunk (gemv_wide_kernel)
 };
 static const GemvVariant kGemvVariants[] = {
     {"v1w4p", 1, 4, true, 1, 0, 1},  {"v1w8p", 1, 8, true, 1, 0, 1},   {"v2w4", 2, 4, false, 1, 0, 1},
@@ -635,6 +908,9 @@ static const GemvVariant kGemvVariants[] = {
     {"dma2x4d1", 1, 8, false, 2, 1, 1},  {"dma2x4d2", 1, 8, false, 2, 2, 1},  {"dma1x1d1", 1, 1, false, 1, 1, 1},
     {"dma1x2d2", 1, 2, false, 1, 2, 1},
     {"dma1x4d1m2", 1, 4, false, 1, 1, 2}, {"dma1x8d1m2", 1, 8, false, 1, 1, 2}, {"dma1x4d1m4", 1, 4, false, 1, 1, 4},
+    // shared staged chunk, eight waves as 4 column tiles x 2 byte halves: wide d<DEPTH> m<MT>
+    {"wided3m4", 1, 8, false, 4, 3, 4, true}, {"wided2m4", 1, 8, false, 4, 2, 4, true},
+    {"wided3m2", 1, 8, false, 4, 3, 2, true}, {"wided2m2", 1, 8, false, 4, 2, 2, true},
 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = 10;
@@ -733,6 +1009,41 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     return hipGetLastError();
 }
 
+template <typename T, int DEPTH, int MT>
+static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
+                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
+                                   int g, void* workspace, int split_k, hipStream_t stream, int act) {
+    const int groups = N / 512;
+    const int total_chunks = K / 128;
+    const int cps = (int)cdiv(total_chunks, split_k);
+    const int splits = (int)cdiv(total_chunks, cps);
+    float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes)
+                                : nullptr;
+    constexpr size_t lds = (size_t)DEPTH * wide_buf_bytes(MT);
+    static_assert(lds <= 160 * 1024 - 1024, "staging buffers exceed the LDS");
+    auto kern = gemv_wide_kernel<T, DEPTH, MT>;
+    static bool raised = false;  // once per process and instantiation
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    (void)hipGetLastError();
+    PrefetchRegions pf;
+    take_prefetch_hint(&pf);   // this kernel fills the chip; a pending hint is dropped
+    hipLaunchKernelGGL(kern, dim3(groups, splits), dim3(512), lds, stream,
+                       reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
+                       reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials,
+                       M, N, K, g / 128, cps, splits, act);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || splits == 1) return e;
+    hipLaunchKernelGGL(gemv_wide_reduce_kernel<T>, dim3((unsigned)cdiv((int64_t)M * (N / 8), 256)), dim3(256), 0, stream, partials,
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, splits, act);
+    return hipGetLastError();
+}
+
 // Upper bound that does not depend on the group size: the kernel never uses
 // more K-splits than asked for.
 static size_t gemv_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k) {
@@ -775,7 +1086,14 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         const int64_t tiles = N / 128;
         int v = 10 /* dma1x4d1 */;
         int64_t s = 1;
-        if (M > 16) {
+        if (M > 16 && N % 512 == 0 && N >= 5120 && K * N >= (M > 32 ? (24ll << 20) : (40ll << 20))) {
+            // 17..64 rows on large weights (from sweeps: 12-34 % faster there, slower on small ones and on
+            // narrow N): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that
+            // about one workgroup per CU exists, four chunks per split at least
+            v = M > 32 ? 24 /* wided2m4 */ : 26 /* wided2m2 */;
+            s = 256 / (N / 512);
+            if (s > chunks / 4) s = chunks / 4;
+        } else if (M > 16) {
             // 17..64 rows: short K with 32 column tiles or more runs as one 8-wave workgroup per tile;
             // otherwise 4-wave workgroups, K split until about 200 of them exist (4 chunks per split at least)
             if (M <= 32 && tiles >= 32 && chunks <= 8) {
@@ -872,6 +1190,29 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         if (N % (128 * gv.wn) != 0 || g % 128 != 0) {
             set_error("%s: variant %s needs N %% %d == 0 and group_size %% 128 == 0", fn, gv.name, 128 * gv.wn);
             return AWQ_ERR_UNSUPPORTED;
+        }
+        if (gv.wide) {
+            if (N % 512 != 0 || g % 128 != 0) {
+                set_error("%s: variant %s needs N %% 512 == 0 and group_size %% 128 == 0", fn, gv.name);
+                return AWQ_ERR_UNSUPPORTED;
+            }
+            if (split_k > 1 && N / 512 > kMaxSplitTiles) {
+                set_error("%s: split-K supports at most %lld column groups (N=%lld)", fn, (long long)kMaxSplitTiles,
+                          (long long)N);
+                return AWQ_ERR_UNSUPPORTED;
+            }
+#define AWQ_WIDE_CASE(DD, MM)                                                                              \
+    if (gv.depth == DD && gv.mt == MM)                                                                     \
+        e = dtype == AWQ_F16 ? launch_gemv_wide<F16, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
+                                                             (int)N, (int)K, (int)g, workspace, split_k, s, act) \
+                             : launch_gemv_wide<BF16, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
+                                                              (int)N, (int)K, (int)g, workspace, split_k, s, act);
+            AWQ_WIDE_CASE(3, 4)
+            AWQ_WIDE_CASE(2, 4)
+            AWQ_WIDE_CASE(3, 2)
+            AWQ_WIDE_CASE(2, 2)
+#undef AWQ_WIDE_CASE
+            return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
         }
         if ((size_t)gv.waves * gv.depth * dma_wave_bytes((int)M) > 160 * 1024 - 1024) {
             set_error("%s: variant %s does not fit the LDS at M=%lld", fn, gv.name, (long long)M);

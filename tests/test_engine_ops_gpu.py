@@ -155,7 +155,8 @@ def test_silu_mul(dtype, rows, inter):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,K,inter", [(1, 1024, 3072), (32, 1024, 3072), (16, 2048, 1024), (64, 5120, 1280), (3, 4096, 64)])
+@pytest.mark.parametrize("M,K,inter", [(1, 1024, 3072), (32, 1024, 3072), (16, 2048, 1024), (64, 5120, 1280), (3, 4096, 64),
+                                           (48, 4096, 3072), (24, 8192, 2560)])   # the last two: shared-chunk kernel
 def test_gemv_swiglu_equals_unfused(dtype, M, K, inter):
     """Gate and up interleaved + gated epilogue must give, bit for bit, what the plain GEMV over gate|up side by
     side followed by the SiLU*up kernel gives (a column's sum does not depend on where the column sits)."""

@@ -88,6 +88,24 @@ def test_gemv_batched_decode_rows(dtype, M):
         _check(y, xb, p, dtype)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,K,N", [(64, 4096, 6144), (33, 4096, 6144), (24, 8192, 5120), (17, 8192, 5120)])
+def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N):
+    # 17..64 rows on weights large enough for the default dispatch to take the shared-chunk kernel
+    # (eight waves per 512 columns, K split, second-pass reduction), with a bias
+    print(f"gemv shared-chunk {dtype} M={M} K={K} N={N}", flush=True)
+    p = random_packed(K, N, 128, dtype, seed=K + N + M)
+    xb = make_x(M, K, dtype, seed=M)
+    bias = np.linspace(-1, 1, N).astype(np.float32)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    from nanoquantization_amd.layers.gemm import _linear   # awq_gemm's entry point, with the bias argument
+    bd = to_dev(o.to_bits16(bias, dtype), dtype)
+    y = _linear("awq_linear", to_dev(xb, dtype), *dev, bd)
+    torch.cuda.synchronize()
+    _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
+    assert torch.equal(y, _linear("awq_linear", to_dev(xb, dtype), *dev, bd))
+
+
 def test_gemv_reference_test_shape():
     # the reference's own GEMM test: K=1024, N=2048, g=32, 8 tokens, atol=1.0 against x @ w_dq.T
     # (awq/tests/dequantization_kernel.py:108-138)
