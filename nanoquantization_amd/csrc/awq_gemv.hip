@@ -530,7 +530,7 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     extern __shared__ float red[];  // staging while streaming, [WAVES][32][64] floats afterwards
     __shared__ int s_last;
     if ((int)blockIdx.x >= groups) {
-        if (blockIdx.y != 0) return;   // with K splits the extra workgroups exist once per split; one set works
+        if (blockIdx.y != 0 || blockIdx.z != 0) return;   // the extra workgroups exist once per split and row block; one set works
         // Prefetch workgroups (launched beside the compute grid on CUs a small GEMV leaves idle): touch one
         // dword of every 128-byte line of the hinted regions -- the packed weights, scales and zeros of the
         // NEXT launch -- so that it finds them in the Infinity Cache instead of HBM.
@@ -554,6 +554,17 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         return;
     }
 
+    if constexpr (MT == 1) {
+        // More than 16 rows: blockIdx.z picks a block of 16 rows, an independent product with its own slice of
+        // x, y, the partials and the arrival counters.  The weights are then read once per row block, the
+        // later ones mostly from cache: worthwhile where a launch is latency-bound, not on large weights.
+        const int rb = blockIdx.z;
+        x += (size_t)rb * 16 * K;
+        y += (size_t)rb * 16 * (act ? N >> 1 : N);
+        partials += (size_t)rb * splits * 16 * N;
+        counters += rb * groups;
+        M = min(16, M - 16 * rb);
+    }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, kb = lane >> 4;
@@ -967,7 +978,7 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
                                                             kCounterBytes)
                                 : nullptr;
-    size_t lds = (size_t)WAVES * DEPTH * dma_wave_bytes(M);
+    size_t lds = (size_t)WAVES * DEPTH * dma_wave_bytes(MT == 1 && M > 16 ? 16 : M);
     const size_t red_bytes = WK > 1 ? (size_t)WAVES * 32 * 64 * sizeof(float) : 0;
     if (lds < red_bytes) lds = red_bytes;
     auto kern = gemv_dma_kernel<T, WN, WK, DEPTH, MT>;
@@ -991,15 +1002,17 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     long long pf_bytes = 0;
     for (int r = 0; r < pf.count; ++r) pf_bytes += pf.bytes[r];
     int pf_wgs = 0;
-    if (pf_bytes >= 128 && (long long)groups * splits < 192) {
+    const int row_blocks = MT == 1 ? (int)cdiv(M, 16) : 1;
+    const long long compute_wgs = (long long)groups * splits * row_blocks;
+    if (pf_bytes >= 128 && compute_wgs < 192) {
         const long long want = cdiv(pf_bytes >> 7, 64 * WAVES * 2);   // about 2 lines per thread
-        const long long room = (256 - (long long)groups * splits) / splits;   // stay within one wave of workgroups
+        const long long room = (256 - compute_wgs) / ((long long)splits * row_blocks);   // stay within one wave of workgroups
         pf_wgs = (int)(want < room ? want : room);
         if (pf_wgs < 1) pf_wgs = 1;
     } else {
         pf.count = 0;
     }
-    hipLaunchKernelGGL(kern, dim3(groups + pf_wgs, splits), dim3(64 * WAVES), lds, stream,
+    hipLaunchKernelGGL(kern, dim3(groups + pf_wgs, splits, row_blocks), dim3(64 * WAVES), lds, stream,
                        reinterpret_cast<const uint16_t*>(x),
                        reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales),
@@ -1049,7 +1062,7 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
 static size_t gemv_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k) {
     (void)variant;
     if (split_k <= 1 || K < 64) return 0;
-    return kCounterBytes + (size_t)split_k * M * N * sizeof(float);
+    return kCounterBytes + (size_t)split_k * (M > 16 ? cdiv(M, 16) * 16 : M) * N * sizeof(float);   // row blocks of 16
 }
 
 // Launch shape for the default entry point.
@@ -1086,24 +1099,15 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         const int64_t tiles = N / 128;
         int v = 10 /* dma1x4d1 */;
         int64_t s = 1;
-        if (M > 16 && N % 512 == 0 && N >= 5120 && K * N >= (M > 32 ? (24ll << 20) : (40ll << 20))) {
-            // 17..64 rows on large weights (from sweeps: 12-34 % faster there, slower on small ones and on
-            // narrow N): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that
-            // about one workgroup per CU exists, four chunks per split at least
+        const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
+        if (M > 16 && N % 512 == 0 && N >= 5120 && K * N >= (M > 32 ? (50ll << 20) : (100ll << 20))) {
+            // 17..64 rows on the largest weights (from sweeps: Qwen3-32B MLP and, above 32 rows, its fused
+            // q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
+            // one workgroup per CU exists, four chunks per split at least.  Below these sizes re-reading the
+            // weights once per block of 16 rows (mostly from cache) is faster than the shared chunk's second pass.
             v = M > 32 ? 24 /* wided2m4 */ : 26 /* wided2m2 */;
             s = 256 / (N / 512);
             if (s > chunks / 4) s = chunks / 4;
-        } else if (M > 16) {
-            // 17..64 rows: short K with 32 column tiles or more runs as one 8-wave workgroup per tile;
-            // otherwise 4-wave workgroups, K split until about 200 of them exist (4 chunks per split at least)
-            if (M <= 32 && tiles >= 32 && chunks <= 8) {
-                v = 21 /* dma1x8d1m2 */;
-            } else {
-                v = M > 32 ? 22 /* dma1x4d1m4 */ : 20 /* dma1x4d1m2 */;
-                if (tiles < 200) s = cdiv(200, tiles);
-                if (s > chunks / 4) s = chunks / 4;
-                s = balance_splits(chunks, s, 4, chunks / 4);
-            }
         } else if (chunks <= 8) {
             v = 11 /* dma1x8d1 */;
         } else if (M <= 4) {
@@ -1112,8 +1116,8 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             const int64_t cap = chunks < 64 ? (chunks / 2 < 10 ? chunks / 2 : 10) : 32;
             if (s > cap) s = cap;
             s = balance_splits(chunks, s, 4, cap);
-        } else if (tiles < 200) {
-            s = cdiv(200, tiles);   // about 200 workgroups
+        } else if (tiles * row_blocks < 200) {
+            s = cdiv(200, tiles * row_blocks);   // about 200 workgroups
             if (s > chunks / 4) s = chunks / 4;
             s = balance_splits(chunks, s, 4, chunks / 4);
         }
@@ -1163,7 +1167,9 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         return AWQ_ERR_INVALID_ARG;
     }
     const GemvVariant& gv = kGemvVariants[variant];
-    if (M > 16 * gv.mt) {
+    // the staged one-m-tile variants take up to 64 rows as independent blocks of 16
+    const bool row_blocked = variant >= kFirstDmaVariant && !gv.wide && gv.mt == 1;
+    if (M > 16 * gv.mt && !row_blocked) {
         set_error("%s: variant %s takes at most %d rows (M=%lld); rows 17..64 need the staged path "
                   "(N %% 128 == 0, group_size %% 128 == 0)", fn, gv.name, 16 * gv.mt, (long long)M);
         return AWQ_ERR_UNSUPPORTED;
@@ -1172,7 +1178,7 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         set_error("%s: variant %s needs N %% %d == 0 (N=%lld)", fn, gv.name, 8 * gv.V, (long long)N);
         return AWQ_ERR_UNSUPPORTED;
     }
-    if (split_k > 1 && cdiv(N / 8, 16 * gv.V) > kMaxSplitTiles) {
+    if (split_k > 1 && cdiv(N / 8, 16 * gv.V) * (row_blocked ? cdiv(M, 16) : 1) > kMaxSplitTiles) {
         set_error("%s: split-K supports at most %lld column tiles (N=%lld)", fn,
                   (long long)kMaxSplitTiles, (long long)N);
         return AWQ_ERR_UNSUPPORTED;
@@ -1214,7 +1220,7 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
 #undef AWQ_WIDE_CASE
             return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
         }
-        if ((size_t)gv.waves * gv.depth * dma_wave_bytes((int)M) > 160 * 1024 - 1024) {
+        if ((size_t)gv.waves * gv.depth * dma_wave_bytes(row_blocked && M > 16 ? 16 : (int)M) > 160 * 1024 - 1024) {
             set_error("%s: variant %s does not fit the LDS at M=%lld", fn, gv.name, (long long)M);
             return AWQ_ERR_UNSUPPORTED;
         }
