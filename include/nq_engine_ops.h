@@ -69,6 +69,12 @@ int nq_paged_attention_decode(const void* q, const void* k_cache, const void* v_
  * Qwen3QuantizedMLP.forward, nanoquantization/models/qwen3_quantized.py:147-152. */
 int nq_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream);
 
+/* out[r] = argmax_i logits[r, i] as int64, the lowest index among equal maxima (NaNs are never selected);
+ * logits [rows, vocab] dense.  Greedy sampling for the engine's decode loop; the reference has no generation
+ * loop, the logits are those of Qwen3QuantizedForCausalLM.forward
+ * (nanoquantization/models/qwen3_quantized.py:312-314). */
+int nq_argmax_rows(const void* logits, int64_t* out, int64_t rows, int64_t vocab, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -344,6 +344,49 @@ __global__ __launch_bounds__(HD) void paged_attn_merge_kernel(const float* __res
 
 // ---------------------------------------------------------------------------------------------
 // out[r, i] = SiLU(gate_up[r, i]) * gate_up[r, inter + i], SiLU rounded to the tensor type first.
+// Greedy sampler: out[r] = index of the largest logits[r, :] (the lowest index among equal maxima; NaNs are never
+// selected).  One workgroup of 16 waves per row, 16-byte loads.
+template <typename T>
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* __restrict__ logits,
+                                                           int64_t* __restrict__ out, int vocab) {
+    const uint16_t* row = logits + (size_t)blockIdx.x * vocab;
+    float best = -__builtin_inff();
+    int bi = 0x7fffffff;
+    auto take = [&](float f, int idx) {
+        if (f > best || (f == best && idx < bi)) {
+            best = f;
+            bi = idx;
+        }
+    };
+    const int nvec = (vocab & 7) == 0 ? vocab >> 3 : 0;   // rows are 16-byte aligned only then
+    for (int v = threadIdx.x; v < nvec; v += 1024) {
+        const u32x4 d = *reinterpret_cast<const u32x4*>(row + (size_t)v * 8);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            take(T::to_f32((uint16_t)(d[i] & 0xFFFFu)), v * 8 + 2 * i);
+            take(T::to_f32((uint16_t)(d[i] >> 16)), v * 8 + 2 * i + 1);
+        }
+    }
+    for (int i = nvec * 8 + threadIdx.x; i < vocab; i += 1024) take(T::to_f32(row[i]), i);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) take(__shfl_xor(best, off), __shfl_xor(bi, off));
+    __shared__ float s_best[16];
+    __shared__ int s_idx[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+        s_best[wave] = best;
+        s_idx[wave] = bi;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        best = lane < 16 ? s_best[lane] : -__builtin_inff();
+        bi = lane < 16 ? s_idx[lane] : 0x7fffffff;
+#pragma unroll
+        for (int off = 8; off >= 1; off >>= 1) take(__shfl_xor(best, off), __shfl_xor(bi, off));
+        if (lane == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate_up,
                                                        uint16_t* __restrict__ out, int64_t rows, int inter) {
@@ -526,6 +569,23 @@ extern "C" int nq_paged_attention_decode(const void* q, const void* k_cache, con
                                            batch, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,
                                            (int)num_blocks, nsplit, scale, st);
     if (rc != AWQ_OK) return rc;
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" int nq_argmax_rows(const void* logits, int64_t* out, int64_t rows, int64_t vocab, int dtype,
+                              void* stream) {
+    const char* fn = "nq_argmax_rows";
+    if (!logits || !out) return bad(fn, "null pointer argument");
+    if (!aligned16(logits)) return bad(fn, "logits must be 16-byte aligned");
+    if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
+    if (rows <= 0 || vocab <= 0 || rows > 0x7fffffff || vocab > 0x7ffffff0) return bad(fn, "rows and vocab must be positive 31-bit counts");
+    hipStream_t st = (hipStream_t)stream;
+    (void)hipGetLastError();
+    if (dtype == AWQ_F16)
+        argmax_rows_kernel<F16><<<dim3((unsigned)rows), dim3(1024), 0, st>>>((const uint16_t*)logits, out, (int)vocab);
+    else
+        argmax_rows_kernel<BF16><<<dim3((unsigned)rows), dim3(1024), 0, st>>>((const uint16_t*)logits, out, (int)vocab);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }

@@ -137,7 +137,7 @@ class LLMEngine:
         last = x.view(b, s, -1)[:, -1].contiguous()
         dlast = delta.view(b, s, -1)[:, -1].contiguous()
         h = ops.add_rmsnorm(last, dlast, m.norm.weight, m.norm.eps)
-        return self.model.lm_head(h).argmax(dim=-1)
+        return ops.argmax_rows(self.model.lm_head(h))
 
     # ---- decode: one token per sequence, attention over the paged cache --------------------------
     def _decode_step(self) -> None:
@@ -171,7 +171,7 @@ class LLMEngine:
                 prefetch_hint(nq_.qweight, nq_.qscales)
             delta = layer.mlp.down_proj(act)
         h = ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps)
-        nxt = self.model.lm_head(h).argmax(dim=-1)
+        nxt = ops.argmax_rows(self.model.lm_head(h))
         self.s_out.index_copy_(0, self.s_step, nxt.unsqueeze(0))
         self.s_ids.copy_(nxt)
         self.s_pos.add_(self.s_active.to(torch.long))               # idle rows stay where they are

@@ -105,6 +105,18 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
+    """Greedy sampler: int64 [rows] index of the largest logit per row (lowest index among equal maxima)."""
+    dev = _dev(logits)
+    rows, vocab = logits.shape
+    assert logits.is_contiguous()
+    out = torch.empty(rows, dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_argmax_rows(logits.data_ptr(), out.data_ptr(), rows, vocab,
+                                             _lib.dtype_id(logits.dtype), _stream()))
+    return out
+
+
 def interleave_gate_up(gate, up):
     """Packed buffers (qweight, qscales, qzeros) of the gate and the up projection -> one set with the word
     columns interleaved (word 2t = gate word t, word 2t+1 = up word t), the layout awq_gemv_swiglu takes."""

@@ -175,3 +175,24 @@ def test_gemv_swiglu_equals_unfused(dtype, M, K, inter):
     ref = ops.silu_mul(nq.awq_gemm(x, side[0], side[1], side[2], 8))
     assert fused.shape == (M, inter)
     assert torch.equal(fused, ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,vocab", [(1, 8), (3, 1000), (32, 151936), (5, 151943), (2, 7)])
+def test_argmax_rows(dtype, rows, vocab):
+    from nanoquantization_amd.engine import ops
+    print(f"argmax_rows {dtype} rows={rows} vocab={vocab}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(rows + vocab)
+    logits = torch.randn(rows, vocab, device="cuda", generator=g).to(dtype)
+    out = ops.argmax_rows(logits)
+    assert out.dtype == torch.int64 and tuple(out.shape) == (rows,)
+    # 16-bit logits tie often: the winner must hold the maximum and be the first to do so
+    mx = logits.float().max(dim=1).values
+    first = (logits.float() == mx[:, None]).float().argmax(dim=1)
+    assert torch.equal(out, first)
+    # planted ties and extremes
+    logits[0, :] = -float("inf")
+    assert ops.argmax_rows(logits)[0].item() == 0
+    logits[0, vocab - 1] = 3.0
+    logits[0, vocab // 2] = 3.0
+    assert ops.argmax_rows(logits)[0].item() == vocab // 2
