@@ -325,6 +325,173 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_kernel(
     }
 }
 
+// The same for 4 or 8 query heads per kv head and 128 head dims, where the kernel above is bound by its
+// vector-ALU dot products (8 FMAs, 4 shuffles and an online-softmax update per token, head and lane).
+// A wave takes tiles of 16 tokens.  Scores: S^T = K q^T on the 16x16x32 MFMA (A = 16 token rows of K, 32 head dims
+// per instruction; B = the G query heads as columns, the rest zero), so a lane ends up with 4 tokens of one head and
+// the softmax bookkeeping is done once per tile and head, not per token and lane.  The probabilities cross to the
+// value phase through a 16 x G array in LDS (private to the wave); there a lane holds 8 head dims of one token's V row
+// as before and adds p * v for the G heads.  Tiles start at multiples of 16 tokens inside a context split and
+// block_size % 16 == 0, so a tile never straddles a cache block.
+template <typename T, int G, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_mfma_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, const int32_t* __restrict__ context_lens, uint16_t* __restrict__ out,
+    float* __restrict__ partial, int nkv, int block_size, int max_blocks, int num_blocks, int nsplit, float scale) {
+    constexpr int HD = 128, TT = 16;
+    static_assert(G == 4 || G == 8, "query heads per kv head");
+    const int sp = blockIdx.x % nsplit;
+    const int kvh = (blockIdx.x / nsplit) % nkv;
+    const int b = blockIdx.x / (nsplit * nkv);
+    const int nh = nkv * G;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lo = lane & 15, hi = lane >> 4;   // score phase: head lo, token quad hi; value phase: dims 8*lo.., token hi
+
+    int ctx = context_lens[b];
+    ctx = ctx < 0 ? 0 : (ctx > max_blocks * block_size ? max_blocks * block_size : ctx);
+    const int per = ((ctx + nsplit - 1) / nsplit + TT - 1) / TT * TT;
+    const int t0 = sp * per, t1 = min(ctx, t0 + per);
+
+    __shared__ float s_p[WAVES][TT * G + G];   // per wave: p[token][head], then the rescale factor per head
+    __shared__ float s_acc[WAVES][G][HD + 2];
+    float* P = s_p[wave];
+
+    u32x4 bq[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bq[i] = u32x4{0u, 0u, 0u, 0u};
+        if (lo < G)
+            bq[i] = *reinterpret_cast<const u32x4*>(q + ((int64_t)b * nh + kvh * G + lo) * HD + 32 * i + 8 * hi);
+    }
+    const float sc = scale * kLog2e;
+    float m = kNegBig, lpart = 0.f;
+    float acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+
+    const int32_t* table = block_table + (int64_t)b * max_blocks;
+    for (int tb = t0 + wave * TT; tb < t1; tb += WAVES * TT) {
+        int blk = table[tb / block_size];                         // wave-uniform
+        blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);
+        const int64_t base = (((int64_t)blk * nkv + kvh) * block_size + tb % block_size) * HD;
+        u32x4 ka[4], va[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)   // K row of token tb + lo (rows past the context are masked below)
+            ka[i] = *reinterpret_cast<const u32x4*>(k_cache + base + (int64_t)lo * HD + 32 * i + 8 * hi);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {   // V rows: a masked token reads the last valid row (its p is 0, the row is finite)
+            const int tv = min(4 * u + hi, t1 - 1 - tb);
+            va[u] = *reinterpret_cast<const u32x4*>(v_cache + base + (int64_t)tv * HD + 8 * lo);
+        }
+        f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) st = T::mfma16(ka[i], bq[i], st);
+        // st[r]: head lo, token tb + 4*hi + r
+        float sv[4], mx = kNegBig;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            sv[r] = (tb + 4 * hi + r < t1) ? st[r] * sc : kNegBig;
+            mx = fmaxf(mx, sv[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mn = fmaxf(m, mx);
+        const float c = exp2f(m - mn);
+        m = mn;
+        float ps = 0.f;
+        float pr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            pr[r] = (tb + 4 * hi + r < t1) ? exp2f(sv[r] - mn) : 0.f;
+            ps += pr[r];
+        }
+        lpart = lpart * c + ps;
+        if (lo < G) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) P[(4 * hi + r) * G + lo] = pr[r];
+            if (hi == 0) P[TT * G + lo] = c;
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_wave_barrier();   // LDS operations of a wave execute in order: the reads below see these writes
+        asm volatile("" ::: "memory");
+        float cg[G];
+#pragma unroll
+        for (int g = 0; g < G; g += 4) {
+            const f32x4 v4 = *reinterpret_cast<const f32x4*>(P + TT * G + g);
+            cg[g] = v4[0]; cg[g + 1] = v4[1]; cg[g + 2] = v4[2]; cg[g + 3] = v4[3];
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[g][e] *= cg[g];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            float vf[8], pg[G];
+            unpack8<T>(va[u], vf);
+#pragma unroll
+            for (int g = 0; g < G; g += 4) {
+                const f32x4 v4 = *reinterpret_cast<const f32x4*>(P + (4 * u + hi) * G + g);
+                pg[g] = v4[0]; pg[g + 1] = v4[1]; pg[g + 2] = v4[2]; pg[g + 3] = v4[3];
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[g][e] += pg[g] * vf[e];
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_wave_barrier();   // the next tile's writes come after these reads
+        asm volatile("" ::: "memory");
+    }
+
+    // the four token groups of the wave share m: their accumulators and partial sums just add
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            acc[g][e] += __shfl_xor(acc[g][e], 16);
+            acc[g][e] += __shfl_xor(acc[g][e], 32);
+        }
+    lpart += __shfl_xor(lpart, 16);
+    lpart += __shfl_xor(lpart, 32);
+    if (hi == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s_acc[wave][g][lo * 8 + e] = acc[g][e];
+        if (lo < G) {
+            s_acc[wave][lo][HD] = m;
+            s_acc[wave][lo][HD + 1] = lpart;
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * HD; idx += 64 * WAVES) {
+        const int g = idx / HD, d = idx % HD;
+        float mn = kNegBig;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) mn = fmaxf(mn, s_acc[w][g][HD]);
+        float lt = 0.f, at = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float c = exp2f(s_acc[w][g][HD] - mn);
+            lt += s_acc[w][g][HD + 1] * c;
+            at += s_acc[w][g][d] * c;
+        }
+        const int64_t head = (int64_t)b * nh + kvh * G + g;
+        if (nsplit == 1) {
+            out[head * HD + d] = T::from_f32(lt > 0.f ? at / lt : 0.f);
+        } else {
+            float* dst = partial + (head * nsplit + sp) * (HD + 2);
+            dst[d] = at;
+            if (d == 0) {
+                dst[HD] = mn;
+                dst[HD + 1] = lt;
+            }
+        }
+    }
+}
+
 // Merge of the context splits: one workgroup of HD threads per (sequence, query head).
 template <typename T, int HD>
 __global__ __launch_bounds__(HD) void paged_attn_merge_kernel(const float* __restrict__ partial,
@@ -424,6 +591,17 @@ void launch_attn(const void* q, const void* kc, const void* vc, const int32_t* t
                  float* partial, int64_t batch, int nkv, int bs, int max_blocks, int num_blocks, int nsplit,
                  float scale, hipStream_t st) {
     constexpr int WAVES = G <= 2 ? 16 : (G <= 4 ? 8 : 4);
+    if constexpr (HD == 128 && (G == 4 || G == 8)) {
+        if (bs % 16 == 0) {
+            paged_attn_decode_mfma_kernel<T, G, WAVES><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(64 * WAVES), 0, st>>>(
+                (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, table, ctx, (uint16_t*)out, partial, nkv,
+                bs, max_blocks, num_blocks, nsplit, scale);
+            if (nsplit > 1)
+                paged_attn_merge_kernel<T, HD><<<dim3((unsigned)(batch * nkv * G)), dim3(HD), 0, st>>>(
+                    partial, (uint16_t*)out, nsplit);
+            return;
+        }
+    }
     paged_attn_decode_kernel<T, G, HD, WAVES><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(64 * WAVES), 0, st>>>(
         (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, table, ctx, (uint16_t*)out, partial, nkv, bs,
         max_blocks, num_blocks, nsplit, scale);

@@ -114,6 +114,10 @@ def _attn_ref(q, kc, vc, table, ctx, scale):
     (5, 4, 4, 64, 32, 9),         # head_dim 64, no grouping
     (130, 8, 8, 128, 64, 1),      # one block per sequence, single split
     (2, 4, 1, 128, 48, 7),        # block size that is not a power of two
+    (8, 32, 8, 128, 64, 6),       # 4 query heads per kv head
+    (4, 64, 8, 128, 64, 40),      # 8 per kv head, long context, context splits
+    (9, 16, 2, 128, 16, 11),      # 8 per kv head, one tile per block
+    (3, 8, 1, 128, 24, 5),        # 8 per kv head, block size not a multiple of the tile: the general kernel
 ])
 def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
     from nanoquantization_amd.engine import ops
@@ -131,6 +135,32 @@ def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
     out = ops.paged_attention_decode(q, kc, vc, table, ctx, scale)
     _close(out, _attn_ref(q, kc, vc, table, ctx, scale), dtype, scale=2.0, what="attention")
     assert torch.equal(out, ops.paged_attention_decode(q, kc, vc, table, ctx, scale)), "run-to-run bit-stable"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv", [(16, 8), (64, 8), (16, 4)])
+def test_paged_attention_ignores_rows_past_the_context(dtype, nh, nkv):
+    """Cache rows past a sequence's context (and unused blocks) hold whatever was there before: NaNs planted there
+    must not reach the output."""
+    from nanoquantization_amd.engine import ops
+    B, hd, bs, max_blocks = 6, 128, 32, 5
+    g = torch.Generator().manual_seed(nh)
+    nb = B * max_blocks + 2
+    table = torch.randperm(nb, generator=g)[: B * max_blocks].view(B, max_blocks).to(torch.int32)
+    ctx = torch.tensor([1, 17, 32, 33, 100, 159], dtype=torch.int32)
+    kc = torch.full((nb, nkv, bs, hd), float("nan"))
+    vc = torch.full((nb, nkv, bs, hd), float("nan"))
+    for b in range(B):
+        t = torch.arange(int(ctx[b]))
+        blk, off = table[b, t // bs].long(), t % bs
+        kc[blk, :, off] = torch.randn(len(t), nkv, hd, generator=g)
+        vc[blk, :, off] = torch.randn(len(t), nkv, hd, generator=g)
+    kc, vc, table, ctx = kc.to(dtype).cuda(), vc.to(dtype).cuda(), table.cuda(), ctx.cuda()
+    q = torch.randn(B, nh, hd, generator=g).to(dtype).cuda()
+    scale = 1.0 / math.sqrt(hd)
+    out = ops.paged_attention_decode(q, kc, vc, table, ctx, scale)
+    assert torch.isfinite(out.float()).all()
+    _close(out, _attn_ref(q, kc, vc, table, ctx, scale), dtype, scale=2.0, what="attention")
 
 
 def test_paged_attention_rejects_unsupported():
