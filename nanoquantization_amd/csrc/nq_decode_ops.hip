@@ -526,12 +526,23 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* __res
         }
     };
     const int nvec = (vocab & 7) == 0 ? vocab >> 3 : 0;   // rows are 16-byte aligned only then
-    for (int v = threadIdx.x; v < nvec; v += 1024) {
-        const u32x4 d = *reinterpret_cast<const u32x4*>(row + (size_t)v * 8);
+    for (int v0 = threadIdx.x; v0 < nvec; v0 += 4 * 1024) {
+        u32x4 d[4];   // four loads in flight
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            take(T::to_f32((uint16_t)(d[i] & 0xFFFFu)), v * 8 + 2 * i);
-            take(T::to_f32((uint16_t)(d[i] >> 16)), v * 8 + 2 * i + 1);
+        for (int u = 0; u < 4; ++u) {
+            const int v = v0 + u * 1024;
+            d[u] = *reinterpret_cast<const u32x4*>(row + (size_t)(v < nvec ? v : v0) * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int v = v0 + u * 1024;
+            if (v < nvec) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    take(T::to_f32((uint16_t)(d[u][i] & 0xFFFFu)), v * 8 + 2 * i);
+                    take(T::to_f32((uint16_t)(d[u][i] >> 16)), v * 8 + 2 * i + 1);
+                }
+            }
         }
     }
     for (int i = nvec * 8 + threadIdx.x; i < vocab; i += 1024) take(T::to_f32(row[i]), i);
