@@ -63,6 +63,35 @@ def test_gemv_every_variant_and_split(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("K", [1024, 2048])
+def test_gemv_staged_variants_with_one_group(dtype, K):
+    # group_size == K, the one size above 128 the reference admits (layers/gemm.py:7,152): every 128-row chunk
+    # shares one scale/zero row; on every staged variant, row blocks (17..64 rows on the one-m-tile kernels) and
+    # the shared-chunk kernel included
+    L = _lib.lib()
+    names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
+    N, g = 512, K
+    p = random_packed(K, N, g, dtype, seed=g)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    for M in (5, 17, 64):
+        xb = make_x(M, K, dtype, seed=M + g)
+        xd = to_dev(xb, dtype)
+        for v, name in enumerate(names):
+            if not (name.startswith("dma") or name.startswith("wide")):
+                continue
+            for split in (1, 3):
+                print(f"gemv g={g} variant {name} split={split} M={M} {dtype}", flush=True)
+                try:
+                    y = awq_gemv_variant(xd, *dev, v, split)
+                except _lib.AwqHipError as e:
+                    if "does not fit the LDS" in str(e) or "takes at most" in str(e) or "needs N %" in str(e):
+                        continue
+                    raise
+                torch.cuda.synchronize()
+                _check(y, xb, p, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("K,N,g", [(256, 8, 128), (128, 136, 32), (512, 1000, 64), (384, 2056, 128), (512, 264, 512)])
 def test_gemv_ragged_shapes_and_groups(dtype, K, N, g):
     print(f"gemv ragged {dtype} K={K} N={N} g={g}", flush=True)
