@@ -185,6 +185,76 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     }
 }
 
+// The same with 16-byte accesses, for head dims of 64, 128 or 256 and 16-byte aligned tensors (the scalar kernel
+// above moves 2 bytes per lane and instruction: 260 us per layer for a 16,384-token prefill of Qwen3-0.6B).
+// A lane owns 8 consecutive dims of a head, HD/8 lanes a head, a wave 64/(HD/8) heads; the rotary partner
+// (dims i and i + HD/2) sits HD/16 lanes away.  The arithmetic per element is that of the scalar kernel.
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
+    const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ q_weight, const uint16_t* __restrict__ k_weight,
+    const float* __restrict__ cos_sin, const int64_t* __restrict__ positions, const int64_t* __restrict__ slots,
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_out, uint16_t* __restrict__ k_cache,
+    uint16_t* __restrict__ v_cache, int rows, int nh, int nkv, int max_positions, int64_t num_slots, int block_size,
+    float eps) {
+    constexpr int LPH = HD / 8, HPW = 64 / LPH, HALF = HD / 2;
+    const int heads = nh + 2 * nkv;
+    const int lane = threadIdx.x & 63, sub = lane / LPH, dc = lane % LPH;
+    const int64_t items = (int64_t)rows * heads;
+    int64_t item = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * HPW + sub;
+    const bool live = item < items;   // lanes past the end follow the last item (the shuffles need them) and store nothing
+    item = live ? item : items - 1;
+    const int row = (int)(item / heads), h = (int)(item % heads);
+    const uint16_t* src = qkv + ((int64_t)row * heads + h) * HD + dc * 8;
+    const int64_t slot = slots[row];
+    const bool slot_ok = slot >= 0 && slot < num_slots;
+    float a[8];
+    const u32x4 raw = *reinterpret_cast<const u32x4*>(src);
+    unpack8<T>(raw, a);
+    if (h >= nh + nkv) {   // v: plain copy
+        if (live && slot_ok)
+            *reinterpret_cast<u32x4*>(v_cache + (((slot / block_size) * nkv + (h - nh - nkv)) * block_size +
+                                                  slot % block_size) * HD + dc * 8) = raw;
+        // no return: heads of one wave differ in kind, and the shuffles below need every lane
+    }
+    const bool is_q = h < nh, is_k = !is_q && h < nh + nkv;
+    const uint16_t* w = is_q ? q_weight : k_weight;
+    float wf[8];
+    unpack8<T>(*reinterpret_cast<const u32x4*>(w + dc * 8), wf);
+    int64_t pos = positions[row];
+    pos = pos < 0 ? 0 : (pos >= max_positions ? max_positions - 1 : pos);
+    const int i0 = (dc % (LPH / 2)) * 8;   // index of this lane's first dim inside its half
+    const float* cs = cos_sin + pos * HD;
+    const f32x4 c0 = *reinterpret_cast<const f32x4*>(cs + i0), c1 = *reinterpret_cast<const f32x4*>(cs + i0 + 4);
+    const f32x4 s0 = *reinterpret_cast<const f32x4*>(cs + HALF + i0), s1 = *reinterpret_cast<const f32x4*>(cs + HALF + i0 + 4);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += a[e] * a[e];
+#pragma unroll
+    for (int o = LPH / 2; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
+    const float r = rsqrtf(ss / (float)HD + eps);
+    float xn[8], y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xn[e] = round_to<T>(round_to<T>(a[e] * r) * wf[e]);
+    const bool first = dc < LPH / 2;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float other = __shfl_xor(xn[e], LPH / 2);
+        const float cc = e < 4 ? c0[e] : c1[e - 4], sn = e < 4 ? s0[e] : s1[e - 4];
+        const float x1 = first ? xn[e] : other, x2 = first ? other : xn[e];
+        y[e] = first ? __fsub_rn(__fmul_rn(x1, cc), __fmul_rn(x2, sn)) : __fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cc));
+    }
+    if (!live || !(is_q || is_k)) return;
+    const u32x4 packed = pack8<T>(y);
+    if (is_q) {
+        *reinterpret_cast<u32x4*>(q_out + ((int64_t)row * nh + h) * HD + dc * 8) = packed;
+        return;
+    }
+    if (k_out) *reinterpret_cast<u32x4*>(k_out + ((int64_t)row * nkv + (h - nh)) * HD + dc * 8) = packed;
+    if (slot_ok)
+        *reinterpret_cast<u32x4*>(k_cache + (((slot / block_size) * nkv + (h - nh)) * block_size + slot % block_size) * HD +
+                                  dc * 8) = packed;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Attention of one new token per sequence over its paged KV cache (flash-decoding).
 // Workgroup = (sequence, kv head, context split), WAVES waves (16 for up to 2 query heads per kv head, 8 for
@@ -687,6 +757,28 @@ extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, cons
     if (items > ((int64_t)1 << 32)) return bad(fn, "too many rows");
     hipStream_t st = (hipStream_t)stream;
     (void)hipGetLastError();
+    const bool vec = (head_dim == 64 || head_dim == 128 || head_dim == 256) && aligned16(qkv) && aligned16(q_weight) &&
+                     aligned16(k_weight) && aligned16(cos_sin) && aligned16(q_out) && aligned16(k_out) &&
+                     aligned16(k_cache) && aligned16(v_cache);
+    if (vec) {
+#define NQ_ROPE_VEC(TT, HH)                                                                                          \
+    qk_norm_rope_store_vec_kernel<TT, HH><<<dim3((unsigned)cdiv(items, 4 * (64 / (HH / 8)))), dim3(256), 0, st>>>(  \
+        (const uint16_t*)qkv, (const uint16_t*)q_weight, (const uint16_t*)k_weight, cos_sin, positions, slots,      \
+        (uint16_t*)q_out, (uint16_t*)k_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (int)rows, (int)num_heads,       \
+        (int)num_kv_heads, (int)max_positions, num_slots, (int)block_size, eps)
+        if (dtype == AWQ_F16) {
+            if (head_dim == 64) NQ_ROPE_VEC(F16, 64);
+            else if (head_dim == 128) NQ_ROPE_VEC(F16, 128);
+            else NQ_ROPE_VEC(F16, 256);
+        } else {
+            if (head_dim == 64) NQ_ROPE_VEC(BF16, 64);
+            else if (head_dim == 128) NQ_ROPE_VEC(BF16, 128);
+            else NQ_ROPE_VEC(BF16, 256);
+        }
+#undef NQ_ROPE_VEC
+        const hipError_t ev = hipGetLastError();
+        return ev == hipSuccess ? AWQ_OK : hip_fail(fn, ev);
+    }
     const dim3 grid((unsigned)cdiv(items, 4)), block(256);
     if (dtype == AWQ_F16)
         qk_norm_rope_store_kernel<F16><<<grid, block, 0, st>>>(

@@ -53,7 +53,8 @@ def test_add_rmsnorm_rejects_bad_shapes():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv,hd", [(16, 8, 128), (4, 4, 64), (8, 1, 256), (64, 8, 128)])
+@pytest.mark.parametrize("nh,nkv,hd", [(16, 8, 128), (4, 4, 64), (8, 1, 256), (64, 8, 128),
+                                       (6, 2, 96)])    # 96: the scalar kernel (head dims other than 64/128/256)
 def test_qk_norm_rope_store(dtype, nh, nkv, hd):
     from nanoquantization_amd.engine import ops
     from nanoquantization_amd.layers.rope import RoPE
