@@ -89,6 +89,15 @@ int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void* qscales, 
                     void* y, int64_t M, int64_t N, int64_t K, int64_t group_size, int dtype,
                     void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same gated product for any M: the GEMV above for M <= 64 where it applies, the pipelined MFMA GEMM with the
+ * gate applied in its epilogue otherwise (K % 64 == 0, N % 16 == 0).  Same interleaved buffers, y [M, N/2].
+ * Replaces the two linears and the activation of Qwen3QuantizedMLP.forward,
+ * nanoquantization/models/qwen3_quantized.py:147-152, for prefill as well as decode. */
+size_t awq_linear_swiglu_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int awq_linear_swiglu(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                      void* y, int64_t M, int64_t N, int64_t K, int64_t group_size, int dtype,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* Optional hint for latency-bound decode loops: the next awq_gemv / awq_linear / awq_gemv_swiglu call of
  * the calling thread that takes the staged GEMV path and leaves compute units idle also launches a few
  * spare workgroups that read [ptr, ptr + bytes) -- meant to be the packed qweight of the launch AFTER it --

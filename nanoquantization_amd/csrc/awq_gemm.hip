@@ -296,10 +296,15 @@ static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_
     *split_k = (int)s;
 }
 
+// The same for the pipelined kernel at any M (the gated epilogue exists there only).
+static void pick_gemm_pipe(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
+    pick_gemm(M > 128 ? M : 129, N, K, variant, split_k);   // tile counts depend on ceil(M / 256) only
+}
+
 static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, const void* qscales,
                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
-                         void* stream, int variant, int split_k) {
+                         void* stream, int variant, int split_k, int act = 0) {
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
     if (K % kBK != 0 || !(g % 64 == 0 || (64 % g == 0 && g % 8 == 0))) {
@@ -314,6 +319,10 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     if (variant < 0 || variant >= kNumGemmVariants || split_k < 1) {
         set_error("%s: bad variant %d / split_k %d", fn, variant, split_k);
         return AWQ_ERR_INVALID_ARG;
+    }
+    if (act && (bias || N % 16 != 0 || (variant != kPipeVariant && variant != kPipeTailVariant))) {
+        set_error("%s: the gated epilogue takes no bias, needs N %% 16 == 0 and runs on the pipelined kernel", fn);
+        return AWQ_ERR_UNSUPPORTED;
     }
     const GemmVariant& gv = kGemmVariants[variant];
     if (cdiv(M, gv.BM) > 65535) {
@@ -350,7 +359,7 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         case kPipeVariant:
         case kPipeTailVariant:
             e = launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
-                                 workspace, split_k, variant == kPipeTailVariant, s);
+                                 workspace, split_k, variant == kPipeTailVariant, s, act);
             break;
     }
 #undef AWQ_GEMM_CASE
@@ -403,6 +412,29 @@ extern "C" size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     const size_t a = M <= 64 ? awq_gemv_workspace_bytes(M, N, K) : 0;
     const size_t b = M > 16 ? awq_gemm_workspace_bytes(M, N, K) : 0;
     return a > b ? a : b;
+}
+
+extern "C" size_t awq_linear_swiglu_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (K < awq::kBK || N < 16 || M < 1) return 0;
+    const size_t a = M <= 64 ? awq_gemv_workspace_bytes(M, N, K) : 0;
+    int v, s;
+    awq::pick_gemm_pipe(M, N, K, &v, &s);
+    const size_t b = awq::gemm_ws_bytes(M, N, K, v, s);
+    return a > b ? a : b;
+}
+
+extern "C" int awq_linear_swiglu(const void* x, const int32_t* qweight, const void* qscales,
+                                 const int32_t* qzeros, void* y, int64_t M, int64_t N, int64_t K,
+                                 int64_t group_size, int dtype, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+    const bool staged = N % 128 == 0 && group_size > 0 && group_size % 128 == 0;
+    if (M >= 1 && M <= 64 && staged)
+        return awq_gemv_swiglu(x, qweight, qscales, qzeros, y, M, N, K, group_size, dtype, workspace,
+                               workspace_bytes, stream);
+    int v = awq::kPipeVariant, s = 1;
+    if (K >= awq::kBK && N >= 16 && M >= 1) awq::pick_gemm_pipe(M, N, K, &v, &s);
+    return awq::gemm_dispatch("awq_linear_swiglu", x, qweight, qscales, qzeros, nullptr, y, M, N, K, group_size,
+                              dtype, workspace, workspace_bytes, stream, v, s, 1);
 }
 
 extern "C" int awq_linear(const void* x, const int32_t* qweight, const void* qscales,

@@ -143,6 +143,7 @@ inline hipError_t launch_splitk_reduce(int dtype, const float* partials, const v
 // K slices of `iters_per_split` 64-row steps whose fp32 partials a second kernel adds.
 struct PipePlan {
     int tiles_n, full_tiles, tail_tiles, splits, iters_per_split;
+    int act;   // 1: gate|up word-interleaved along N, y [M, N/2] = dtype(SiLU(gate)) * up (no bias)
 };
 
 // tail_only = false: every tile is cut `split_k` ways (none if that leaves one slice).
@@ -157,6 +158,7 @@ inline PipePlan make_pipe_plan(int64_t M, int64_t N, int64_t K, int split_k, boo
     p.tail_tiles = p.splits <= 1 ? 0 : (tail_only ? tiles % 256 : tiles);
     p.full_tiles = tiles - p.tail_tiles;
     if (p.tail_tiles == 0) p.splits = 1;
+    p.act = 0;
     return p;
 }
 
@@ -167,6 +169,6 @@ inline size_t pipe_ws_bytes(const PipePlan& p) {
 // awq_gemm_pipe.hip: the 256 x 256 software-pipelined kernel (same arguments as the tiled launcher).
 hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
-                            void* workspace, int split_k, bool tail_only, hipStream_t stream);
+                            void* workspace, int split_k, bool tail_only, hipStream_t stream, int act = 0);
 
 }  // namespace awq

@@ -99,6 +99,29 @@ struct Raw {
     u32x4 s;
 };
 
+// Gated epilogue: a lane pair holds a gate word and the up word of the same 8 outputs (already rounded to T); each
+// lane of the pair produces four of them (the even lane outputs 0..3, the odd lane 4..7) and stores 8 bytes:
+// dtype(SiLU(gate)) * up, the rounding points of F.silu(gate_proj(x)) * up_proj(x).  `mine` is this lane's word,
+// `other` its partner's, `odd` says which of the two this lane holds.
+template <typename T>
+__device__ __forceinline__ void swiglu_pair_store(u32x4 mine, u32x4 other, bool odd, uint16_t* __restrict__ dst) {
+    const u32x4 gate = odd ? other : mine, up = odd ? mine : other;
+    uint32_t o[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t gw = odd ? gate[2 + i] : gate[i], uw = odd ? up[2 + i] : up[i];
+        float r[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float g = T::to_f32((uint16_t)(h ? gw >> 16 : gw & 0xFFFFu));
+            const float u = T::to_f32((uint16_t)(h ? uw >> 16 : uw & 0xFFFFu));
+            r[h] = T::to_f32(T::from_f32(g / (1.f + __expf(-g)))) * u;
+        }
+        o[i] = T::pack2(r[0], r[1]);
+    }
+    *reinterpret_cast<u32x2*>(dst + (odd ? 4 : 0)) = u32x2{o[0], o[1]};
+}
+
 template <typename T, int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
@@ -306,7 +329,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
                 const int row = RPP * j + lane / LPR, chunk = lane % LPR;
                 const u32x4 val = *reinterpret_cast<const u32x4*>(stage + row * PITCH + chunk * 8);
                 const int m = m0 + wm0 + a * 32 + row, n = n0 + wn0 + chunk * 8;
-                if (m < M && n < N) *reinterpret_cast<u32x4*>(y + (size_t)m * N + n) = val;
+                if (plan.act) {
+                    // a lane holds one word of 8 columns; even words are gate columns, the next word the up
+                    // columns of the same outputs (N % 16 == 0, so a pair is in range or out of range together)
+                    u32x4 other;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(val[i], 1);
+                    if (m < M && n < N)
+                        swiglu_pair_store<T>(val, other, chunk & 1, y + (size_t)m * (N >> 1) + ((n & ~15) >> 1));
+                } else if (m < M && n < N) {
+                    *reinterpret_cast<u32x4*>(y + (size_t)m * N + n) = val;
+                }
             }
         }
     } else {
@@ -345,6 +378,16 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __re
         hi += *reinterpret_cast<const f32x4*>(p + s * plane + 4);
     }
     float out[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (plan.act) {
+        u32x4 mine, other;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            mine[i] = T::pack2(out[2 * i], out[2 * i + 1]);
+            other[i] = __shfl_xor(mine[i], 1);   // the neighbouring word: in range together with this one
+        }
+        swiglu_pair_store<T>(mine, other, (n >> 3) & 1, y + (size_t)m * (N >> 1) + ((n & ~15) >> 1));
+        return;
+    }
     if (bias) {
         const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + n);
 #pragma unroll
@@ -360,8 +403,9 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __re
 template <typename T, int WM, int WN>
 hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
                        const void* bias, void* y, int M, int N, int K, int g, void* workspace, int split_k,
-                       bool tail_only, hipStream_t stream) {
-    const PipePlan plan = make_pipe_plan(M, N, K, split_k, tail_only);
+                       bool tail_only, hipStream_t stream, int act) {
+    PipePlan plan = make_pipe_plan(M, N, K, split_k, tail_only);
+    plan.act = act;
     float* partials =
         workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes) : nullptr;
     const size_t lds = (size_t)2 * (8 * 256 + 8 * 256) * 16;  // 128 KiB
@@ -389,12 +433,12 @@ hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscale
 
 hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
-                            void* workspace, int split_k, bool tail_only, hipStream_t stream) {
+                            void* workspace, int split_k, bool tail_only, hipStream_t stream, int act) {
     return dtype == AWQ_F16
                ? launch_pipe<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, tail_only,
-                                        stream)
+                                        stream, act)
                : launch_pipe<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, tail_only,
-                                         stream);
+                                         stream, act);
 }
 
 }  // namespace awq

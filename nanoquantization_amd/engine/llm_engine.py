@@ -84,10 +84,11 @@ class LLMEngine:
             num_blocks = max_batch * self.max_blocks
         self.cache = PagedKVCache(len(layers), num_blocks, block_size, self.nkv, self.hd, self.dtype, self.device)
         self.qkv = [_FusedLinear([l.self_attn.q_proj, l.self_attn.k_proj, l.self_attn.v_proj]) for l in layers]
-        self.gate_up = [_FusedLinear([l.mlp.gate_proj, l.mlp.up_proj]) for l in layers]
-        # decode: gate and up interleaved word by word, SiLU(gate) * up applied in the GEMV's epilogue
+        # gate and up interleaved word by word, SiLU(gate) * up applied in the epilogue of the GEMV (decode) or
+        # the GEMM (prefill); shapes that form does not take keep the two projections side by side + silu_mul
         g0 = layers[0].mlp.gate_proj
-        self.swiglu_ok = (max_batch <= 64 and (2 * self.inter) % 128 == 0 and g0.group_size % 128 == 0)
+        self.swiglu_ok = (2 * self.inter) % 128 == 0 and g0.group_size % 128 == 0 and g0.in_features % 64 == 0
+        self.gate_up = None if self.swiglu_ok else [_FusedLinear([l.mlp.gate_proj, l.mlp.up_proj]) for l in layers]
         self.gate_up_il = [ops.interleave_gate_up((l.mlp.gate_proj.qweight, l.mlp.gate_proj.qscales, l.mlp.gate_proj.qzeros),
                                                   (l.mlp.up_proj.qweight, l.mlp.up_proj.qscales, l.mlp.up_proj.qzeros))
                            for l in layers] if self.swiglu_ok else None
@@ -133,7 +134,9 @@ class LLMEngine:
                                                is_causal=True, enable_gqa=gqa)
             o = o.transpose(1, 2).reshape(b * s, self.nh * self.hd)
             h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
-            delta = layer.mlp.down_proj(ops.silu_mul(self.gate_up[li](h)))
+            act = (ops.awq_linear_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
+                   else ops.silu_mul(self.gate_up[li](h)))
+            delta = layer.mlp.down_proj(act)
         last = x.view(b, s, -1)[:, -1].contiguous()
         dlast = delta.view(b, s, -1)[:, -1].contiguous()
         h = ops.add_rmsnorm(last, dlast, m.norm.weight, m.norm.eps)
@@ -164,7 +167,7 @@ class LLMEngine:
             prefetch_hint(*gu)
             h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
             prefetch_hint(layer.mlp.down_proj.qweight, layer.mlp.down_proj.qscales)
-            act = (ops.awq_gemv_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
+            act = (ops.awq_linear_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
                    else ops.silu_mul(self.gate_up[li](h)))
             if li + 1 < nl:
                 nq_ = self.qkv[li + 1]

@@ -130,6 +130,25 @@ def interleave_gate_up(gate, up):
     return qweight, qscales, qzeros
 
 
+def awq_linear_swiglu(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor) -> torch.Tensor:
+    """x [M, K] (any M) and interleaved gate|up buffers [K, 2*inter/8] -> SiLU(x @ Wgate) * (x @ Wup) [M, inter]."""
+    dev = _dev(x, qweight, qscales, qzeros)
+    M, K = x.shape
+    N = qscales.shape[1]
+    g = K // qscales.shape[0]
+    assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    out = torch.empty(M, N // 2, dtype=x.dtype, device=dev)
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        stream = _stream()
+        nbytes = L.awq_linear_swiglu_workspace_bytes(M, N, K)
+        ws = _lib.workspace(dev, stream, nbytes)
+        _lib.check(L.awq_linear_swiglu(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(),
+                                       out.data_ptr(), M, N, K, g, _lib.dtype_id(x.dtype),
+                                       None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), stream))
+    return out
+
+
 def awq_gemv_swiglu(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor) -> torch.Tensor:
     """x [M <= 64, K] and interleaved gate|up buffers [K, 2*inter/8] -> SiLU(x @ Wgate) * (x @ Wup) [M, inter]."""
     dev = _dev(x, qweight, qscales, qzeros)
