@@ -98,6 +98,21 @@ int awq_linear_swiglu(const void* x, const int32_t* qweight, const void* qscales
                       void* y, int64_t M, int64_t N, int64_t K, int64_t group_size, int dtype,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* awq_gemv on the fused q|k|v projection of a decode step with what follows it fused in (head_dim 128, so a
+ * 128-column tile is one head): per-head RMSNorm of q and k, half-split rotary at positions[row], q written to
+ * q_out [M, num_heads, 128], k and v to slot slots[row] of the paged cache [blocks, kv heads, block_size, 128]
+ * (a negative slot writes no k/v).  N = (num_heads + 2 * num_kv_heads) * 128, M <= 64, N % 128 == 0,
+ * group_size % 128 == 0; cos_sin fp32 [max_positions, 128] (64 cosines, 64 sines); workspace as for
+ * awq_gemv(M, N, K).  Same arithmetic as awq_gemv followed by nq_qk_norm_rope_store (include/nq_engine_ops.h):
+ * Qwen3QuantizedAttention.forward, nanoquantization/models/qwen3_quantized.py:79-92. */
+int awq_gemv_qkv_rope_store(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                            const void* q_weight, const void* k_weight, const float* cos_sin,
+                            const int64_t* positions, const int64_t* slots, void* q_out, void* k_cache,
+                            void* v_cache, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                            int64_t num_heads, int64_t num_kv_heads, int64_t max_positions, int64_t num_slots,
+                            int64_t block_size, float eps, int dtype, void* workspace, size_t workspace_bytes,
+                            void* stream);
+
 /* Optional hint for latency-bound decode loops: the next awq_gemv / awq_linear / awq_gemv_swiglu call of
  * the calling thread that takes the staged GEMV path and leaves compute units idle also launches a few
  * spare workgroups that read [ptr, ptr + bytes) -- meant to be the packed qweight of the launch AFTER it --

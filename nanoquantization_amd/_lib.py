@@ -36,6 +36,7 @@ SYMBOLS = {
     "awq_gemv_swiglu": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "awq_linear_swiglu": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "awq_linear_swiglu_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "awq_gemv_qkv_rope_store": (_int, [_vp] * 12 + [_i64] * 9 + [ctypes.c_float, _int, _vp, _sz, _vp]),
     "awq_prefetch_hint": (_int, [_vp, _sz]),
     "awq_gemm": (_int, _LINEAR_ARGS),
     "awq_linear": (_int, _LINEAR_ARGS),

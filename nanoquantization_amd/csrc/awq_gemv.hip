@@ -236,6 +236,85 @@ __device__ __forceinline__ void compute_chunk_bytes(const Chunk<1, CH, MT>& d, f
 // columns of the same outputs), a lane holds one word of a row, its neighbour (lane ^ 1) the partner
 // word.  out = dtype(SiLU(dtype(gate))) * dtype(up), written to y [M, N/2] by the gate lanes.  Every lane
 // of a pair must call this (the exchange is a cross-lane read).
+// Epilogue of the fused q|k|v projection of a decode step (act == 2): the 128 columns of a column tile are one
+// head (head_dim 128).  q and k heads: RMSNorm over the head, half-split rotary at the row's position; q goes
+// to q_out, k to its paged-cache slot; v heads are written to their cache slot as they are.  The arithmetic per
+// element is that of the stand-alone kernel behind nq_qk_norm_rope_store (the GEMV's fp32 sum is rounded to T first,
+// as a separate projection would round it).  Cache layout [blocks][kv heads][block_size][128].
+struct QkvEpilogue {
+    const uint16_t* q_weight;
+    const uint16_t* k_weight;
+    const float* cos_sin;        // [max_positions][128]: 64 cosines, then 64 sines
+    const int64_t* positions;    // [M]
+    const int64_t* slots;        // [M], negative = the row owns no cache slot
+    uint16_t* q_out;             // [M][nh][128]
+    uint16_t* k_cache;
+    uint16_t* v_cache;
+    int nh, nkv, max_positions, block_size;
+    int64_t num_slots;
+    float eps;
+};
+
+// The 16 lanes that hold the 16 words of (row m, head n0 / 128) call this together; `valid` masks the stores.
+template <typename T>
+__device__ __forceinline__ void qkv_rope_store(const float (&out)[8], int m, size_t n0, bool valid,
+                                               const QkvEpilogue& qe) {
+    const int head = (int)(n0 >> 7), dc = (int)((n0 & 127) >> 3);
+    const int row = valid ? m : 0;
+    float a[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[e] = T::to_f32(T::from_f32(out[e]));
+    const int64_t slot = qe.slots[row];
+    const bool slot_ok = slot >= 0 && slot < qe.num_slots;
+    const bool is_q = head < qe.nh, is_k = !is_q && head < qe.nh + qe.nkv;
+    if (!is_q && !is_k) {   // v (uniform over the 16 lanes: no shuffle below is reached by a partial group)
+        if (valid && slot_ok) {
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[i] = T::pack2(a[2 * i], a[2 * i + 1]);
+            *reinterpret_cast<u32x4*>(qe.v_cache + (((slot / qe.block_size) * qe.nkv + (head - qe.nh - qe.nkv)) *
+                                                        qe.block_size + slot % qe.block_size) * 128 + dc * 8) = o;
+        }
+        return;
+    }
+    const uint16_t* w = is_q ? qe.q_weight : qe.k_weight;
+    const u32x4 wraw = *reinterpret_cast<const u32x4*>(w + dc * 8);
+    int64_t pos = qe.positions[row];
+    pos = pos < 0 ? 0 : (pos >= qe.max_positions ? qe.max_positions - 1 : pos);
+    const int i0 = (dc & 7) * 8;
+    const float* cs = qe.cos_sin + pos * 128;
+    const f32x4 c0 = *reinterpret_cast<const f32x4*>(cs + i0), c1 = *reinterpret_cast<const f32x4*>(cs + i0 + 4);
+    const f32x4 s0 = *reinterpret_cast<const f32x4*>(cs + 64 + i0), s1 = *reinterpret_cast<const f32x4*>(cs + 64 + i0 + 4);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += a[e] * a[e];
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
+    const float r = rsqrtf(ss / 128.f + qe.eps);
+    const bool first = dc < 8;
+    uint32_t packed[4];
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float wf = T::to_f32((uint16_t)((e & 1) ? wraw[e >> 1] >> 16 : wraw[e >> 1] & 0xFFFFu));
+        const float xn = T::to_f32(T::from_f32(T::to_f32(T::from_f32(a[e] * r)) * wf));
+        const float other = __shfl_xor(xn, 8);
+        const float cc = e < 4 ? c0[e] : c1[e - 4], sn = e < 4 ? s0[e] : s1[e - 4];
+        const float x1 = first ? xn : other, x2 = first ? other : xn;
+        y[e] = first ? __fsub_rn(__fmul_rn(x1, cc), __fmul_rn(x2, sn)) : __fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cc));
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) packed[i] = T::pack2(y[2 * i], y[2 * i + 1]);
+    const u32x4 o = u32x4{packed[0], packed[1], packed[2], packed[3]};
+    if (!valid) return;
+    if (is_q) {
+        *reinterpret_cast<u32x4*>(qe.q_out + ((int64_t)m * qe.nh + head) * 128 + dc * 8) = o;
+    } else if (slot_ok) {
+        *reinterpret_cast<u32x4*>(qe.k_cache + (((slot / qe.block_size) * qe.nkv + (head - qe.nh)) * qe.block_size +
+                                                slot % qe.block_size) * 128 + dc * 8) = o;
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ void swiglu_store(const float (&out)[8], uint16_t* __restrict__ y, int m, int N,
                                              size_t n0) {
@@ -265,7 +344,7 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
                                                   int wave, int group, int split, int splits,
                                                   const uint16_t* __restrict__ bias,
                                                   uint16_t* __restrict__ y, float* __restrict__ partials,
-                                                  int M, int N, int act) {
+                                                  int M, int N, int act, const QkvEpilogue* qe = nullptr) {
     constexpr int NF = 8 * V, NQ = 4 * V;
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
@@ -306,6 +385,10 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
 #pragma unroll
                         for (int c = 0; c < 8; ++c) out[c] = acc[vv * 8 + c][rr];
         }
+        if (splits == 1 && act == 2) {   // every lane takes part (cross-lane sums); the stores are masked
+            qkv_rope_store<T>(out, m, ((size_t)wv_col * V + v) * 8, m < M && col_ok, *qe);
+            continue;
+        }
         if (m < M && col_ok) {
             const size_t n0 = ((size_t)wv_col * V + v) * 8;
             if (splits == 1 && act) {
@@ -339,7 +422,8 @@ template <typename T, int V, int WN, int WK>
 __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int splits,
                                                 const uint16_t* __restrict__ bias,
                                                 uint16_t* __restrict__ y, float* __restrict__ partials,
-                                                int* __restrict__ counters, int M, int N, int act) {
+                                                int* __restrict__ counters, int M, int N, int act,
+                                                const QkvEpilogue* qe = nullptr) {
     constexpr int WAVES = WN * WK;
     const int words = N >> 3;
     if (!arrive_last(&counters[group], splits, s_last)) return;
@@ -371,6 +455,10 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
                     }
                 }
         }
+        if (act == 2) {   // w_count == 16 here: the 16 lanes of a head run the same iterations
+            qkv_rope_store<T>(out, m, n0, true, *qe);
+            continue;
+        }
         if (act) {   // w_count is even here: a gate word and its up word sit in neighbouring lanes
             swiglu_store<T>(out, y, m, N, n0);
             continue;
@@ -399,7 +487,8 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* re
                                               int wave, int group, int split, int splits,
                                               const uint16_t* __restrict__ bias,
                                               uint16_t* __restrict__ y, float* __restrict__ partials,
-                                              int* __restrict__ counters, int M, int N, int act = 0) {
+                                              int* __restrict__ counters, int M, int N, int act = 0,
+                                              const QkvEpilogue* qe = nullptr) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (mt > 0) {
@@ -407,10 +496,10 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* re
             __syncthreads();          // the reduction buffer is reused per m-tile
         }
         gemv_reduce_store<T, V, WN, WK>(acc[mt], 16 * mt, red, lane, wave, group, split, splits, bias, y,
-                                        partials, M, N, act);
+                                        partials, M, N, act, qe);
     }
     if (splits == 1) return;
-    gemv_split_tail<T, V, WN, WK>(s_last, group, splits, bias, y, partials, counters, M, N, act);
+    gemv_split_tail<T, V, WN, WK>(s_last, group, splits, bias, y, partials, counters, M, N, act, qe);
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
@@ -525,7 +614,7 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
-    int splits, int act, int groups, PrefetchRegions pf) {
+    int splits, int act, int groups, PrefetchRegions pf, QkvEpilogue qe) {
     constexpr int CH = 4;
     extern __shared__ float red[];  // staging while streaming, [WAVES][32][64] floats afterwards
     __shared__ int s_last;
@@ -564,6 +653,11 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         partials += (size_t)rb * splits * 16 * N;
         counters += rb * groups;
         M = min(16, M - 16 * rb);
+        if (act == 2) {
+            qe.positions += rb * 16;
+            qe.slots += rb * 16;
+            qe.q_out += (size_t)rb * 16 * qe.nh * 128;
+        }
     }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -688,7 +782,7 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     }
     __syncthreads();  // staging area becomes the reduction buffer
     gemv_epilogue<T, 1, WN, WK, MT>(acc, red, &s_last, lane, wave, group, split, splits, bias, y, partials,
-                                counters, M, N, act);
+                                counters, M, N, act, &qe);
 }
 
 // ---- data path 3: a workgroup of eight waves shares one staged chunk --------------------------
@@ -968,7 +1062,8 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
 template <typename T, int WN, int WK, int DEPTH, int MT>
 static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
-                                  int g, void* workspace, int split_k, hipStream_t stream, int act) {
+                                  int g, void* workspace, int split_k, hipStream_t stream, int act,
+                                  const QkvEpilogue* qe = nullptr) {
     constexpr int WAVES = WN * WK;
     const int groups = N / (128 * WN);
     const int total_chunks = K / 128;
@@ -1018,7 +1113,8 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
                        reinterpret_cast<const uint16_t*>(qscales),
                        reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
-                       partials, counters, M, N, K, g / 128, cps, splits, act, groups, pf);
+                       partials, counters, M, N, K, g / 128, cps, splits, act, groups, pf,
+                       qe ? *qe : QkvEpilogue{});
     return hipGetLastError();
 }
 
@@ -1090,7 +1186,8 @@ static int64_t balance_splits(int64_t chunks, int64_t s, int64_t wk, int64_t cap
     return best;
 }
 
-static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, int* split_k) {
+static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, int* split_k,
+                      bool allow_shared_chunk = true) {
     const int64_t chunks = K / 128 > 0 ? K / 128 : 1;
     if (N % 128 == 0 && g % 128 == 0) {
         // From sweeps on MI355X (HBM-streaming): short K runs best as one workgroup of 8 waves per
@@ -1100,7 +1197,8 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int v = 10 /* dma1x4d1 */;
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
-        if (M > 16 && N % 512 == 0 && N >= 5120 && K * N >= (M > 32 ? (50ll << 20) : (100ll << 20))) {
+        if (allow_shared_chunk && M > 16 && N % 512 == 0 && N >= 5120 &&
+            K * N >= (M > 32 ? (50ll << 20) : (100ll << 20))) {
             // 17..64 rows on the largest weights (from sweeps: Qwen3-32B MLP and, above 32 rows, its fused
             // q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
             // one workgroup per CU exists, four chunks per split at least.  Below these sizes re-reading the
@@ -1142,12 +1240,18 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
 static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, const void* qscales,
                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
-                         void* stream, int variant, int split_k, int act = 0) {
+                         void* stream, int variant, int split_k, int act = 0,
+                         const QkvEpilogue* qe = nullptr) {
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
     if (act && (variant < kFirstDmaVariant || bias)) {
         set_error("%s: the gated epilogue runs on the staged path only (N %% 128 == 0, group_size %% 128 == 0) "
                   "and takes no bias", fn);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    if (act == 2 && (!qe || kGemvVariants[variant < 0 || variant >= kNumGemvVariants ? 0 : variant].wide ||
+                     kGemvVariants[variant < 0 || variant >= kNumGemvVariants ? 0 : variant].wn != 1)) {
+        set_error("%s: the q|k|v epilogue runs on the one-tile-per-workgroup staged kernels only", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
     if (M > 64) {
@@ -1228,9 +1332,9 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     if (gv.wn == NN && gv.waves == NN * KK && gv.depth == DD && gv.mt == MM)                        \
         e = dtype == AWQ_F16                                                                        \
                 ? launch_gemv_dma<F16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                       (int)N, (int)K, (int)g, workspace, split_k, s, act) \
+                                                       (int)N, (int)K, (int)g, workspace, split_k, s, act, qe) \
                 : launch_gemv_dma<BF16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                        (int)N, (int)K, (int)g, workspace, split_k, s, act);
+                                                        (int)N, (int)K, (int)g, workspace, split_k, s, act, qe);
         AWQ_DMA_CASE(1, 4, 1, 1)
         AWQ_DMA_CASE(1, 8, 1, 1)
         AWQ_DMA_CASE(1, 16, 1, 1)
@@ -1309,6 +1413,52 @@ extern "C" int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void
     if (K >= 32 && N >= 8 && group_size > 0) awq::pick_gemv(M, N, K, group_size, &v, &s);
     return awq::gemv_dispatch("awq_gemv_swiglu", x, qweight, qscales, qzeros, nullptr, y, M, N, K, group_size,
                               dtype, workspace, workspace_bytes, stream, v, s, 1);
+}
+
+extern "C" int awq_gemv_qkv_rope_store(const void* x, const int32_t* qweight, const void* qscales,
+                                       const int32_t* qzeros, const void* q_weight, const void* k_weight,
+                                       const float* cos_sin, const int64_t* positions, const int64_t* slots,
+                                       void* q_out, void* k_cache, void* v_cache, int64_t M, int64_t N, int64_t K,
+                                       int64_t group_size, int64_t num_heads, int64_t num_kv_heads,
+                                       int64_t max_positions, int64_t num_slots, int64_t block_size, float eps,
+                                       int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "awq_gemv_qkv_rope_store";
+    if (!q_weight || !k_weight || !cos_sin || !positions || !slots || !q_out || !k_cache || !v_cache) {
+        awq::set_error("%s: null pointer argument", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    if ((reinterpret_cast<uintptr_t>(q_weight) | reinterpret_cast<uintptr_t>(k_weight) |
+         reinterpret_cast<uintptr_t>(cos_sin) | reinterpret_cast<uintptr_t>(q_out) |
+         reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15u) {
+        awq::set_error("%s: every tensor must be 16-byte aligned", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    if (num_heads <= 0 || num_kv_heads <= 0 || N != (num_heads + 2 * num_kv_heads) * 128 || max_positions <= 0 ||
+        max_positions > 0x7fffffff || block_size <= 0 || block_size > 0x7fffffff || num_slots <= 0 ||
+        num_slots % block_size != 0) {
+        awq::set_error("%s: needs head_dim 128 (N == (num_heads + 2 * num_kv_heads) * 128), positive max_positions and "
+                       "block_size, and num_slots a multiple of block_size", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    awq::QkvEpilogue qe;
+    qe.q_weight = reinterpret_cast<const uint16_t*>(q_weight);
+    qe.k_weight = reinterpret_cast<const uint16_t*>(k_weight);
+    qe.cos_sin = cos_sin;
+    qe.positions = positions;
+    qe.slots = slots;
+    qe.q_out = reinterpret_cast<uint16_t*>(q_out);
+    qe.k_cache = reinterpret_cast<uint16_t*>(k_cache);
+    qe.v_cache = reinterpret_cast<uint16_t*>(v_cache);
+    qe.nh = (int)num_heads;
+    qe.nkv = (int)num_kv_heads;
+    qe.max_positions = (int)max_positions;
+    qe.block_size = (int)block_size;
+    qe.num_slots = num_slots;
+    qe.eps = eps;
+    int v = 0, s = 1;
+    if (K >= 32 && N >= 8 && group_size > 0) awq::pick_gemv(M, N, K, group_size, &v, &s, false);
+    return awq::gemv_dispatch(fn, x, qweight, qscales, qzeros, nullptr, q_out, M, N, K, group_size, dtype, workspace,
+                              workspace_bytes, stream, v, s, 2, &qe);
 }
 
 extern "C" int awq_gemv_ex(const void* x, const int32_t* qweight, const void* qscales,

@@ -92,6 +92,8 @@ class LLMEngine:
         self.gate_up_il = [ops.interleave_gate_up((l.mlp.gate_proj.qweight, l.mlp.gate_proj.qscales, l.mlp.gate_proj.qzeros),
                                                   (l.mlp.up_proj.qweight, l.mlp.up_proj.qscales, l.mlp.up_proj.qzeros))
                            for l in layers] if self.swiglu_ok else None
+        q0 = layers[0].self_attn.q_proj
+        self.qkv_fused_ok = (self.hd == 128 and max_batch <= 64 and q0.group_size % 128 == 0 and q0.bias is None)
         self.use_graph = use_graph
         self._graph = None
         B, dev = max_batch, self.device
@@ -160,9 +162,15 @@ class LLMEngine:
             # every AWQ launch also pulls the next launch's packed weights and scales towards the Infinity Cache
             # (the small zero-point tensor measured as a net loss)
             prefetch_hint(attn.o_proj.qweight, attn.o_proj.qscales)
-            q = ops.qk_norm_rope_store(self.qkv[li](h), attn.q_norm.weight, attn.k_norm.weight,
-                                       attn.rope.cos_sin_cache, pos, slots, self.cache.k[li], self.cache.v[li],
-                                       self.nh, self.nkv, self.hd, attn.q_norm.eps)
+            if self.qkv_fused_ok:   # projection, q/k norm, rotary and cache write in one launch
+                lin = self.qkv[li]
+                q = ops.awq_gemv_qkv_rope_store(h, lin.qweight, lin.qscales, lin.qzeros, attn.q_norm.weight,
+                                                attn.k_norm.weight, attn.rope.cos_sin_cache, pos, slots,
+                                                self.cache.k[li], self.cache.v[li], self.nh, self.nkv, attn.q_norm.eps)
+            else:
+                q = ops.qk_norm_rope_store(self.qkv[li](h), attn.q_norm.weight, attn.k_norm.weight,
+                                           attn.rope.cos_sin_cache, pos, slots, self.cache.k[li], self.cache.v[li],
+                                           self.nh, self.nkv, self.hd, attn.q_norm.eps)
             o = ops.paged_attention_decode(q, self.cache.k[li], self.cache.v[li], self.s_table, ctx, self.scale)
             prefetch_hint(*gu)
             h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)

@@ -69,6 +69,41 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torc
     return (q, k) if dense_k else q
 
 
+def awq_gemv_qkv_rope_store(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor,
+                            q_weight: torch.Tensor, k_weight: torch.Tensor, cos_sin: torch.Tensor,
+                            positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                            num_heads: int, num_kv_heads: int, eps: float) -> torch.Tensor:
+    """Fused q|k|v projection of x [M <= 64, K] + q/k RMSNorm + rotary + cache write (head_dim 128): returns
+    q [M, nh, 128]; k and v go to their cache slots."""
+    dev = _dev(x, qweight, qscales, qzeros, q_weight, k_weight, cos_sin, positions, slots, k_cache, v_cache)
+    M, K = x.shape
+    N = qscales.shape[1]
+    g = K // qscales.shape[0]
+    hd = 128
+    assert N == (num_heads + 2 * num_kv_heads) * hd
+    assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    assert q_weight.shape == (hd,) and k_weight.shape == (hd,) and q_weight.dtype == x.dtype and k_weight.dtype == x.dtype
+    assert k_cache.dtype == x.dtype and v_cache.dtype == x.dtype and k_cache.shape == v_cache.shape
+    assert k_cache.dim() == 4 and k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == hd
+    assert cos_sin.dtype == torch.float32 and cos_sin.numel() % hd == 0
+    assert positions.dtype == torch.int64 and slots.dtype == torch.int64 and positions.numel() == M and slots.numel() == M
+    block_size = k_cache.shape[2]
+    num_slots = k_cache.numel() // (num_kv_heads * hd)
+    q = torch.empty(M, num_heads, hd, dtype=x.dtype, device=dev)
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        stream = _stream()
+        nbytes = L.awq_gemv_workspace_bytes(M, N, K)
+        ws = _lib.workspace(dev, stream, nbytes)
+        _lib.check(L.awq_gemv_qkv_rope_store(
+            x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(), q_weight.data_ptr(),
+            k_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(), slots.data_ptr(), q.data_ptr(),
+            k_cache.data_ptr(), v_cache.data_ptr(), M, N, K, g, num_heads, num_kv_heads, cos_sin.numel() // hd,
+            num_slots, block_size, eps, _lib.dtype_id(x.dtype), None if ws is None else ws.data_ptr(),
+            0 if ws is None else ws.numel(), stream))
+    return q
+
+
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                            context_lens: torch.Tensor, scale: float) -> torch.Tensor:
     """q [batch, nh, hd]; caches [num_blocks, nkv, block_size, hd]; block_table int32 [batch, max_blocks];

@@ -91,6 +91,48 @@ def test_qk_norm_rope_store(dtype, nh, nkv, hd):
     assert not by_slot(kc)[untouched].any() and not by_slot(vc)[untouched].any(), "other slots must stay untouched"
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,nh,nkv", [(1, 1024, 16, 8), (32, 1024, 16, 8), (64, 1024, 16, 8), (5, 3072, 4, 2),
+                                        (40, 5120, 64, 8), (16, 2048, 8, 8)])
+def test_gemv_qkv_rope_store_equals_unfused(dtype, M, K, nh, nkv):
+    """Projection + q/k norm + rotary + cache write in one launch against the GEMV followed by the stand-alone
+    kernel: v (a plain copy of the projection) bit for bit; q and k within one rounding step (the per-head sum of
+    squares is added up in another order)."""
+    import nanoquantization_amd as nq
+    from nanoquantization_amd.engine import ops
+    from nanoquantization_amd.layers.rope import RoPE
+    hd, bs, max_pos = 128, 16, 512
+    num_slots = 256
+    N = (nh + 2 * nkv) * hd
+    g = torch.Generator(device="cuda").manual_seed(M * 131 + K + nh)
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    qs = (torch.rand(K // 128, N, device="cuda", generator=g) * 0.02 + 0.001).to(dtype)
+    qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    x = (torch.randn(M, K, device="cuda", generator=g) * 0.3).to(dtype)
+    nqw = (1 + 0.1 * torch.randn(hd, device="cuda", generator=g)).to(dtype)
+    nkw = (1 + 0.1 * torch.randn(hd, device="cuda", generator=g)).to(dtype)
+    pos = torch.randint(0, max_pos, (M,), device="cuda", generator=g)
+    slots = torch.randperm(num_slots, device="cuda", generator=g)[:M]
+    if M > 3:
+        slots[3] = -1
+    rope = RoPE(hd, max_pos).cuda()
+    print(f"gemv_qkv_rope_store M={M} K={K} nh={nh} nkv={nkv} {dtype}", flush=True)
+    kc = torch.zeros(num_slots // bs, nkv, bs, hd, dtype=dtype, device="cuda")
+    vc = torch.zeros_like(kc)
+    q = ops.awq_gemv_qkv_rope_store(x, qw, qs, qz, nqw, nkw, rope.cos_sin_cache, pos, slots, kc, vc, nh, nkv, 1e-6)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    q2 = ops.qk_norm_rope_store(nq.awq_gemm(x, qw, qs, qz, 8), nqw, nkw, rope.cos_sin_cache, pos, slots, kc2, vc2,
+                                nh, nkv, hd, 1e-6)
+    if M > 32 and K * N >= 50 << 20:
+        _close(vc, vc2.float(), dtype, what="v cache")   # the plain projection runs the shared-chunk kernel here: another sum order
+    else:
+        assert torch.equal(vc, vc2), "v is the projection itself"
+    _close(q, q2.float(), dtype, what="q")
+    _close(kc, kc2.float(), dtype, what="k cache")
+    assert torch.equal(q, ops.awq_gemv_qkv_rope_store(x, qw, qs, qz, nqw, nkw, rope.cos_sin_cache, pos, slots,
+                                                      torch.zeros_like(kc), torch.zeros_like(vc), nh, nkv, 1e-6))
+
+
 def _attn_ref(q, kc, vc, table, ctx, scale):
     B, nh, hd = q.shape
     nb, nkv, bs, _ = kc.shape
