@@ -339,7 +339,7 @@ __device__ __forceinline__ void swiglu_store(const float (&out)[8], uint16_t* __
 }
 
 // kPlain: the partials are read by a later kernel, not by a concurrent workgroup: ordinary stores do.
-template <typename T, int V, int WN, int WK, bool kPlain = false>
+template <typename T, int V, int WN, int WK, bool kPlain = false, bool kQkv = false>
 __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_base, float* red, int lane,
                                                   int wave, int group, int split, int splits,
                                                   const uint16_t* __restrict__ bias,
@@ -385,9 +385,11 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
 #pragma unroll
                         for (int c = 0; c < 8; ++c) out[c] = acc[vv * 8 + c][rr];
         }
-        if (splits == 1 && act == 2) {   // every lane takes part (cross-lane sums); the stores are masked
-            qkv_rope_store<T>(out, m, ((size_t)wv_col * V + v) * 8, m < M && col_ok, *qe);
-            continue;
+        if constexpr (kQkv) {
+            if (splits == 1) {   // every lane takes part (cross-lane sums); the stores are masked
+                qkv_rope_store<T>(out, m, ((size_t)wv_col * V + v) * 8, m < M && col_ok, *qe);
+                continue;
+            }
         }
         if (m < M && col_ok) {
             const size_t n0 = ((size_t)wv_col * V + v) * 8;
@@ -418,7 +420,7 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
     }
 }
 
-template <typename T, int V, int WN, int WK>
+template <typename T, int V, int WN, int WK, bool kQkv = false>
 __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int splits,
                                                 const uint16_t* __restrict__ bias,
                                                 uint16_t* __restrict__ y, float* __restrict__ partials,
@@ -455,7 +457,7 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
                     }
                 }
         }
-        if (act == 2) {   // w_count == 16 here: the 16 lanes of a head run the same iterations
+        if constexpr (kQkv) {   // w_count == 16 here: the 16 lanes of a head run the same iterations
             qkv_rope_store<T>(out, m, n0, true, *qe);
             continue;
         }
@@ -482,7 +484,7 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
 // (fixed order), then either store y (splits == 1) or publish this split's
 // partial and let the last workgroup of the tile group add the partials in
 // split order.  `group` is the workgroup's index along N.
-template <typename T, int V, int WN, int WK, int MT = 1>
+template <typename T, int V, int WN, int WK, int MT = 1, bool kQkv = false>
 __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* red, int* s_last, int lane,
                                               int wave, int group, int split, int splits,
                                               const uint16_t* __restrict__ bias,
@@ -495,11 +497,11 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* re
             if (16 * mt >= M) break;  // uniform
             __syncthreads();          // the reduction buffer is reused per m-tile
         }
-        gemv_reduce_store<T, V, WN, WK>(acc[mt], 16 * mt, red, lane, wave, group, split, splits, bias, y,
-                                        partials, M, N, act, qe);
+        gemv_reduce_store<T, V, WN, WK, false, kQkv>(acc[mt], 16 * mt, red, lane, wave, group, split, splits, bias,
+                                                     y, partials, M, N, act, qe);
     }
     if (splits == 1) return;
-    gemv_split_tail<T, V, WN, WK>(s_last, group, splits, bias, y, partials, counters, M, N, act, qe);
+    gemv_split_tail<T, V, WN, WK, kQkv>(s_last, group, splits, bias, y, partials, counters, M, N, act, qe);
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
@@ -608,15 +610,19 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
 
 __host__ __device__ constexpr int dma_wave_bytes(int M) { return 8192 + 256 * M + 512; }
 
-template <typename T, int WN, int WK, int DEPTH, int MT = 1>
-__global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
+struct NoEpilogue {};
+
+// QKV: the kernel behind awq_gemv_qkv_rope_store; its extra arguments stay out of the plain kernel's argument
+// block (the launch-bound decode GEMVs measured 0.2-0.5 us slower with them).
+template <typename T, int WK, bool QKV = false>
+__global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
-    int splits, int act, int groups, PrefetchRegions pf, QkvEpilogue qe) {
+    int splits, int act, int groups, PrefetchRegions pf, std::conditional_t<QKV, QkvEpilogue, NoEpilogue> qe) {
     constexpr int CH = 4;
-    extern __shared__ float red[];  // staging while streaming, [WAVES][32][64] floats afterwards
+    extern __shared__ float red[];  // staging while streaming, [WK][32][64] floats afterwards
     __shared__ int s_last;
     if ((int)blockIdx.x >= groups) {
         if (blockIdx.y != 0 || blockIdx.z != 0) return;   // the extra workgroups exist once per split and row block; one set works
@@ -643,17 +649,17 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         return;
     }
 
-    if constexpr (MT == 1) {
+    {
         // More than 16 rows: blockIdx.z picks a block of 16 rows, an independent product with its own slice of
         // x, y, the partials and the arrival counters.  The weights are then read once per row block, the
         // later ones mostly from cache: worthwhile where a launch is latency-bound, not on large weights.
         const int rb = blockIdx.z;
         x += (size_t)rb * 16 * K;
-        y += (size_t)rb * 16 * (act ? N >> 1 : N);
+        y += (size_t)rb * 16 * (act == 1 ? N >> 1 : N);
         partials += (size_t)rb * splits * 16 * N;
         counters += rb * groups;
         M = min(16, M - 16 * rb);
-        if (act == 2) {
+        if constexpr (QKV) {
             qe.positions += rb * 16;
             qe.slots += rb * 16;
             qe.q_out += (size_t)rb * 16 * qe.nh * 128;
@@ -663,19 +669,17 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
-    const int group = xcd_aware_group(blockIdx.x, groups), split = blockIdx.y;
-    const int tile = group * WN + wave % WN;   // host guarantees N % (128 * WN) == 0
+    const int tile = xcd_aware_group(blockIdx.x, groups), split = blockIdx.y;   // host guarantees N % 128 == 0
 
     const int total_chunks = K / 128;
     const int c_begin = split * chunks_per_split;
     const int c_end = min(c_begin + chunks_per_split, total_chunks);
     const int per_wave = (max(c_end - c_begin, 0) + WK - 1) / WK;
-    const int c0 = c_begin + (wave / WN) * per_wave;
+    const int c0 = c_begin + wave * per_wave;
     const int c1 = min(c0 + per_wave, c_end);
 
-    // DEPTH staging buffers per wave: chunk c lives in buffer (c - c0) % DEPTH
-    const int buf_bytes = dma_wave_bytes(M);
-    char* stage = reinterpret_cast<char*>(red) + (size_t)wave * (DEPTH * buf_bytes);
+    // one staging buffer per wave
+    char* stage = reinterpret_cast<char*>(red) + (size_t)wave * dma_wave_bytes(M);
     const int x_off = 8192, zs_off = 8192 + 256 * M;
 
     // DMA lane roles
@@ -686,29 +690,15 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
         const int slot = h * 16 + dsl;
         wsrc[h] = (uint32_t)((slot & 3) * 8 + (slot >> 2)) * (uint32_t)words + (uint32_t)(tile * 16 + dq * 4);
     }
-    // x: per m-tile one DMA instruction per step; lane = (m - 16*mt)*4 + k-block
-    static_assert(MT == 1 || DEPTH == 1, "the vmcnt arithmetic of deeper pipelines assumes one m-tile");
-    bool x_lane[MT];
-    uint32_t xsrc[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = 16 * mt + (lane >> 2);
-        x_lane[mt] = m < M;
-        xsrc[mt] = (uint32_t)(x_lane[mt] ? m : 0) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
-    }
+    // x: one DMA instruction per step; lane = m * 4 + k-block
+    const bool x_lane = (lane >> 2) < M;
+    const uint32_t xsrc = (uint32_t)(x_lane ? lane >> 2 : 0) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
     const bool zs_lane = lane < 16;
     const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
 
-    // exactly kDmaOps vector-memory instructions per call (the vmcnt arithmetic below counts on it):
-    // lanes 0..3 and 0..15 exist in every wave, so neither guarded block is ever skipped
-    constexpr int kDmaOps = 2 * CH + CH + 2;
-    static_assert(kDmaOps == 14, "vmcnt immediates below assume 14 DMA instructions per chunk (one m-tile)");
-    auto issue_dma = [&](int c, int buf) {
+    auto issue_dma = [&](int c) {
         const int row0 = c * 128;
-        char* base = stage + buf * buf_bytes;
-        uint32_t* w_lds = reinterpret_cast<uint32_t*>(base);
-        char* x_lds = base + x_off;
-        char* zs_lds = base + zs_off;
+        uint32_t* w_lds = reinterpret_cast<uint32_t*>(stage);
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
             const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
@@ -717,72 +707,59 @@ __global__ __launch_bounds__(64 * WN * WK) void gemv_dma_kernel(
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
                                                  16, 0, 0);
         }
+        if (x_lane) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            if (x_lane[mt]) {
-#pragma unroll
-                for (int s = 0; s < CH; ++s)
-                    __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc[mt]),
-                                                     AWQ_LPTR(x_lds + s * 64 * M + mt * 1024), 16, 0, 0);
-            }
+            for (int s = 0; s < CH; ++s)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc),
+                                                 AWQ_LPTR(stage + x_off + s * 64 * M), 16, 0, 0);
+        }
         if (zs_lane) {
             const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
-            __builtin_amdgcn_global_load_lds(AWQ_GPTR(qzeros + (size_t)gi * words + zsrc), AWQ_LPTR(zs_lds), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(AWQ_GPTR(qzeros + (size_t)gi * words + zsrc), AWQ_LPTR(stage + zs_off),
+                                             4, 0, 0);
             __builtin_amdgcn_global_load_lds(AWQ_GPTR(scales + ((size_t)gi * words + zsrc) * 8),
-                                             AWQ_LPTR(zs_lds + 64), 16, 0, 0);
+                                             AWQ_LPTR(stage + zs_off + 64), 16, 0, 0);
         }
     };
 
-    // compute-lane read offsets inside a staging buffer (bytes)
-    const int w_rd_off = (kb * 16 + j) * 4;                   // + (s*512 + r*64) * 4
-    int x_rd_off[MT];                                         // + s * 64 * M
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) x_rd_off[mt] = x_off + (min(16 * mt + j, M - 1) * 4 + kb) * 16;
+    // compute-lane read offsets inside the staging buffer (bytes)
+    const uint32_t* w_rd = reinterpret_cast<const uint32_t*>(stage + (kb * 16 + j) * 4);   // + (s*512 + r*64) words
+    const int x_rd_off = x_off + (min(j, M - 1) * 4 + kb) * 16;                            // + s * 64 * M
     const int z_rd_off = zs_off + j * 4;
     const int s_rd_off = zs_off + 64 + j * 16;
 
-    f32x4 acc[MT][8];
+    f32x4 acc[1][8];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int f = 0; f < 8; ++f) acc[mt][f] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int f = 0; f < 8; ++f) acc[0][f] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d)
-        if (c0 + d < c1) issue_dma(c0 + d, d);
-    int buf = 0;
+    if (c0 < c1) issue_dma(c0);
     for (int c = c0; c < c1; ++c) {
-        // chunk c has landed once at most the DMA of the chunks issued after it is outstanding.
         // The compiler does not order LDS reads after the DMA by itself.
-        const int newer = min(c1 - 1 - c, DEPTH - 1);
-        if (DEPTH == 1 || newer == 0) __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
-        else if (newer == 1) __builtin_amdgcn_s_waitcnt(0x0F7E);                 // vmcnt(14)
-        else __builtin_amdgcn_s_waitcnt(0x4F7C);                                 // vmcnt(28)
+        __builtin_amdgcn_s_waitcnt(0x0F70);                                      // vmcnt(0): chunk c has landed
         asm volatile("" ::: "memory");
-        const char* base = stage + buf * buf_bytes;
-        const uint32_t* w_rd = reinterpret_cast<const uint32_t*>(base + w_rd_off);
-        Chunk<1, CH, MT> d;
+        Chunk<1, CH, 1> d;
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) d.w[s][r] = w_rd[s * 512 + r * 64];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                d.xa[s][mt] = *reinterpret_cast<const u32x4*>(base + x_rd_off[mt] + s * 64 * M);
+            d.xa[s][0] = *reinterpret_cast<const u32x4*>(stage + x_rd_off + s * 64 * M);
         }
-        d.zw = *reinterpret_cast<const uint32_t*>(base + z_rd_off);
-        d.sv[0] = *reinterpret_cast<const u32x4*>(base + s_rd_off);
-        // every LDS read has returned before a later chunk's DMA may overwrite this buffer
+        d.zw = *reinterpret_cast<const uint32_t*>(stage + z_rd_off);
+        d.sv[0] = *reinterpret_cast<const u32x4*>(stage + s_rd_off);
+        // every LDS read has returned before the next chunk's DMA may overwrite the buffer
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xC07F);                                      // lgkmcnt(0)
         asm volatile("" ::: "memory");
-        if (c + DEPTH < c1) issue_dma(c + DEPTH, buf);
-        buf = (buf + 1 == DEPTH) ? 0 : buf + 1;
-        compute_chunk<T, 1, CH, MT>(d, acc);
+        if (c + 1 < c1) issue_dma(c + 1);
+        compute_chunk<T, 1, CH, 1>(d, acc);
     }
     __syncthreads();  // staging area becomes the reduction buffer
-    gemv_epilogue<T, 1, WN, WK, MT>(acc, red, &s_last, lane, wave, group, split, splits, bias, y, partials,
-                                counters, M, N, act, &qe);
+    if constexpr (QKV)
+        gemv_epilogue<T, 1, 1, WK, 1, true>(acc, red, &s_last, lane, wave, tile, split, splits, bias, y, partials,
+                                            counters, M, N, act, &qe);
+    else
+        gemv_epilogue<T, 1, 1, WK, 1>(acc, red, &s_last, lane, wave, tile, split, splits, bias, y, partials,
+                                      counters, M, N, act);
 }
 
 // ---- data path 3: a workgroup of eight waves shares one staged chunk --------------------------
@@ -1003,22 +980,19 @@ struct GemvVariant {
     bool wide;  // a workgroup of eight waves shares one staged chunk (gemv_wide_kernel)
 };
 static const GemvVariant kGemvVariants[] = {
-    {"v1w4p", 1, 4, true, 1, 0, 1},  {"v1w8p", 1, 8, true, 1, 0, 1},   {"v2w4", 2, 4, false, 1, 0, 1},
-    {"v2w8", 2, 8, false, 1, 0, 1},  {"v2w4p", 2, 4, true, 1, 0, 1},   {"v1w16", 1, 16, false, 1, 0, 1},
-    {"v1w1p", 1, 1, true, 1, 0, 1},  {"v2w1", 2, 1, false, 1, 0, 1},   {"v1w4", 1, 4, false, 1, 0, 1},
-    {"v1w8", 1, 8, false, 1, 0, 1},
-    // DMA variants, named dma<WN>x<WK>d<DEPTH>[m<MT>]
-    {"dma1x4d1", 1, 4, false, 1, 1, 1},  {"dma1x8d1", 1, 8, false, 1, 1, 1},  {"dma1x16d1", 1, 16, false, 1, 1, 1},
-    {"dma1x4d2", 1, 4, false, 1, 2, 1},  {"dma1x8d2", 1, 8, false, 1, 2, 1},  {"dma1x4d3", 1, 4, false, 1, 3, 1},
-    {"dma2x4d1", 1, 8, false, 2, 1, 1},  {"dma2x4d2", 1, 8, false, 2, 2, 1},  {"dma1x1d1", 1, 1, false, 1, 1, 1},
-    {"dma1x2d2", 1, 2, false, 1, 2, 1},
-    {"dma1x4d1m2", 1, 4, false, 1, 1, 2}, {"dma1x8d1m2", 1, 8, false, 1, 1, 2}, {"dma1x4d1m4", 1, 4, false, 1, 1, 4},
+    // register path, named v<V>w<waves>[p = next chunk prefetched]
+    {"v1w4p", 1, 4, true, 1, 0, 1},
+    {"v2w4", 2, 4, false, 1, 0, 1},
+    // staged (DMA) path, one column tile per workgroup, named dma1x<WK>; 17..64 rows run as blocks of 16 (grid z)
+    {"dma1x4", 1, 4, false, 1, 1, 1},
+    {"dma1x8", 1, 8, false, 1, 1, 1},
     // shared staged chunk, eight waves as 4 column tiles x 2 byte halves: wide d<DEPTH> m<MT>
-    {"wided3m4", 1, 8, false, 4, 3, 4, true}, {"wided2m4", 1, 8, false, 4, 2, 4, true},
-    {"wided3m2", 1, 8, false, 4, 3, 2, true}, {"wided2m2", 1, 8, false, 4, 2, 2, true},
+    {"wided2m4", 1, 8, false, 4, 2, 4, true},
+    {"wided2m2", 1, 8, false, 4, 2, 2, true},
 };
+enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
-constexpr int kFirstDmaVariant = 10;
+constexpr int kFirstDmaVariant = kDma1x4;
 
 // rows per chunk: 128 when the group size allows it, else 32
 static inline int chunk_steps(int64_t g) { return g % 128 == 0 ? 4 : 1; }
@@ -1059,13 +1033,12 @@ static hipError_t launch_gemv(const void* x, const int32_t* qweight, const void*
     return hipGetLastError();
 }
 
-template <typename T, int WN, int WK, int DEPTH, int MT>
+template <typename T, int WK>
 static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                                   int g, void* workspace, int split_k, hipStream_t stream, int act,
                                   const QkvEpilogue* qe = nullptr) {
-    constexpr int WAVES = WN * WK;
-    const int groups = N / (128 * WN);
+    const int groups = N / 128;
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
     const int splits = (int)cdiv(total_chunks, cps);
@@ -1073,19 +1046,19 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
                                                             kCounterBytes)
                                 : nullptr;
-    size_t lds = (size_t)WAVES * DEPTH * dma_wave_bytes(MT == 1 && M > 16 ? 16 : M);
-    const size_t red_bytes = WK > 1 ? (size_t)WAVES * 32 * 64 * sizeof(float) : 0;
+    const int row_blocks = (int)cdiv(M, 16);   // 17..64 rows: independent blocks of 16 rows along grid z
+    size_t lds = (size_t)WK * dma_wave_bytes(M > 16 ? 16 : M);
+    const size_t red_bytes = (size_t)WK * 32 * 64 * sizeof(float);
     if (lds < red_bytes) lds = red_bytes;
-    auto kern = gemv_dma_kernel<T, WN, WK, DEPTH, MT>;
-    // what the largest M that still fits asks for (the dispatcher rejects bigger requests)
-    constexpr size_t kLdsCap = 160 * 1024 - 1024;
-    constexpr size_t kWant = (size_t)WAVES * DEPTH * dma_wave_bytes(16 * MT);
-    constexpr size_t kMaxLds = kWant < kLdsCap ? kWant : kLdsCap;
+    constexpr size_t kMaxLds = (size_t)WK * dma_wave_bytes(16);
     if (kMaxLds > 64 * 1024) {
-        static bool raised = false;  // once per process and instantiation
+        static bool raised = false;  // once per process and instantiation (both forms of the kernel)
         if (!raised) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, false>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
+            if (e == hipSuccess)
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
             if (e != hipSuccess) return e;
             raised = true;
         }
@@ -1097,24 +1070,28 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     long long pf_bytes = 0;
     for (int r = 0; r < pf.count; ++r) pf_bytes += pf.bytes[r];
     int pf_wgs = 0;
-    const int row_blocks = MT == 1 ? (int)cdiv(M, 16) : 1;
     const long long compute_wgs = (long long)groups * splits * row_blocks;
     if (pf_bytes >= 128 && compute_wgs < 192) {
-        const long long want = cdiv(pf_bytes >> 7, 64 * WAVES * 2);   // about 2 lines per thread
+        const long long want = cdiv(pf_bytes >> 7, 64 * WK * 2);   // about 2 lines per thread
         const long long room = (256 - compute_wgs) / ((long long)splits * row_blocks);   // stay within one wave of workgroups
         pf_wgs = (int)(want < room ? want : room);
         if (pf_wgs < 1) pf_wgs = 1;
     } else {
         pf.count = 0;
     }
-    hipLaunchKernelGGL(kern, dim3(groups + pf_wgs, splits, row_blocks), dim3(64 * WAVES), lds, stream,
-                       reinterpret_cast<const uint16_t*>(x),
-                       reinterpret_cast<const uint32_t*>(qweight),
-                       reinterpret_cast<const uint16_t*>(qscales),
-                       reinterpret_cast<const uint32_t*>(qzeros),
-                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y),
-                       partials, counters, M, N, K, g / 128, cps, splits, act, groups, pf,
-                       qe ? *qe : QkvEpilogue{});
+    const dim3 grid(groups + pf_wgs, splits, row_blocks), block(64 * WK);
+    if (qe)
+        hipLaunchKernelGGL((gemv_dma_kernel<T, WK, true>), grid, block, lds, stream,
+                           reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
+                           reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
+                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
+                           M, N, K, g / 128, cps, splits, act, groups, pf, *qe);
+    else
+        hipLaunchKernelGGL((gemv_dma_kernel<T, WK, false>), grid, block, lds, stream,
+                           reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
+                           reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
+                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
+                           M, N, K, g / 128, cps, splits, act, groups, pf, NoEpilogue{});
     return hipGetLastError();
 }
 
@@ -1194,7 +1171,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         // column tile; otherwise 4-wave workgroups, split over K for M <= 4 until ~3000 waves exist
         // (the split's tail grows with M, so larger M splits only to cover the CUs).
         const int64_t tiles = N / 128;
-        int v = 10 /* dma1x4d1 */;
+        int v = kDma1x4;
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
         if (allow_shared_chunk && M > 16 && N % 512 == 0 && N >= 5120 &&
@@ -1203,11 +1180,11 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             // q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
             // one workgroup per CU exists, four chunks per split at least.  Below these sizes re-reading the
             // weights once per block of 16 rows (mostly from cache) is faster than the shared chunk's second pass.
-            v = M > 32 ? 24 /* wided2m4 */ : 26 /* wided2m2 */;
+            v = M > 32 ? kWideM4 : kWideM2;
             s = 256 / (N / 512);
             if (s > chunks / 4) s = chunks / 4;
         } else if (chunks <= 8) {
-            v = 11 /* dma1x8d1 */;
+            v = kDma1x8;
         } else if (M <= 4) {
             s = cdiv(3072, tiles * 4);
             // short K: at most 10 splits (the tail is a larger share of a 6 us launch); long K: up to 32
@@ -1225,7 +1202,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         return;
     }
     const bool wide = (N % 16 == 0) && N >= 4096;
-    const int v = wide ? 2 /* v2w4 */ : 0 /* v1w4p */;
+    const int v = wide ? kV2W4 : kV1W4P;
     const GemvVariant& gv = kGemvVariants[v];
     const int64_t tiles = cdiv(N / 8, 16 * gv.V);
     int64_t s = cdiv(512, tiles);
@@ -1271,8 +1248,9 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         return AWQ_ERR_INVALID_ARG;
     }
     const GemvVariant& gv = kGemvVariants[variant];
-    // the staged one-m-tile variants take up to 64 rows as independent blocks of 16
-    const bool row_blocked = variant >= kFirstDmaVariant && !gv.wide && gv.mt == 1;
+    const bool staged = variant >= kFirstDmaVariant;
+    // 17..64 rows: blocks of 16 on the one-tile staged kernels, up to 16 * mt on the shared-chunk kernel
+    const bool row_blocked = staged && !gv.wide;
     if (M > 16 * gv.mt && !row_blocked) {
         set_error("%s: variant %s takes at most %d rows (M=%lld); rows 17..64 need the staged path "
                   "(N %% 128 == 0, group_size %% 128 == 0)", fn, gv.name, 16 * gv.mt, (long long)M);
@@ -1280,6 +1258,10 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     }
     if ((N / 8) % gv.V != 0) {
         set_error("%s: variant %s needs N %% %d == 0 (N=%lld)", fn, gv.name, 8 * gv.V, (long long)N);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    if (staged && (N % (128 * gv.wn) != 0 || g % 128 != 0)) {
+        set_error("%s: variant %s needs N %% %d == 0 and group_size %% 128 == 0", fn, gv.name, 128 * gv.wn);
         return AWQ_ERR_UNSUPPORTED;
     }
     if (split_k > 1 && cdiv(N / 8, 16 * gv.V) * (row_blocked ? cdiv(M, 16) : 1) > kMaxSplitTiles) {
@@ -1295,88 +1277,39 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     if (need == 0) split_k = 1;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
-    const bool big_chunk = chunk_steps(g) == 4;
-    if (variant >= kFirstDmaVariant) {
-        if (N % (128 * gv.wn) != 0 || g % 128 != 0) {
-            set_error("%s: variant %s needs N %% %d == 0 and group_size %% 128 == 0", fn, gv.name, 128 * gv.wn);
-            return AWQ_ERR_UNSUPPORTED;
-        }
-        if (gv.wide) {
-            if (N % 512 != 0 || g % 128 != 0) {
-                set_error("%s: variant %s needs N %% 512 == 0 and group_size %% 128 == 0", fn, gv.name);
-                return AWQ_ERR_UNSUPPORTED;
-            }
-            if (split_k > 1 && N / 512 > kMaxSplitTiles) {
-                set_error("%s: split-K supports at most %lld column groups (N=%lld)", fn, (long long)kMaxSplitTiles,
-                          (long long)N);
-                return AWQ_ERR_UNSUPPORTED;
-            }
-#define AWQ_WIDE_CASE(DD, MM)                                                                              \
-    if (gv.depth == DD && gv.mt == MM)                                                                     \
-        e = dtype == AWQ_F16 ? launch_gemv_wide<F16, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                             (int)N, (int)K, (int)g, workspace, split_k, s, act) \
-                             : launch_gemv_wide<BF16, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                              (int)N, (int)K, (int)g, workspace, split_k, s, act);
-            AWQ_WIDE_CASE(3, 4)
-            AWQ_WIDE_CASE(2, 4)
-            AWQ_WIDE_CASE(3, 2)
-            AWQ_WIDE_CASE(2, 2)
-#undef AWQ_WIDE_CASE
-            return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
-        }
-        if ((size_t)gv.waves * gv.depth * dma_wave_bytes(row_blocked && M > 16 ? 16 : (int)M) > 160 * 1024 - 1024) {
-            set_error("%s: variant %s does not fit the LDS at M=%lld", fn, gv.name, (long long)M);
-            return AWQ_ERR_UNSUPPORTED;
-        }
-#define AWQ_DMA_CASE(NN, KK, DD, MM)                                                                \
-    if (gv.wn == NN && gv.waves == NN * KK && gv.depth == DD && gv.mt == MM)                        \
-        e = dtype == AWQ_F16                                                                        \
-                ? launch_gemv_dma<F16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                       (int)N, (int)K, (int)g, workspace, split_k, s, act, qe) \
-                : launch_gemv_dma<BF16, NN, KK, DD, MM>(x, qweight, qscales, qzeros, bias, y, (int)M, \
-                                                        (int)N, (int)K, (int)g, workspace, split_k, s, act, qe);
-        AWQ_DMA_CASE(1, 4, 1, 1)
-        AWQ_DMA_CASE(1, 8, 1, 1)
-        AWQ_DMA_CASE(1, 16, 1, 1)
-        AWQ_DMA_CASE(1, 4, 2, 1)
-        AWQ_DMA_CASE(1, 8, 2, 1)
-        AWQ_DMA_CASE(1, 4, 3, 1)
-        AWQ_DMA_CASE(2, 4, 1, 1)
-        AWQ_DMA_CASE(2, 4, 2, 1)
-        AWQ_DMA_CASE(1, 1, 1, 1)
-        AWQ_DMA_CASE(1, 2, 2, 1)
-        AWQ_DMA_CASE(1, 4, 1, 2)
-        AWQ_DMA_CASE(1, 8, 1, 2)
-        AWQ_DMA_CASE(1, 4, 1, 4)
-#undef AWQ_DMA_CASE
-        return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
-    }
-#define AWQ_GEMV_LAUNCH(TT, VV, WW, CC, PP)                                                        \
-    launch_gemv<TT, VV, WW, CC, PP>(x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, \
-                                    (int)g, workspace, split_k, s)
-#define AWQ_GEMV_CASE(IDX, VV, WW, PP)                                                     \
-    case IDX:                                                                              \
-        if (big_chunk)                                                                     \
-            e = dtype == AWQ_F16 ? AWQ_GEMV_LAUNCH(F16, VV, WW, 4, PP)                     \
-                                 : AWQ_GEMV_LAUNCH(BF16, VV, WW, 4, PP);                   \
-        else /* group sizes 32/64/96...: one 32-row step per chunk, no prefetch variant */ \
-            e = dtype == AWQ_F16 ? AWQ_GEMV_LAUNCH(F16, VV, WW, 1, true)                   \
-                                 : AWQ_GEMV_LAUNCH(BF16, VV, WW, 1, true);                 \
-        break;
+    const int Mi = (int)M, Ni = (int)N, Ki = (int)K, gi = (int)g;
+    const bool f16 = dtype == AWQ_F16;
     switch (variant) {
-        AWQ_GEMV_CASE(0, 1, 4, true)
-        AWQ_GEMV_CASE(1, 1, 8, true)
-        AWQ_GEMV_CASE(2, 2, 4, false)
-        AWQ_GEMV_CASE(3, 2, 8, false)
-        AWQ_GEMV_CASE(4, 2, 4, true)
-        AWQ_GEMV_CASE(5, 1, 16, false)
-        AWQ_GEMV_CASE(6, 1, 1, true)
-        AWQ_GEMV_CASE(7, 2, 1, false)
-        AWQ_GEMV_CASE(8, 1, 4, false)
-        AWQ_GEMV_CASE(9, 1, 8, false)
-    }
-#undef AWQ_GEMV_CASE
+        case kWideM4:
+            e = f16 ? launch_gemv_wide<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
+                    : launch_gemv_wide<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            break;
+        case kWideM2:
+            e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
+                    : launch_gemv_wide<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            break;
+        case kDma1x4:
+            e = f16 ? launch_gemv_dma<F16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe)
+                    : launch_gemv_dma<BF16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe);
+            break;
+        case kDma1x8:
+            e = f16 ? launch_gemv_dma<F16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe)
+                    : launch_gemv_dma<BF16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe);
+            break;
+        default: {
+            // register path; group sizes 32/64/96...: one 32-row step per chunk, always with the next chunk prefetched
+            const bool big_chunk = chunk_steps(g) == 4;
+#define AWQ_GEMV_LAUNCH(TT, VV, CC, PP) \
+    launch_gemv<TT, VV, 4, CC, PP>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s)
+            if (variant == kV1W4P)
+                e = big_chunk ? (f16 ? AWQ_GEMV_LAUNCH(F16, 1, 4, true) : AWQ_GEMV_LAUNCH(BF16, 1, 4, true))
+                              : (f16 ? AWQ_GEMV_LAUNCH(F16, 1, 1, true) : AWQ_GEMV_LAUNCH(BF16, 1, 1, true));
+            else
+                e = big_chunk ? (f16 ? AWQ_GEMV_LAUNCH(F16, 2, 4, false) : AWQ_GEMV_LAUNCH(BF16, 2, 4, false))
+                              : (f16 ? AWQ_GEMV_LAUNCH(F16, 2, 1, true) : AWQ_GEMV_LAUNCH(BF16, 2, 1, true));
 #undef AWQ_GEMV_LAUNCH
+        }
+    }
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }
 
