@@ -202,13 +202,15 @@ struct GemmVariant {
     int BM, BN, waves;
 };
 static const GemmVariant kGemmVariants[] = {
-    {"256x256w8", 256, 256, 8}, {"128x256w8", 128, 256, 8}, {"128x128", 128, 128, 4},
-    {"64x256", 64, 256, 4},     {"32x256", 32, 256, 4},     {"64x128", 64, 128, 4},
-    {"256x256", 256, 256, 4},   {"128x256", 128, 256, 4},   {"256x128w8", 256, 128, 8},
+    // narrow tiles of gemm_kernel for up to 128 rows (wider and 8-wave forms of it were measured and removed)
+    {"128x128", 128, 128, 4},
+    {"64x256", 64, 256, 4},
+    {"32x256", 32, 256, 4},
     {"256x256p", 256, 256, 8},   // the software-pipelined kernel of awq_gemm_pipe.hip, every tile cut split_k ways
     {"256x256pt", 256, 256, 8},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
 };
-constexpr int kPipeVariant = 9, kPipeTailVariant = 10;
+enum { k128x128 = 0, k64x256 = 1, k32x256 = 2 };
+constexpr int kPipeVariant = 3, kPipeTailVariant = 4;
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 template <typename T, int BM, int BN, int WM, int WN>
@@ -266,7 +268,7 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
 static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     const int kCUs = 256;
     // indices into kGemmVariants
-    constexpr int kPipe8 = kPipeVariant, k128x128 = 2, k64x256 = 3, k32x256 = 4;
+    constexpr int kPipe8 = kPipeVariant;
     int v;
     if (M <= 32) v = k32x256;
     else if (M <= 64) v = k64x256;
@@ -347,15 +349,9 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                                                         workspace, split_k, s);                   \
         break;
     switch (variant) {
-        AWQ_GEMM_CASE(0, 256, 256, 2, 4)
-        AWQ_GEMM_CASE(1, 128, 256, 2, 4)
-        AWQ_GEMM_CASE(2, 128, 128, 2, 2)
-        AWQ_GEMM_CASE(3, 64, 256, 1, 4)
-        AWQ_GEMM_CASE(4, 32, 256, 1, 4)
-        AWQ_GEMM_CASE(5, 64, 128, 1, 4)
-        AWQ_GEMM_CASE(6, 256, 256, 2, 2)
-        AWQ_GEMM_CASE(7, 128, 256, 2, 2)
-        AWQ_GEMM_CASE(8, 256, 128, 4, 2)
+        AWQ_GEMM_CASE(k128x128, 128, 128, 2, 2)
+        AWQ_GEMM_CASE(k64x256, 64, 256, 1, 4)
+        AWQ_GEMM_CASE(k32x256, 32, 256, 1, 4)
         case kPipeVariant:
         case kPipeTailVariant:
             e = launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,

@@ -79,13 +79,14 @@ def test_gemm_bias_and_determinism(dtype):
     xb = make_x(M, K, dtype, seed=81)
     xd = to_dev(xb, dtype)
     bias = np.linspace(-2, 2, N).astype(np.float32)
+    v = 0   # the 128 x 128 tile
     for split in (1, 4):
-        y = awq_gemm_variant(xd, *dev, 2, split, bias=to_dev(o.to_bits16(bias, dtype), dtype))
+        y = awq_gemm_variant(xd, *dev, v, split, bias=to_dev(o.to_bits16(bias, dtype), dtype))
         _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
-    y1 = awq_gemm_variant(xd, *dev, 2, 4)
-    y2 = awq_gemm_variant(xd, *dev, 2, 4)
+    y1 = awq_gemm_variant(xd, *dev, v, 4)
+    y2 = awq_gemm_variant(xd, *dev, v, 4)
     assert torch.equal(y1, y2)
-    assert torch.count_nonzero(awq_gemm_variant(torch.zeros_like(xd), *dev, 2, 4)) == 0
+    assert torch.count_nonzero(awq_gemm_variant(torch.zeros_like(xd), *dev, v, 4)) == 0
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
