@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 # (FETCH_SIZE, then WRITE_SIZE; profiles/gemv_cfg2_sweep_hbm_traffic.txt).  Each counter is scaled by
 # what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,014 -> 2047 B per count,
 # WRITE_SIZE 64,000 -> 1024 B per count.
-MEASURED_FETCH_BYTES_PER_LAUNCH = 1492.2 * 2047.1
+MEASURED_FETCH_BYTES_PER_LAUNCH = 1514.2 * 2047.1
 MEASURED_WRITE_BYTES_PER_LAUNCH = 108.9 * 1024.0
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
@@ -143,11 +143,11 @@ def main():
     avg_launch_us = ms_graph * 1e3 / launches_per_step
     avg_bytes = bytes_per_step / launches_per_step
     roofline = {
-        "kernel": "awq::gemv_dma_kernel<F16, WN=1, WK=4|8, DEPTH=1, MT=1>", "bound": "hbm",
+        "kernel": "awq::gemv_dma_kernel<F16, WK=4|8>", "bound": "hbm",
         "achieved": avg_bytes / (avg_launch_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "traffic": MEASURED_FETCH_BYTES_PER_LAUNCH + MEASURED_WRITE_BYTES_PER_LAUNCH,
-        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 3.05 MB + write 0.11 MB) from rocprofv3 "
+        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 3.10 MB + write 0.11 MB) from rocprofv3 "
                         "FETCH_SIZE / WRITE_SIZE, copy-calibrated.  The counters sit between the L2s and the fabric "
                         "and cannot tell Infinity Cache hits from HBM reads: 0.87 MB of the fetch is the prefetch "
                         "(spare workgroups read the next launch's weights once to park them in the Infinity Cache, "
