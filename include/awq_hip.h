@@ -48,6 +48,14 @@ const char* awq_hip_last_error(void);
 int awq_dequantize(const int32_t* qweight, const void* qscales, const int32_t* qzeros, void* out,
                    int64_t K, int64_t N, int64_t group_size, int dtype, void* stream);
 
+/* The same weight transposed: out [N, K] row-major (k-contiguous rows), out[n, k] = awq_dequantize's [k, n],
+ * bit for bit.  This is the layout a dense GEMM library multiplies fastest (y = x @ out^T); the host layer
+ * uses it for the reference's large-M branch, awq_dequantize + torch.matmul,
+ * nanoquantization/layers/gemm.py:558-561.  K % 64 == 0; group sizes 8, 16, 32 or a multiple of 64. */
+int awq_dequantize_transposed(const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                              void* out, int64_t K, int64_t N, int64_t group_size, int dtype,
+                              void* stream);
+
 /* Offline path: weight f32 [N, K] (the nn.Linear layout) -> packed AWQ buffers in one pass:
  * per group of `group_size` input features s = max(max - min, 1e-5) / 15,
  * z = clamp(-round(min / s), 0, 15), q = clamp(round(w / s) + z, 0, 15); qweight [K, N/8] and

@@ -4,7 +4,9 @@ Host-side mirror of nanoquantization/layers/gemm.py and
 nanoquantization/utils/quantization.py of liyuan24/nanoquantization, running on
 hand-written HIP kernels (csrc/) behind the C ABI of include/awq_hip.h.
 """
-from .layers.gemm import WQLinear_GEMM, awq_dequantize, awq_gemm, prefetch_hint  # noqa: F401
+from .layers.gemm import (WQLinear_GEMM, awq_dequantize, awq_dequantize_transposed, awq_gemm,  # noqa: F401
+                          prefetch_hint)
 from .utils.quantization import pseudo_quantize, quantize_pack  # noqa: F401
 
-__all__ = ["WQLinear_GEMM", "awq_dequantize", "awq_gemm", "pseudo_quantize", "quantize_pack", "prefetch_hint"]
+__all__ = ["WQLinear_GEMM", "awq_dequantize", "awq_dequantize_transposed", "awq_gemm", "pseudo_quantize", "quantize_pack",
+           "prefetch_hint"]

@@ -28,6 +28,7 @@ SYMBOLS = {
     "awq_hip_version": (_int, []),
     "awq_hip_last_error": (ctypes.c_char_p, []),
     "awq_dequantize": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
+    "awq_dequantize_transposed": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "awq_quantize_pack": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "awq_gemv_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "awq_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),

@@ -364,6 +364,23 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
 
 }  // namespace awq
 
+extern "C" int awq_dequantize_transposed(const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                                         void* out, int64_t K, int64_t N, int64_t group_size, int dtype,
+                                         void* stream) {
+    const char* fn = "awq_dequantize_transposed";
+    int rc = awq::check_linear_args(fn, out, qweight, qscales, qzeros, out, 1, N, K, group_size, dtype);
+    if (rc != AWQ_OK) return rc;
+    if (K % awq::kBK != 0 || !(group_size % 64 == 0 || (64 % group_size == 0 && group_size % 8 == 0)) ||
+        N > 0x7fffffff || K > 0x7fffffff) {
+        awq::set_error("%s: needs K %% 64 == 0 and a group size of 8, 16, 32 or a multiple of 64 (K=%lld, g=%lld)", fn,
+                       (long long)K, (long long)group_size);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    const hipError_t e = awq::launch_dequant_transpose(dtype, qweight, qscales, qzeros, out, (int)N, (int)K,
+                                                       (int)group_size, reinterpret_cast<hipStream_t>(stream));
+    return e == hipSuccess ? AWQ_OK : awq::hip_fail(fn, e);
+}
+
 extern "C" int awq_gemm_variant_count(void) { return awq::kNumGemmVariants; }
 
 extern "C" const char* awq_gemm_variant_name(int variant) {

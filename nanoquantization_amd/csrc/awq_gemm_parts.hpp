@@ -171,4 +171,9 @@ hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, co
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
                             void* workspace, int split_k, bool tail_only, hipStream_t stream, int act = 0);
 
+// awq_gemm_pipe.hip: wt [N][K] = the dequantised weight, transposed (K % 64 == 0, group size a multiple of 64 or
+// a divisor of 64 that is a multiple of 8).
+hipError_t launch_dequant_transpose(int dtype, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                                    void* wt, int N, int K, int g, hipStream_t stream);
+
 }  // namespace awq

@@ -358,6 +358,51 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     }
 }
 
+// wt[n][k] = RN_T((q - z) * s): the weight dequantised exactly as the fused kernel does, transposed to k-contiguous
+// rows -- the B layout a dense library GEMM runs fastest on (x @ wt^T).  A workgroup turns a 64 (k) x 256 (n) block:
+// a lane owns word column wc for 8 k rows (reads of 128 B per k row), writes its 8 x 8 values as eight 16-byte
+// chunks into an LDS tile [256 n][64 k], and the block leaves as full 128-byte rows.
+// HBM-bound: 0.52 B read + 2 B written per weight.
+template <typename T>
+__global__ __launch_bounds__(256) void dequant_transpose_kernel(const uint32_t* __restrict__ qweight,
+                                                                const uint16_t* __restrict__ scales,
+                                                                const uint32_t* __restrict__ qzeros,
+                                                                uint16_t* __restrict__ wt, int N, int K, int g) {
+    __shared__ u32x4 tile[256 * 8];   // [n][8 chunks of 8 k], chunk kc of row n at n*8 + (kc ^ ((n >> 3) & 7))
+    const int tid = threadIdx.x, wc = tid & 31, rb = tid >> 5;
+    const int words = N >> 3;
+    const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 256;
+    const int gwc = min((n0 >> 3) + wc, words - 1);
+    const int krow = k0 + rb * 8;
+    uint32_t w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = qweight[(size_t)(krow + i) * words + gwc];
+    const size_t grow = (size_t)(krow / g) * words + gwc;
+    const uint32_t zw = qzeros[grow];
+    const u32x4 sv = *reinterpret_cast<const u32x4*>(scales + grow * 8);
+    PipeUnpack<T> up;
+    up.init();
+    up.set_group(zw, sv);
+    uint32_t cols[8][4];
+#pragma unroll
+    for (int rp = 0; rp < 4; ++rp) {
+        uint32_t o[8];
+        up.pair(w[2 * rp], w[2 * rp + 1], o);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) cols[c][rp] = o[c];
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        tile[(wc * 8 + c) * 8 + (rb ^ (wc & 7))] = u32x4{cols[c][0], cols[c][1], cols[c][2], cols[c][3]};
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int n = j * 32 + (tid >> 3), kc = tid & 7;
+        if (n0 + n < N)
+            *reinterpret_cast<u32x4*>(wt + (size_t)(n0 + n) * K + k0 + kc * 8) = tile[n * 8 + (kc ^ ((n >> 3) & 7))];
+    }
+}
+
 // Second pass over the tail tiles: y = dtype(sum over K slices, in slice order, of the fp32 partials (+ bias)).
 // 32 workgroups per tile; a thread owns 8 consecutive columns of one row.
 template <typename T>
@@ -439,6 +484,21 @@ hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, co
                                         stream, act)
                : launch_pipe<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace, split_k, tail_only,
                                          stream, act);
+}
+
+hipError_t launch_dequant_transpose(int dtype, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                                    void* wt, int N, int K, int g, hipStream_t stream) {
+    (void)hipGetLastError();
+    const dim3 grid((N + 255) / 256, K / 64), block(256);
+    if (dtype == AWQ_F16)
+        hipLaunchKernelGGL(dequant_transpose_kernel<F16>, grid, block, 0, stream,
+                           reinterpret_cast<const uint32_t*>(qweight), reinterpret_cast<const uint16_t*>(qscales),
+                           reinterpret_cast<const uint32_t*>(qzeros), reinterpret_cast<uint16_t*>(wt), N, K, g);
+    else
+        hipLaunchKernelGGL(dequant_transpose_kernel<BF16>, grid, block, 0, stream,
+                           reinterpret_cast<const uint32_t*>(qweight), reinterpret_cast<const uint16_t*>(qscales),
+                           reinterpret_cast<const uint32_t*>(qzeros), reinterpret_cast<uint16_t*>(wt), N, K, g);
+    return hipGetLastError();
 }
 
 }  // namespace awq

@@ -253,7 +253,7 @@ def test_gemv_swiglu_equals_unfused(dtype, M, K, inter):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,inter", [(65, 1024, 3072), (300, 1024, 3072), (1000, 2048, 1032), (4100, 1024, 8192),
                                        (130, 256, 8)])
-def test_gemm_swiglu_equals_unfused(dtype, M, K, inter):
+def test_gemm_swiglu_equals_unfused(dtype, M, K, inter, monkeypatch):
     """Above the GEMV regime the gate runs in the GEMM's epilogue (whole tiles and K-split tiles alike): bit for bit
     what the plain GEMM over gate|up side by side followed by the SiLU*up kernel gives."""
     import nanoquantization_amd as nq
@@ -269,7 +269,10 @@ def test_gemm_swiglu_equals_unfused(dtype, M, K, inter):
     fused = ops.awq_linear_swiglu(x, *ops.interleave_gate_up(gate, up))
     side = [torch.cat([a, b], dim=1).contiguous() for a, b in zip(gate, up)]
     if M > 128:
-        ref_lin = nq.awq_gemm(x, side[0], side[1], side[2], 8)      # same kernel and K split as the fused call
+        # same kernel and K split as the fused call (the plain entry would hand 1024 rows or more to the library GEMM)
+        from nanoquantization_amd.layers import gemm as gemm_layer
+        monkeypatch.setattr(gemm_layer, "TWO_PASS_MIN_ROWS", 1 << 62)
+        ref_lin = nq.awq_gemm(x, side[0], side[1], side[2], 8)
     else:
         # up to 128 rows the plain dispatch takes a narrower tile; force the pipelined kernel with its split rule
         from nanoquantization_amd import _lib

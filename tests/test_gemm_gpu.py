@@ -117,6 +117,43 @@ def test_gemm_tail_tiles_split(dtype):
         assert torch.equal(y[2048:, :16 * 256], y1[2048:, :16 * 256])
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N,g", [(1024, 1032, 128), (256, 8, 64), (512, 264, 32), (128, 4096, 128), (1024, 520, 1024)])
+def test_dequantize_transposed_bit_exact(dtype, K, N, g):
+    # out [N, K] must be awq_dequantize's [K, N] transposed, bit for bit (and so the oracle's RN((q - z) * s))
+    print(f"dequantize transposed {dtype} K={K} N={N} g={g}", flush=True)
+    p = random_packed(K, N, g, dtype, seed=K + N + g)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    wt = nq.awq_dequantize_transposed(*dev)
+    assert tuple(wt.shape) == (N, K)
+    assert torch.equal(wt, nq.awq_dequantize(*dev).t())
+    ref_bits = o.dequant(p["qweight"], p["qzeros"], p["qscales"], dtype)
+    assert np.array_equal(to_bits(wt).T, ref_bits)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,K,N,g", [(1024, 1024, 1032, 128), (1500, 512, 2048, 64), (2048, 256, 264, 32)])
+def test_linear_two_pass_large_m(dtype, M, K, N, g):
+    # 1024 rows and more: transposed dequantise + the dense library matmul (the reference's large-M structure,
+    # layers/gemm.py:558-561), against the fp32 oracle, with and without bias, and against the fused kernel
+    from nanoquantization_amd.layers.gemm import _linear
+    print(f"two-pass linear {dtype} M={M} K={K} N={N} g={g}", flush=True)
+    p = make_case(K, N, g, dtype, seed=M + N)
+    xb = make_x(M, K, dtype, seed=M)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    xd = to_dev(xb, dtype)
+    y = nq.awq_gemm(xd, *dev, 8)
+    _check(y, xb, p, dtype)
+    bias = np.linspace(-1, 1, N).astype(np.float32)
+    yb = _linear("awq_linear", xd, *dev, to_dev(o.to_bits16(bias, dtype), dtype))
+    _check(yb, xb, p, dtype, o.to_dtype_f32(bias, dtype))
+    L = _lib.lib()
+    names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
+    fused = awq_gemm_variant(xd, *dev, names.index("256x256p"), 1)
+    err = (y.float() - fused.float()).abs().max().item() / fused.float().abs().max().item()
+    assert err <= (2e-3 if dtype == "f16" else 1.6e-2), err     # both round an fp32 sum of the same products once
+
+
 def test_gemm_prefill_full_size_bf16():
     # Qwen3-8B MLP gate/up at M=512, its real size (oracle: numpy float64 matmul, a few seconds)
     print("gemm full size M=512 4096x12288 bf16", flush=True)
