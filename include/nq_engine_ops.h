@@ -69,6 +69,11 @@ int nq_paged_attention_decode(const void* q, const void* k_cache, const void* v_
  * Qwen3QuantizedMLP.forward, nanoquantization/models/qwen3_quantized.py:147-152. */
 int nq_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream);
 
+/* The same for gate|up interleaved in words of 8 columns (word 2t = gate outputs 8t..8t+7, word 2t+1 = the up
+ * columns of the same outputs): the output layout of a plain product with the interleaved buffers of
+ * awq_gemv_swiglu (include/awq_hip.h). */
+int nq_silu_mul_interleaved(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream);
+
 /* out[r] = argmax_i logits[r, i] as int64, the lowest index among equal maxima (NaNs are never selected);
  * logits [rows, vocab] dense.  Greedy sampling for the engine's decode loop; the reference has no generation
  * loop, the logits are those of Qwen3QuantizedForCausalLM.forward

@@ -55,6 +55,7 @@ SYMBOLS = {
     "nq_paged_attention_workspace_bytes": (_sz, [_i64] * 5),
     "nq_paged_attention_decode": (_int, [_vp] * 6 + [_i64] * 7 + [ctypes.c_float, _int, _vp, _sz, _vp]),
     "nq_silu_mul": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "nq_silu_mul_interleaved": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "nq_argmax_rows": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
 }
 

@@ -635,7 +635,9 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* __res
     }
 }
 
-template <typename T>
+// IL: gate and up interleaved in words of 8 columns (word 2t = gate outputs 8t.., word 2t+1 = the up columns of the
+// same outputs) instead of side by side.
+template <typename T, bool IL>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate_up,
                                                        uint16_t* __restrict__ out, int64_t rows, int inter) {
     const int64_t vec = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -644,8 +646,9 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
     const int64_t r = vec / per_row;
     const int i = (int)(vec % per_row) * 8;
     float g[8], u[8], o[8];
-    unpack8<T>(*reinterpret_cast<const u32x4*>(gate_up + r * 2 * inter + i), g);
-    unpack8<T>(*reinterpret_cast<const u32x4*>(gate_up + r * 2 * inter + inter + i), u);
+    const uint16_t* row = gate_up + r * 2 * inter;
+    unpack8<T>(*reinterpret_cast<const u32x4*>(row + (IL ? 2 * i : i)), g);
+    unpack8<T>(*reinterpret_cast<const u32x4*>(row + (IL ? 2 * i + 8 : inter + i)), u);
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = round_to<T>(g[e] / (1.f + __expf(-g[e]))) * u[e];
     *reinterpret_cast<u32x4*>(out + r * inter + i) = pack8<T>(o);
@@ -871,8 +874,8 @@ extern "C" int nq_argmax_rows(const void* logits, int64_t* out, int64_t rows, in
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }
 
-extern "C" int nq_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream) {
-    const char* fn = "nq_silu_mul";
+static int silu_mul_entry(const char* fn, bool interleaved, const void* gate_up, void* out, int64_t rows, int64_t inter,
+                          int dtype, void* stream) {
     if (!gate_up || !out) return bad(fn, "null pointer argument");
     if (!aligned16(gate_up) || !aligned16(out)) return bad(fn, "tensors must be 16-byte aligned");
     if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
@@ -882,10 +885,22 @@ extern "C" int nq_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t
     hipStream_t st = (hipStream_t)stream;
     (void)hipGetLastError();
     const dim3 grid((unsigned)cdiv(vecs, 256)), block(256);
-    if (dtype == AWQ_F16)
-        silu_mul_kernel<F16><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
-    else
-        silu_mul_kernel<BF16><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
+    if (dtype == AWQ_F16) {
+        if (interleaved) silu_mul_kernel<F16, true><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
+        else silu_mul_kernel<F16, false><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
+    } else {
+        if (interleaved) silu_mul_kernel<BF16, true><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
+        else silu_mul_kernel<BF16, false><<<grid, block, 0, st>>>((const uint16_t*)gate_up, (uint16_t*)out, rows, (int)inter);
+    }
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" int nq_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream) {
+    return silu_mul_entry("nq_silu_mul", false, gate_up, out, rows, inter, dtype, stream);
+}
+
+extern "C" int nq_silu_mul_interleaved(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype,
+                                       void* stream) {
+    return silu_mul_entry("nq_silu_mul_interleaved", true, gate_up, out, rows, inter, dtype, stream);
 }

@@ -127,16 +127,17 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     return out
 
 
-def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
-    """gate_up [rows, 2*inter] -> SiLU(gate) * up [rows, inter]."""
+def silu_mul(gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """gate_up [rows, 2*inter] -> SiLU(gate) * up [rows, inter]; gate | up side by side, or interleaved in words
+    of 8 columns (the layout of interleave_gate_up)."""
     dev = _dev(gate_up)
     rows, two = gate_up.shape
     inter = two // 2
-    assert two == 2 * inter
+    assert two == 2 * inter and gate_up.is_contiguous()
     out = torch.empty(rows, inter, dtype=gate_up.dtype, device=dev)
+    fn = _lib.lib().nq_silu_mul_interleaved if interleaved else _lib.lib().nq_silu_mul
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().nq_silu_mul(gate_up.data_ptr(), out.data_ptr(), rows, inter,
-                                          _lib.dtype_id(gate_up.dtype), _stream()))
+        _lib.check(fn(gate_up.data_ptr(), out.data_ptr(), rows, inter, _lib.dtype_id(gate_up.dtype), _stream()))
     return out
 
 
@@ -166,12 +167,16 @@ def interleave_gate_up(gate, up):
 
 
 def awq_linear_swiglu(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor) -> torch.Tensor:
-    """x [M, K] (any M) and interleaved gate|up buffers [K, 2*inter/8] -> SiLU(x @ Wgate) * (x @ Wup) [M, inter]."""
+    """x [M, K] (any M) and interleaved gate|up buffers [K, 2*inter/8] -> SiLU(x @ Wgate) * (x @ Wup) [M, inter].
+    From layers.gemm.TWO_PASS_MIN_ROWS rows on: the plain product on the two-pass path, then the gate as its own pass."""
     dev = _dev(x, qweight, qscales, qzeros)
     M, K = x.shape
     N = qscales.shape[1]
     g = K // qscales.shape[0]
     assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    from ..layers import gemm as _gemm
+    if _gemm._two_pass_ok(M, K, g):
+        return silu_mul(_gemm._linear("awq_linear", x, qweight, qscales, qzeros, None), interleaved=True)
     out = torch.empty(M, N // 2, dtype=x.dtype, device=dev)
     L = _lib.lib()
     with torch.cuda.device(dev):

@@ -251,6 +251,17 @@ def test_gemv_swiglu_equals_unfused(dtype, M, K, inter):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul_interleaved_equals_side_by_side(dtype):
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(5)
+    rows, inter = 37, 3072
+    gate = torch.randn(rows, inter, device="cuda", generator=g).to(dtype)
+    up = torch.randn(rows, inter, device="cuda", generator=g).to(dtype)
+    il = torch.stack([gate.view(rows, inter // 8, 8), up.view(rows, inter // 8, 8)], dim=2).reshape(rows, 2 * inter)
+    assert torch.equal(ops.silu_mul(il.contiguous(), interleaved=True), ops.silu_mul(torch.cat([gate, up], dim=1)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,inter", [(65, 1024, 3072), (300, 1024, 3072), (1000, 2048, 1032), (4100, 1024, 8192),
                                        (130, 256, 8)])
 def test_gemm_swiglu_equals_unfused(dtype, M, K, inter, monkeypatch):
@@ -266,13 +277,13 @@ def test_gemm_swiglu_equals_unfused(dtype, M, K, inter, monkeypatch):
     gate, up = packed(inter), packed(inter)
     x = torch.randn(M, K, device="cuda", generator=g).to(dtype)
     print(f"gemm_swiglu M={M} K={K} inter={inter} {dtype}", flush=True)
+    # keep 1024 rows and more on the fused kernel too (by default they go to the library GEMM, checked below)
+    from nanoquantization_amd.layers import gemm as gemm_layer
+    monkeypatch.setattr(gemm_layer, "TWO_PASS_MIN_ROWS", 1 << 62)
     fused = ops.awq_linear_swiglu(x, *ops.interleave_gate_up(gate, up))
     side = [torch.cat([a, b], dim=1).contiguous() for a, b in zip(gate, up)]
     if M > 128:
-        # same kernel and K split as the fused call (the plain entry would hand 1024 rows or more to the library GEMM)
-        from nanoquantization_amd.layers import gemm as gemm_layer
-        monkeypatch.setattr(gemm_layer, "TWO_PASS_MIN_ROWS", 1 << 62)
-        ref_lin = nq.awq_gemm(x, side[0], side[1], side[2], 8)
+        ref_lin = nq.awq_gemm(x, side[0], side[1], side[2], 8)      # same kernel and K split as the fused call
     else:
         # up to 128 rows the plain dispatch takes a narrower tile; force the pipelined kernel with its split rule
         from nanoquantization_amd import _lib
@@ -285,6 +296,11 @@ def test_gemm_swiglu_equals_unfused(dtype, M, K, inter, monkeypatch):
     ref = ops.silu_mul(ref_lin)
     assert fused.shape == (M, inter)
     assert torch.equal(fused, ref)
+    if M >= 1024:
+        # the default path at this size: transposed dequantise + library GEMM + the gate as its own pass
+        monkeypatch.undo()
+        two_pass = ops.awq_linear_swiglu(x, *ops.interleave_gate_up(gate, up))
+        _close(two_pass, ref.float(), dtype, scale=4.0, what="two-pass gated product")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
