@@ -121,6 +121,38 @@ int awq_gemv_qkv_rope_store(const void* x, const int32_t* qweight, const void* q
                             int64_t block_size, float eps, int dtype, void* workspace, size_t workspace_bytes,
                             void* stream);
 
+/* A decode step without stand-alone residual-add + RMSNorm launches (Qwen3QuantizedBlock.forward,
+ * nanoquantization/models/qwen3_quantized.py:194-215: x + attn(norm(x)), x + mlp(norm(x))).  The statistics
+ * travel between the GEMVs as ssq, fp32 [hidden / 128][M]: ssq[t][m] = sum of squares of residual[m, 128 t .. 128 t + 127]
+ * (8 consecutive squares per lane by fused multiply-add in column order, 16 lanes combined by xor 8, 4, 2, 1; the
+ * tiles are added in index order).  nq_row_ssq (include/nq_engine_ops.h) produces the same statistics for a residual
+ * stream that comes from elsewhere (the embedding), and nq_add_rmsnorm sums in the same order, so every entry point
+ * below returns the bits of the separate kernels.  All of them: M <= 64, N % 128 == 0, K % 128 == 0,
+ * group_size % 128 == 0, no bias, workspace as for awq_gemv(M, N, K).
+ *
+ * awq_gemv_add_residual: residual [M, N] = dtype(residual + dtype(x @ W)) in place (o_proj, down_proj), and
+ *   ssq [N / 128][M] of the new residual.
+ * awq_gemv_rmsnorm: y = (RMSNorm(x) * norm_weight) @ W with x [M, K] the residual stream and ssq [K / 128][M] its
+ *   statistics: the operand is h = dtype(dtype(x * rsqrt(sum(ssq[:, m]) / K + norm_eps)) * norm_weight), the
+ *   arithmetic of RMSNorm.rms_norm, nanoquantization/layers/norm.py:18-32.  gated != 0: the interleaved gate/up
+ *   buffers and the SiLU(gate) * up epilogue of awq_gemv_swiglu, y [M, N / 2].
+ * awq_gemv_rmsnorm_qkv_rope_store: awq_gemv_qkv_rope_store with the same prologue on x. */
+int awq_gemv_add_residual(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                          void* residual, float* ssq, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                          int dtype, void* workspace, size_t workspace_bytes, void* stream);
+int awq_gemv_rmsnorm(const void* x, const float* ssq, const void* norm_weight, float norm_eps,
+                     const int32_t* qweight, const void* qscales, const int32_t* qzeros, void* y, int64_t M,
+                     int64_t N, int64_t K, int64_t group_size, int gated, int dtype, void* workspace,
+                     size_t workspace_bytes, void* stream);
+int awq_gemv_rmsnorm_qkv_rope_store(const void* x, const float* ssq, const void* norm_weight, float norm_eps,
+                                    const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                                    const void* q_weight, const void* k_weight, const float* cos_sin,
+                                    const int64_t* positions, const int64_t* slots, void* q_out, void* k_cache,
+                                    void* v_cache, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                                    int64_t num_heads, int64_t num_kv_heads, int64_t max_positions,
+                                    int64_t num_slots, int64_t block_size, float eps, int dtype, void* workspace,
+                                    size_t workspace_bytes, void* stream);
+
 /* Optional hint for latency-bound decode loops: the next awq_gemv / awq_linear / awq_gemv_swiglu call of
  * the calling thread that takes the staged GEMV path and leaves compute units idle also launches a few
  * spare workgroups that read [ptr, ptr + bytes) -- meant to be the packed qweight of the launch AFTER it --

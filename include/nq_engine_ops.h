@@ -27,6 +27,12 @@ extern "C" {
 int nq_add_rmsnorm(void* residual, const void* delta, const void* weight, void* y, int64_t rows,
                    int64_t hidden, float eps, int dtype, void* stream);
 
+/* ssq [ceil(hidden / 128)][rows] (fp32): ssq[t][r] = sum of squares of x[r, 128 t .. 128 t + 127], in the summation
+ * order of nq_add_rmsnorm.  The RMSNorm statistics that awq_gemv_rmsnorm (include/awq_hip.h) reads, for a residual
+ * stream that no awq_gemv_add_residual has produced (the embedding output of a decode step).  hidden % 8 == 0,
+ * hidden <= 8192.  The mean of squares of RMSNorm.rms_norm, nanoquantization/layers/norm.py:18-32. */
+int nq_row_ssq(const void* x, float* ssq, int64_t rows, int64_t hidden, int dtype, void* stream);
+
 /* qkv [rows, (num_heads + 2*num_kv_heads) * head_dim] is the output of the q|k|v projections
  * side by side.  Every q and k head is RMS-normalised (q_weight / k_weight, [head_dim]) and rotated
  * (half-split rotary, angle table cos_sin f32 [max_positions, head_dim] = cos | sin) at

@@ -38,6 +38,10 @@ SYMBOLS = {
     "awq_linear_swiglu": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "awq_linear_swiglu_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "awq_gemv_qkv_rope_store": (_int, [_vp] * 12 + [_i64] * 9 + [ctypes.c_float, _int, _vp, _sz, _vp]),
+    "awq_gemv_add_residual": (_int, [_vp] * 6 + [_i64] * 4 + [_int, _vp, _sz, _vp]),
+    "awq_gemv_rmsnorm": (_int, [_vp, _vp, _vp, ctypes.c_float] + [_vp] * 4 + [_i64] * 4 + [_int, _int, _vp, _sz, _vp]),
+    "awq_gemv_rmsnorm_qkv_rope_store": (_int, [_vp, _vp, _vp, ctypes.c_float] + [_vp] * 11 + [_i64] * 9 +
+                                        [ctypes.c_float, _int, _vp, _sz, _vp]),
     "awq_prefetch_hint": (_int, [_vp, _sz]),
     "awq_gemm": (_int, _LINEAR_ARGS),
     "awq_linear": (_int, _LINEAR_ARGS),
@@ -51,6 +55,7 @@ SYMBOLS = {
     "awq_gemm_ex": (_int, _LINEAR_ARGS + [_int, _int]),
     # include/nq_engine_ops.h
     "nq_add_rmsnorm": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_float, _int, _vp]),
+    "nq_row_ssq": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "nq_qk_norm_rope_store": (_int, [_vp] * 10 + [_i64] * 7 + [ctypes.c_float, _int, _vp]),
     "nq_paged_attention_workspace_bytes": (_sz, [_i64] * 5),
     "nq_paged_attention_decode": (_int, [_vp] * 6 + [_i64] * 7 + [ctypes.c_float, _int, _vp, _sz, _vp]),

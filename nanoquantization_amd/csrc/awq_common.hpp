@@ -126,6 +126,28 @@ __device__ __forceinline__ bool arrive_last(int* counter, int splits, int* s_fla
     return *s_flag != 0;
 }
 
+// T(a * b) for a genuine fp32 factor: the product is rounded to fp32, then to T, as torch's `x.float() * r`
+// followed by `.to(dtype)` does.  Without the barrier the compiler may pick the mixed-precision FMA for fp16, which
+// rounds once, and two kernels that should agree bit for bit would depend on its choice.
+template <typename T>
+__device__ __forceinline__ float mul_round(float a, float b) {
+    float p = a * b;
+    asm("" : "+v"(p));
+    return T::to_f32(T::from_f32(p));
+}
+
+// Sum of squares of one 128-column tile of a row, 8 consecutive values per lane, 16 lanes (an aligned group) per
+// tile: the lane's 8 squares in column order by fused multiply-add, then the lanes by xor 8, 4, 2, 1.  Every
+// kernel that produces or consumes RMSNorm statistics uses this order, so their results agree bit for bit.
+__device__ __forceinline__ float tile_ssq(const float (&v)[8]) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = __builtin_fmaf(v[e], v[e], ss);
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
+    return ss;
+}
+
 // ---- host-side error plumbing -------------------------------------------
 void set_error(const char* fmt, ...);
 int check_linear_args(const char* fn, const void* x, const int32_t* qweight, const void* qscales,

@@ -338,13 +338,71 @@ __device__ __forceinline__ void swiglu_store(const float (&out)[8], uint16_t* __
     }
 }
 
+// Residual epilogue (the o_proj / down_proj of a decode step): the product is added to the residual stream in
+// place, residual = T(residual + T(product)) -- the two roundings of a separate linear followed by an addition --
+// and the sum of squares of the new residual over the workgroup's 128 columns goes to ssq[tile][row], so that the
+// next GEMV can apply the RMSNorm of its input without a pass over the row.  The order of that sum is fixed: a
+// lane adds its 8 squares in column order (fused multiply-add), the 16 lanes of a tile combine by xor 8, 4, 2, 1.
+struct ResidEpilogue {
+    float* ssq;      // [N / 128][m_stride]
+    int m_stride;    // rows of the whole launch
+};
+
+// RMSNorm of the GEMV's input applied on the way into the MFMA operand: h = T(T(x * r) * weight), with
+// r = rsqrt(sum over tiles of ssq[tile][row] / K + eps), the tiles added in index order.
+struct NormPrologue {
+    const uint16_t* weight;   // [K]
+    const float* ssq;         // [K / 128][m_stride]
+    int m_stride;
+    float eps;
+};
+
+// The 16 lanes that hold the 16 words of (row m, column tile n0 / 128) call this together; `valid` masks the stores.
+// `rv` = the 8 residual values at (m, n0), loaded by the caller ahead of time (residual_load) so that their latency
+// hides behind the reduction.
+__device__ __forceinline__ u32x4 residual_load(const uint16_t* __restrict__ y, int m, int N, size_t n0, bool valid) {
+    return *reinterpret_cast<const u32x4*>(y + (size_t)(valid ? m : 0) * N + (valid ? n0 : 0));
+}
+template <typename T>
+__device__ __forceinline__ void residual_store(const float (&out)[8], u32x4 rv, uint16_t* __restrict__ y, int m, int N,
+                                               size_t n0, bool valid, const ResidEpilogue& re) {
+    float xn[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float xr = T::to_f32((uint16_t)((e & 1) ? rv[e >> 1] >> 16 : rv[e >> 1] & 0xFFFFu));
+        xn[e] = T::to_f32(T::from_f32(xr + T::to_f32(T::from_f32(out[e]))));
+    }
+    const float ss = tile_ssq(xn);
+    if (!valid) return;
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = T::pack2(xn[2 * i], xn[2 * i + 1]);
+    *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
+    if (((n0 >> 3) & 15) == 0) re.ssq[(n0 >> 7) * re.m_stride + m] = ss;
+}
+
+// What a kernel's epilogue may need beyond y: kEpi 0 nothing, 1 the q|k|v epilogue, 2 the residual epilogue.
+struct EpiArgs {
+    const QkvEpilogue* qe = nullptr;
+    const ResidEpilogue* re = nullptr;
+};
+
+// Host side: the optional parts of a launch of the staged kernel (at most one epilogue; the prologue combines
+// with none or with the q|k|v epilogue).
+struct GemvFusion {
+    const QkvEpilogue* qe = nullptr;
+    const NormPrologue* np = nullptr;
+    const ResidEpilogue* re = nullptr;
+    bool any() const { return qe || np || re; }
+};
+
 // kPlain: the partials are read by a later kernel, not by a concurrent workgroup: ordinary stores do.
-template <typename T, int V, int WN, int WK, bool kPlain = false, bool kQkv = false>
+template <typename T, int V, int WN, int WK, bool kPlain = false, int kEpi = 0>
 __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_base, float* red, int lane,
                                                   int wave, int group, int split, int splits,
                                                   const uint16_t* __restrict__ bias,
                                                   uint16_t* __restrict__ y, float* __restrict__ partials,
-                                                  int M, int N, int act, const QkvEpilogue* qe = nullptr) {
+                                                  int M, int N, int act, EpiArgs ea = EpiArgs{}) {
     constexpr int NF = 8 * V, NQ = 4 * V;
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
@@ -352,6 +410,12 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
     const int wv_col = (group * WN + wn) * 16 + j;  // this lane's column, in units of V words
     const bool col_ok = wv_col * V < words;
     // slot q = v*4 + r holds 8 consecutive output columns of row m_base + 4*kb + r
+    u32x4 rv_pre = u32x4{0u, 0u, 0u, 0u};
+    if constexpr (kEpi == 2) {   // a wave stores at most one slot (q = wk): fetch its residual before the reduction
+        static_assert(V == 1 && WK >= 4, "residual epilogue: one slot per wave");
+        if (splits == 1 && wk < NQ)
+            rv_pre = residual_load(y, m_base + 4 * kb + wk, N, (size_t)wv_col * 8, m_base + 4 * kb + wk < M && col_ok);
+    }
     if constexpr (WK > 1) {
         float* mine = red + (size_t)wave * (NF * 4 * 64);
 #pragma unroll
@@ -385,9 +449,12 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
 #pragma unroll
                         for (int c = 0; c < 8; ++c) out[c] = acc[vv * 8 + c][rr];
         }
-        if constexpr (kQkv) {
+        if constexpr (kEpi != 0) {
             if (splits == 1) {   // every lane takes part (cross-lane sums); the stores are masked
-                qkv_rope_store<T>(out, m, ((size_t)wv_col * V + v) * 8, m < M && col_ok, *qe);
+                if constexpr (kEpi == 1)
+                    qkv_rope_store<T>(out, m, ((size_t)wv_col * V + v) * 8, m < M && col_ok, *ea.qe);
+                else
+                    residual_store<T>(out, rv_pre, y, m, N, ((size_t)wv_col * V + v) * 8, m < M && col_ok, *ea.re);
                 continue;
             }
         }
@@ -420,12 +487,12 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
     }
 }
 
-template <typename T, int V, int WN, int WK, bool kQkv = false>
+template <typename T, int V, int WN, int WK, int kEpi = 0>
 __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int splits,
                                                 const uint16_t* __restrict__ bias,
                                                 uint16_t* __restrict__ y, float* __restrict__ partials,
                                                 int* __restrict__ counters, int M, int N, int act,
-                                                const QkvEpilogue* qe = nullptr) {
+                                                EpiArgs ea = EpiArgs{}) {
     constexpr int WAVES = WN * WK;
     const int words = N >> 3;
     if (!arrive_last(&counters[group], splits, s_last)) return;
@@ -436,6 +503,8 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
         const int m = idx / w_count, wc = idx - m * w_count;
         const size_t n0 = (size_t)(w_begin + wc) * 8;
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        u32x4 rv = u32x4{0u, 0u, 0u, 0u};
+        if constexpr (kEpi == 2) rv = residual_load(y, m, N, n0, true);   // in flight beside the partials
         // fetch 8 splits at a time (two 16-byte loads each) so that their loads overlap; add in split order
         for (int s0 = 0; s0 < splits; s0 += 8) {
             f32x4 lo[8], hi[8];
@@ -457,8 +526,12 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
                     }
                 }
         }
-        if constexpr (kQkv) {   // w_count == 16 here: the 16 lanes of a head run the same iterations
-            qkv_rope_store<T>(out, m, n0, true, *qe);
+        if constexpr (kEpi == 1) {   // w_count == 16 here: the 16 lanes of a head run the same iterations
+            qkv_rope_store<T>(out, m, n0, true, *ea.qe);
+            continue;
+        }
+        if constexpr (kEpi == 2) {   // likewise: 16 lanes per row and column tile
+            residual_store<T>(out, rv, y, m, N, n0, true, *ea.re);
             continue;
         }
         if (act) {   // w_count is even here: a gate word and its up word sit in neighbouring lanes
@@ -484,24 +557,24 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
 // (fixed order), then either store y (splits == 1) or publish this split's
 // partial and let the last workgroup of the tile group add the partials in
 // split order.  `group` is the workgroup's index along N.
-template <typename T, int V, int WN, int WK, int MT = 1, bool kQkv = false>
+template <typename T, int V, int WN, int WK, int MT = 1, int kEpi = 0>
 __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* red, int* s_last, int lane,
                                               int wave, int group, int split, int splits,
                                               const uint16_t* __restrict__ bias,
                                               uint16_t* __restrict__ y, float* __restrict__ partials,
                                               int* __restrict__ counters, int M, int N, int act = 0,
-                                              const QkvEpilogue* qe = nullptr) {
+                                              EpiArgs ea = EpiArgs{}) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (mt > 0) {
             if (16 * mt >= M) break;  // uniform
             __syncthreads();          // the reduction buffer is reused per m-tile
         }
-        gemv_reduce_store<T, V, WN, WK, false, kQkv>(acc[mt], 16 * mt, red, lane, wave, group, split, splits, bias,
-                                                     y, partials, M, N, act, qe);
+        gemv_reduce_store<T, V, WN, WK, false, kEpi>(acc[mt], 16 * mt, red, lane, wave, group, split, splits, bias,
+                                                     y, partials, M, N, act, ea);
     }
     if (splits == 1) return;
-    gemv_split_tail<T, V, WN, WK, kQkv>(s_last, group, splits, bias, y, partials, counters, M, N, act, qe);
+    gemv_split_tail<T, V, WN, WK, kEpi>(s_last, group, splits, bias, y, partials, counters, M, N, act, ea);
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
@@ -610,17 +683,29 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
 
 __host__ __device__ constexpr int dma_wave_bytes(int M) { return 8192 + 256 * M + 512; }
 
-struct NoEpilogue {};
+// Forms of the staged kernel (MODE): bit 0 the q|k|v epilogue, bit 1 the RMSNorm prologue, bit 2 the residual
+// epilogue.  The extra arguments of a form stay out of the plain kernel's argument block (the launch-bound decode
+// GEMVs measured 0.2-0.5 us slower with them).
+constexpr int kModeQkv = 1, kModeNorm = 2, kModeResid = 4;
+template <int MODE>
+struct GemvExtra {};
+template <>
+struct GemvExtra<kModeQkv> { QkvEpilogue qe; };
+template <>
+struct GemvExtra<kModeNorm> { NormPrologue np; };
+template <>
+struct GemvExtra<kModeQkv | kModeNorm> { QkvEpilogue qe; NormPrologue np; };
+template <>
+struct GemvExtra<kModeResid> { ResidEpilogue re; };
 
-// QKV: the kernel behind awq_gemv_qkv_rope_store; its extra arguments stay out of the plain kernel's argument
-// block (the launch-bound decode GEMVs measured 0.2-0.5 us slower with them).
-template <typename T, int WK, bool QKV = false>
+template <typename T, int WK, int MODE = 0>
 __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
-    int splits, int act, int groups, PrefetchRegions pf, std::conditional_t<QKV, QkvEpilogue, NoEpilogue> qe) {
+    int splits, int act, int groups, PrefetchRegions pf, GemvExtra<MODE> ex) {
+    constexpr bool QKV = (MODE & kModeQkv) != 0, NORM = (MODE & kModeNorm) != 0, RESID = (MODE & kModeResid) != 0;
     constexpr int CH = 4;
     extern __shared__ float red[];  // staging while streaming, [WK][32][64] floats afterwards
     __shared__ int s_last;
@@ -660,10 +745,12 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
         counters += rb * groups;
         M = min(16, M - 16 * rb);
         if constexpr (QKV) {
-            qe.positions += rb * 16;
-            qe.slots += rb * 16;
-            qe.q_out += (size_t)rb * 16 * qe.nh * 128;
+            ex.qe.positions += rb * 16;
+            ex.qe.slots += rb * 16;
+            ex.qe.q_out += (size_t)rb * 16 * ex.qe.nh * 128;
         }
+        if constexpr (NORM) ex.np.ssq += rb * 16;
+        if constexpr (RESID) ex.re.ssq += rb * 16;
     }
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -732,8 +819,29 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
 #pragma unroll
     for (int f = 0; f < 8; ++f) acc[0][f] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    if (c0 < c1) issue_dma(c0);
+    float rstd = 0.f;
+    if constexpr (NORM) {   // the lane's row: 1 / rms from the tile sums, added in tile order (eight loads in flight)
+        const float* sp = ex.np.ssq + min(j, M - 1);
+        float tot = 0.f;
+        for (int t0 = 0; t0 < total_chunks; t0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = sp[(size_t)min(t0 + u, total_chunks - 1) * ex.np.m_stride];
+            if (t0 == 0 && c0 < c1) issue_dma(c0);   // behind the first statistics loads, ahead of their use
+#pragma unroll
+            for (int u = 0; u < 8; ++u) tot += t0 + u < total_chunks ? v[u] : 0.f;
+        }
+        rstd = rsqrtf(tot / (float)K + ex.np.eps);
+    } else {
+        if (c0 < c1) issue_dma(c0);
+    }
     for (int c = c0; c < c1; ++c) {
+        u32x4 nw[CH];
+        if constexpr (NORM) {
+#pragma unroll
+            for (int s = 0; s < CH; ++s)
+                nw[s] = *reinterpret_cast<const u32x4*>(ex.np.weight + c * 128 + s * 32 + kb * 8);
+        }
         // The compiler does not order LDS reads after the DMA by itself.
         __builtin_amdgcn_s_waitcnt(0x0F70);                                      // vmcnt(0): chunk c has landed
         asm volatile("" ::: "memory");
@@ -751,15 +859,27 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
         __builtin_amdgcn_s_waitcnt(0xC07F);                                      // lgkmcnt(0)
         asm volatile("" ::: "memory");
         if (c + 1 < c1) issue_dma(c + 1);
+        if constexpr (NORM) {
+#pragma unroll
+            for (int s = 0; s < CH; ++s)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t xv = d.xa[s][0][i], wv = nw[s][i];
+                    const float lo = mul_round<T>(T::to_f32((uint16_t)(xv & 0xFFFFu)), rstd) *
+                                     T::to_f32((uint16_t)(wv & 0xFFFFu));
+                    const float hi = mul_round<T>(T::to_f32((uint16_t)(xv >> 16)), rstd) *
+                                     T::to_f32((uint16_t)(wv >> 16));
+                    d.xa[s][0][i] = T::pack2(lo, hi);
+                }
+        }
         compute_chunk<T, 1, CH, 1>(d, acc);
     }
     __syncthreads();  // staging area becomes the reduction buffer
-    if constexpr (QKV)
-        gemv_epilogue<T, 1, 1, WK, 1, true>(acc, red, &s_last, lane, wave, tile, split, splits, bias, y, partials,
-                                            counters, M, N, act, &qe);
-    else
-        gemv_epilogue<T, 1, 1, WK, 1>(acc, red, &s_last, lane, wave, tile, split, splits, bias, y, partials,
-                                      counters, M, N, act);
+    EpiArgs ea;
+    if constexpr (QKV) ea.qe = &ex.qe;
+    if constexpr (RESID) ea.re = &ex.re;
+    gemv_epilogue<T, 1, 1, WK, 1, QKV ? 1 : (RESID ? 2 : 0)>(acc, red, &s_last, lane, wave, tile, split, splits, bias,
+                                                            y, partials, counters, M, N, act, ea);
 }
 
 // ---- data path 3: a workgroup of eight waves shares one staged chunk --------------------------
@@ -1037,7 +1157,7 @@ template <typename T, int WK>
 static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                                   int g, void* workspace, int split_k, hipStream_t stream, int act,
-                                  const QkvEpilogue* qe = nullptr) {
+                                  const GemvFusion& fu = GemvFusion{}) {
     const int groups = N / 128;
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
@@ -1052,14 +1172,17 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     if (lds < red_bytes) lds = red_bytes;
     constexpr size_t kMaxLds = (size_t)WK * dma_wave_bytes(16);
     if (kMaxLds > 64 * 1024) {
-        static bool raised = false;  // once per process and instantiation (both forms of the kernel)
+        static bool raised = false;  // once per process and instantiation (every form of the kernel)
         if (!raised) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, false>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
-            if (e == hipSuccess)
-                e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
-            if (e != hipSuccess) return e;
+            const void* forms[] = {reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, 0>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeQkv>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeNorm>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeQkv | kModeNorm>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeResid>)};
+            for (const void* f : forms) {
+                hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
+                if (e != hipSuccess) return e;
+            }
             raised = true;
         }
     }
@@ -1080,18 +1203,23 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
         pf.count = 0;
     }
     const dim3 grid(groups + pf_wgs, splits, row_blocks), block(64 * WK);
-    if (qe)
-        hipLaunchKernelGGL((gemv_dma_kernel<T, WK, true>), grid, block, lds, stream,
-                           reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
-                           reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
-                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
-                           M, N, K, g / 128, cps, splits, act, groups, pf, *qe);
+#define AWQ_DMA_LAUNCH(MODE, EXTRA)                                                                                \
+    hipLaunchKernelGGL((gemv_dma_kernel<T, WK, MODE>), grid, block, lds, stream,                                  \
+                       reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),          \
+                       reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),     \
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters, \
+                       M, N, K, g / 128, cps, splits, act, groups, pf, EXTRA)
+    if (fu.qe && fu.np)
+        AWQ_DMA_LAUNCH(kModeQkv | kModeNorm, (GemvExtra<kModeQkv | kModeNorm>{*fu.qe, *fu.np}));
+    else if (fu.qe)
+        AWQ_DMA_LAUNCH(kModeQkv, (GemvExtra<kModeQkv>{*fu.qe}));
+    else if (fu.np)
+        AWQ_DMA_LAUNCH(kModeNorm, (GemvExtra<kModeNorm>{*fu.np}));
+    else if (fu.re)
+        AWQ_DMA_LAUNCH(kModeResid, (GemvExtra<kModeResid>{*fu.re}));
     else
-        hipLaunchKernelGGL((gemv_dma_kernel<T, WK, false>), grid, block, lds, stream,
-                           reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
-                           reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
-                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
-                           M, N, K, g / 128, cps, splits, act, groups, pf, NoEpilogue{});
+        AWQ_DMA_LAUNCH(0, (GemvExtra<0>{}));
+#undef AWQ_DMA_LAUNCH
     return hipGetLastError();
 }
 
@@ -1218,7 +1346,7 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
                          void* stream, int variant, int split_k, int act = 0,
-                         const QkvEpilogue* qe = nullptr) {
+                         const GemvFusion& fu = GemvFusion{}) {
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
     if (act && (variant < kFirstDmaVariant || bias)) {
@@ -1226,9 +1354,14 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                   "and takes no bias", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
-    if (act == 2 && (!qe || kGemvVariants[variant < 0 || variant >= kNumGemvVariants ? 0 : variant].wide ||
-                     kGemvVariants[variant < 0 || variant >= kNumGemvVariants ? 0 : variant].wn != 1)) {
-        set_error("%s: the q|k|v epilogue runs on the one-tile-per-workgroup staged kernels only", fn);
+    if ((act == 2) != (fu.qe != nullptr) || (fu.re && (act || fu.np || bias))) {
+        set_error("%s: inconsistent epilogue arguments", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    if (fu.any() && (variant < kFirstDmaVariant || variant >= kNumGemvVariants || kGemvVariants[variant].wide ||
+                     kGemvVariants[variant].wn != 1)) {
+        set_error("%s: the q|k|v / residual epilogues and the RMSNorm prologue run on the one-tile-per-workgroup "
+                  "staged kernels only (N %% 128 == 0, group_size %% 128 == 0)", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
     if (M > 64) {
@@ -1289,12 +1422,12 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                     : launch_gemv_wide<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
             break;
         case kDma1x4:
-            e = f16 ? launch_gemv_dma<F16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe)
-                    : launch_gemv_dma<BF16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe);
+            e = f16 ? launch_gemv_dma<F16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu)
+                    : launch_gemv_dma<BF16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu);
             break;
         case kDma1x8:
-            e = f16 ? launch_gemv_dma<F16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe)
-                    : launch_gemv_dma<BF16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, qe);
+            e = f16 ? launch_gemv_dma<F16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu)
+                    : launch_gemv_dma<BF16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu);
             break;
         default: {
             // register path; group sizes 32/64/96...: one 32-row step per chunk, always with the next chunk prefetched
@@ -1348,32 +1481,49 @@ extern "C" int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void
                               dtype, workspace, workspace_bytes, stream, v, s, 1);
 }
 
-extern "C" int awq_gemv_qkv_rope_store(const void* x, const int32_t* qweight, const void* qscales,
-                                       const int32_t* qzeros, const void* q_weight, const void* k_weight,
-                                       const float* cos_sin, const int64_t* positions, const int64_t* slots,
-                                       void* q_out, void* k_cache, void* v_cache, int64_t M, int64_t N, int64_t K,
-                                       int64_t group_size, int64_t num_heads, int64_t num_kv_heads,
-                                       int64_t max_positions, int64_t num_slots, int64_t block_size, float eps,
-                                       int dtype, void* workspace, size_t workspace_bytes, void* stream) {
-    const char* fn = "awq_gemv_qkv_rope_store";
+namespace awq {
+static int make_norm_prologue(const char* fn, const float* ssq, const void* norm_weight, float norm_eps, int64_t M,
+                              NormPrologue* np) {
+    if (!ssq || !norm_weight) {
+        set_error("%s: null pointer argument", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    if ((reinterpret_cast<uintptr_t>(norm_weight) & 15u) || (reinterpret_cast<uintptr_t>(ssq) & 3u)) {
+        set_error("%s: the norm weight must be 16-byte aligned, the sums of squares 4-byte aligned", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    np->weight = reinterpret_cast<const uint16_t*>(norm_weight);
+    np->ssq = ssq;
+    np->m_stride = (int)M;
+    np->eps = norm_eps;
+    return AWQ_OK;
+}
+
+static int qkv_rope_store_entry(const char* fn, const void* x, const NormPrologue* np, const int32_t* qweight,
+                                const void* qscales, const int32_t* qzeros, const void* q_weight, const void* k_weight,
+                                const float* cos_sin, const int64_t* positions, const int64_t* slots, void* q_out,
+                                void* k_cache, void* v_cache, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                                int64_t num_heads, int64_t num_kv_heads, int64_t max_positions, int64_t num_slots,
+                                int64_t block_size, float eps, int dtype, void* workspace, size_t workspace_bytes,
+                                void* stream) {
     if (!q_weight || !k_weight || !cos_sin || !positions || !slots || !q_out || !k_cache || !v_cache) {
-        awq::set_error("%s: null pointer argument", fn);
+        set_error("%s: null pointer argument", fn);
         return AWQ_ERR_INVALID_ARG;
     }
     if ((reinterpret_cast<uintptr_t>(q_weight) | reinterpret_cast<uintptr_t>(k_weight) |
          reinterpret_cast<uintptr_t>(cos_sin) | reinterpret_cast<uintptr_t>(q_out) |
          reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15u) {
-        awq::set_error("%s: every tensor must be 16-byte aligned", fn);
+        set_error("%s: every tensor must be 16-byte aligned", fn);
         return AWQ_ERR_INVALID_ARG;
     }
     if (num_heads <= 0 || num_kv_heads <= 0 || N != (num_heads + 2 * num_kv_heads) * 128 || max_positions <= 0 ||
         max_positions > 0x7fffffff || block_size <= 0 || block_size > 0x7fffffff || num_slots <= 0 ||
         num_slots % block_size != 0) {
-        awq::set_error("%s: needs head_dim 128 (N == (num_heads + 2 * num_kv_heads) * 128), positive max_positions and "
-                       "block_size, and num_slots a multiple of block_size", fn);
+        set_error("%s: needs head_dim 128 (N == (num_heads + 2 * num_kv_heads) * 128), positive max_positions and "
+                  "block_size, and num_slots a multiple of block_size", fn);
         return AWQ_ERR_INVALID_ARG;
     }
-    awq::QkvEpilogue qe;
+    QkvEpilogue qe;
     qe.q_weight = reinterpret_cast<const uint16_t*>(q_weight);
     qe.k_weight = reinterpret_cast<const uint16_t*>(k_weight);
     qe.cos_sin = cos_sin;
@@ -1389,9 +1539,80 @@ extern "C" int awq_gemv_qkv_rope_store(const void* x, const int32_t* qweight, co
     qe.num_slots = num_slots;
     qe.eps = eps;
     int v = 0, s = 1;
+    if (K >= 32 && N >= 8 && group_size > 0) pick_gemv(M, N, K, group_size, &v, &s, false);
+    GemvFusion fu;
+    fu.qe = &qe;
+    fu.np = np;
+    return gemv_dispatch(fn, x, qweight, qscales, qzeros, nullptr, q_out, M, N, K, group_size, dtype, workspace,
+                         workspace_bytes, stream, v, s, 2, fu);
+}
+}  // namespace awq
+
+extern "C" int awq_gemv_qkv_rope_store(const void* x, const int32_t* qweight, const void* qscales,
+                                       const int32_t* qzeros, const void* q_weight, const void* k_weight,
+                                       const float* cos_sin, const int64_t* positions, const int64_t* slots,
+                                       void* q_out, void* k_cache, void* v_cache, int64_t M, int64_t N, int64_t K,
+                                       int64_t group_size, int64_t num_heads, int64_t num_kv_heads,
+                                       int64_t max_positions, int64_t num_slots, int64_t block_size, float eps,
+                                       int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    return awq::qkv_rope_store_entry("awq_gemv_qkv_rope_store", x, nullptr, qweight, qscales, qzeros, q_weight,
+                                     k_weight, cos_sin, positions, slots, q_out, k_cache, v_cache, M, N, K, group_size,
+                                     num_heads, num_kv_heads, max_positions, num_slots, block_size, eps, dtype,
+                                     workspace, workspace_bytes, stream);
+}
+
+extern "C" int awq_gemv_rmsnorm_qkv_rope_store(const void* x, const float* ssq, const void* norm_weight,
+                                               float norm_eps, const int32_t* qweight, const void* qscales,
+                                               const int32_t* qzeros, const void* q_weight, const void* k_weight,
+                                               const float* cos_sin, const int64_t* positions, const int64_t* slots,
+                                               void* q_out, void* k_cache, void* v_cache, int64_t M, int64_t N,
+                                               int64_t K, int64_t group_size, int64_t num_heads, int64_t num_kv_heads,
+                                               int64_t max_positions, int64_t num_slots, int64_t block_size, float eps,
+                                               int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "awq_gemv_rmsnorm_qkv_rope_store";
+    awq::NormPrologue np;
+    const int rc = awq::make_norm_prologue(fn, ssq, norm_weight, norm_eps, M, &np);
+    if (rc != AWQ_OK) return rc;
+    return awq::qkv_rope_store_entry(fn, x, &np, qweight, qscales, qzeros, q_weight, k_weight, cos_sin, positions,
+                                     slots, q_out, k_cache, v_cache, M, N, K, group_size, num_heads, num_kv_heads,
+                                     max_positions, num_slots, block_size, eps, dtype, workspace, workspace_bytes,
+                                     stream);
+}
+
+extern "C" int awq_gemv_rmsnorm(const void* x, const float* ssq, const void* norm_weight, float norm_eps,
+                                const int32_t* qweight, const void* qscales, const int32_t* qzeros, void* y,
+                                int64_t M, int64_t N, int64_t K, int64_t group_size, int gated, int dtype,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "awq_gemv_rmsnorm";
+    awq::NormPrologue np;
+    const int rc = awq::make_norm_prologue(fn, ssq, norm_weight, norm_eps, M, &np);
+    if (rc != AWQ_OK) return rc;
+    int v = 0, s = 1;
     if (K >= 32 && N >= 8 && group_size > 0) awq::pick_gemv(M, N, K, group_size, &v, &s, false);
-    return awq::gemv_dispatch(fn, x, qweight, qscales, qzeros, nullptr, q_out, M, N, K, group_size, dtype, workspace,
-                              workspace_bytes, stream, v, s, 2, &qe);
+    awq::GemvFusion fu;
+    fu.np = &np;
+    return awq::gemv_dispatch(fn, x, qweight, qscales, qzeros, nullptr, y, M, N, K, group_size, dtype, workspace,
+                              workspace_bytes, stream, v, s, gated ? 1 : 0, fu);
+}
+
+extern "C" int awq_gemv_add_residual(const void* x, const int32_t* qweight, const void* qscales,
+                                     const int32_t* qzeros, void* residual, float* ssq, int64_t M, int64_t N,
+                                     int64_t K, int64_t group_size, int dtype, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+    const char* fn = "awq_gemv_add_residual";
+    if (!ssq || (reinterpret_cast<uintptr_t>(ssq) & 3u)) {
+        awq::set_error("%s: ssq must be a 4-byte aligned device pointer", fn);
+        return AWQ_ERR_INVALID_ARG;
+    }
+    awq::ResidEpilogue re;
+    re.ssq = ssq;
+    re.m_stride = (int)M;
+    int v = 0, s = 1;
+    if (K >= 32 && N >= 8 && group_size > 0) awq::pick_gemv(M, N, K, group_size, &v, &s, false);
+    awq::GemvFusion fu;
+    fu.re = &re;
+    return awq::gemv_dispatch(fn, x, qweight, qscales, qzeros, nullptr, residual, M, N, K, group_size, dtype,
+                              workspace, workspace_bytes, stream, v, s, 0, fu);
 }
 
 extern "C" int awq_gemv_ex(const void* x, const int32_t* qweight, const void* qscales,

@@ -37,25 +37,23 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // ---------------------------------------------------------------------------------------------
 // residual (+= delta); y = RMSNorm(residual) * weight.  One workgroup per row, 8 values per lane
-// and pass, at most 4 passes (hidden <= 8192).
+// and pass, at most 4 passes (hidden <= 8192).  The sum of squares is built per 128-column tile
+// (tile_ssq) and the tiles are added in index order: the order the AWQ GEMVs with a residual epilogue
+// and an RMSNorm prologue use, so both routes give the same bits.
 constexpr int kNormThreads = 256;
 constexpr int kNormPasses = 4;
+constexpr int kNormTiles = kNormPasses * kNormThreads / 16;
 
+// Loads the row (adding and storing delta if given), leaves the tile sums in s_tile and returns their total.
 template <typename T>
-__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __restrict__ residual,
-                                                                  const uint16_t* __restrict__ delta,
-                                                                  const uint16_t* __restrict__ weight,
-                                                                  uint16_t* __restrict__ y, int hidden, float eps) {
-    __shared__ float s_part[kNormThreads / kWave];
-    const int64_t base = (int64_t)blockIdx.x * hidden;
-    float v[kNormPasses][8];
-    u32x4 wraw[kNormPasses];   // the weight does not depend on the reduction: fetched up front
-    float ss = 0.f;
+__device__ __forceinline__ float row_load_ssq(uint16_t* __restrict__ residual, const uint16_t* __restrict__ delta,
+                                              int64_t base, int hidden, float (&v)[kNormPasses][8], float* s_tile) {
 #pragma unroll
     for (int p = 0; p < kNormPasses; ++p) {
         const int i = (p * kNormThreads + threadIdx.x) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[p][e] = 0.f;
         if (i < hidden) {
-            wraw[p] = *reinterpret_cast<const u32x4*>(weight + i);
             unpack8<T>(*reinterpret_cast<const u32x4*>(residual + base + i), v[p]);
             if (delta) {
                 float d[8];
@@ -64,16 +62,32 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
                 for (int e = 0; e < 8; ++e) v[p][e] = round_to<T>(v[p][e] + d[e]);
                 *reinterpret_cast<u32x4*>(residual + base + i) = pack8<T>(v[p]);
             }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) ss += v[p][e] * v[p][e];
         }
+        const float ts = tile_ssq(v[p]);   // every lane takes part; lanes past the row add zeros
+        if ((threadIdx.x & 15) == 0) s_tile[p * (kNormThreads / 16) + (threadIdx.x >> 4)] = ts;
     }
-    ss = wave_sum(ss);
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
     __syncthreads();
+    const int tiles = (hidden + 127) >> 7;
     float tot = 0.f;
+    for (int t = 0; t < tiles; ++t) tot += s_tile[t];
+    return tot;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __restrict__ residual,
+                                                                  const uint16_t* __restrict__ delta,
+                                                                  const uint16_t* __restrict__ weight,
+                                                                  uint16_t* __restrict__ y, int hidden, float eps) {
+    __shared__ float s_tile[kNormTiles];
+    const int64_t base = (int64_t)blockIdx.x * hidden;
+    float v[kNormPasses][8];
+    u32x4 wraw[kNormPasses];   // the weight does not depend on the reduction: fetched up front
 #pragma unroll
-    for (int w = 0; w < kNormThreads / kWave; ++w) tot += s_part[w];
+    for (int p = 0; p < kNormPasses; ++p) {
+        const int i = (p * kNormThreads + threadIdx.x) * 8;
+        if (i < hidden) wraw[p] = *reinterpret_cast<const u32x4*>(weight + i);
+    }
+    const float tot = row_load_ssq<T>(residual, delta, base, hidden, v, s_tile);
     const float r = rsqrtf(tot / (float)hidden + eps);
 #pragma unroll
     for (int p = 0; p < kNormPasses; ++p) {
@@ -82,10 +96,22 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
             float w[8], o[8];
             unpack8<T>(wraw[p], w);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = round_to<T>(v[p][e] * r) * w[e];
+            for (int e = 0; e < 8; ++e) o[e] = mul_round<T>(v[p][e], r) * w[e];
             *reinterpret_cast<u32x4*>(y + base + i) = pack8<T>(o);
         }
     }
+}
+
+// ssq[tile][row] = sum of squares of x[row, 128 tile .. 128 tile + 127]: the statistics an AWQ GEMV with an
+// RMSNorm prologue reads, for a residual stream that no GEMV with a residual epilogue has produced yet.
+template <typename T>
+__global__ __launch_bounds__(kNormThreads) void row_ssq_kernel(const uint16_t* __restrict__ x, float* __restrict__ ssq,
+                                                              int rows, int hidden) {
+    __shared__ float s_tile[kNormTiles];
+    float v[kNormPasses][8];
+    row_load_ssq<T>(const_cast<uint16_t*>(x), nullptr, (int64_t)blockIdx.x * hidden, hidden, v, s_tile);
+    const int tiles = (hidden + 127) >> 7;
+    if ((int)threadIdx.x < tiles) ssq[(size_t)threadIdx.x * rows + blockIdx.x] = s_tile[threadIdx.x];
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -736,6 +762,26 @@ extern "C" int nq_add_rmsnorm(void* residual, const void* delta, const void* wei
     else
         add_rmsnorm_kernel<BF16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>(
             (uint16_t*)residual, (const uint16_t*)delta, (const uint16_t*)weight, (uint16_t*)y, (int)hidden, eps);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" int nq_row_ssq(const void* x, float* ssq, int64_t rows, int64_t hidden, int dtype, void* stream) {
+    const char* fn = "nq_row_ssq";
+    if (!x || !ssq) return bad(fn, "null pointer argument");
+    if (!aligned16(x) || (reinterpret_cast<uintptr_t>(ssq) & 3u)) return bad(fn, "x must be 16-byte, ssq 4-byte aligned");
+    if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
+    if (rows <= 0 || hidden <= 0 || hidden % 8 != 0) return bad(fn, "rows > 0 and hidden a positive multiple of 8");
+    if (hidden > kNormThreads * 8 * kNormPasses || rows > 0x7fffffff) {
+        set_error("%s: hidden=%lld exceeds %d", fn, (long long)hidden, kNormThreads * 8 * kNormPasses);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    (void)hipGetLastError();
+    if (dtype == AWQ_F16)
+        row_ssq_kernel<F16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>((const uint16_t*)x, ssq, (int)rows, (int)hidden);
+    else
+        row_ssq_kernel<BF16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>((const uint16_t*)x, ssq, (int)rows, (int)hidden);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }

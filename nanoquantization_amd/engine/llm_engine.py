@@ -67,7 +67,7 @@ class _FusedLinear:
 
 class LLMEngine:
     def __init__(self, model: Qwen3QuantizedForCausalLM, max_batch: int, max_seq_len: int, block_size: int = 64,
-                 num_blocks: Optional[int] = None, use_graph: bool = True):
+                 num_blocks: Optional[int] = None, use_graph: bool = True, fuse_norm: bool = True):
         self.model = model.eval()
         p = next(model.parameters())
         self.device, self.dtype = p.device, p.dtype
@@ -94,6 +94,11 @@ class LLMEngine:
                            for l in layers] if self.swiglu_ok else None
         q0 = layers[0].self_attn.q_proj
         self.qkv_fused_ok = (self.hd == 128 and max_batch <= 64 and q0.group_size % 128 == 0 and q0.bias is None)
+        # residual add + RMSNorm folded into the neighbouring GEMVs (statistics handed from one to the next); not for
+        # models whose MLP weights at this batch run faster on the shared-chunk GEMV, which has no such form
+        hidden = q0.in_features
+        self.norm_fused_ok = (fuse_norm and self.qkv_fused_ok and self.swiglu_ok and hidden % 128 == 0
+                              and (max_batch <= 16 or 2 * self.inter * hidden < (50 << 20)))
         self.use_graph = use_graph
         self._graph = None
         B, dev = max_batch, self.device
@@ -155,6 +160,28 @@ class LLMEngine:
         x = m.embed_tokens(self.s_ids)                                   # residual stream [B, hidden]
         delta = None
         nl = len(m.layers)
+        if self.norm_fused_ok:
+            # five launches per block: the o_proj and down_proj GEMVs add into the residual stream and leave its
+            # RMSNorm statistics, the q|k|v and gate|up GEMVs normalise their input on the way in
+            ssq = ops.row_ssq(x)
+            for li, layer in enumerate(m.layers):
+                attn, lin, mlp = layer.self_attn, self.qkv[li], layer.mlp
+                prefetch_hint(attn.o_proj.qweight, attn.o_proj.qscales)
+                q = ops.awq_gemv_rmsnorm_qkv_rope_store(
+                    x, ssq, layer.input_layernorm.weight, eps, lin.qweight, lin.qscales, lin.qzeros,
+                    attn.q_norm.weight, attn.k_norm.weight, attn.rope.cos_sin_cache, pos, slots, self.cache.k[li],
+                    self.cache.v[li], self.nh, self.nkv, attn.q_norm.eps)
+                o = ops.paged_attention_decode(q, self.cache.k[li], self.cache.v[li], self.s_table, ctx, self.scale)
+                prefetch_hint(*self.gate_up_il[li][:2])
+                ops.awq_gemv_add_residual(o, attn.o_proj.qweight, attn.o_proj.qscales, attn.o_proj.qzeros, x, ssq)
+                prefetch_hint(mlp.down_proj.qweight, mlp.down_proj.qscales)
+                act = ops.awq_gemv_rmsnorm(x, ssq, layer.post_attention_layernorm.weight, eps, *self.gate_up_il[li],
+                                           gated=True)
+                if li + 1 < nl:
+                    prefetch_hint(self.qkv[li + 1].qweight, self.qkv[li + 1].qscales)
+                ops.awq_gemv_add_residual(act, mlp.down_proj.qweight, mlp.down_proj.qscales, mlp.down_proj.qzeros, x, ssq)
+            self._finish_step(ops.add_rmsnorm(x, None, m.norm.weight, m.norm.eps))
+            return
         for li, layer in enumerate(m.layers):
             attn = layer.self_attn
             gu = self.gate_up_il[li][:2] if self.swiglu_ok else (self.gate_up[li].qweight, self.gate_up[li].qscales)
@@ -181,7 +208,9 @@ class LLMEngine:
                 nq_ = self.qkv[li + 1]
                 prefetch_hint(nq_.qweight, nq_.qscales)
             delta = layer.mlp.down_proj(act)
-        h = ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps)
+        self._finish_step(ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps))
+
+    def _finish_step(self, h: torch.Tensor) -> None:
         nxt = ops.argmax_rows(self.model.lm_head(h))
         self.s_out.index_copy_(0, self.s_step, nxt.unsqueeze(0))
         self.s_ids.copy_(nxt)

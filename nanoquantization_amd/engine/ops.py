@@ -104,6 +104,95 @@ def awq_gemv_qkv_rope_store(x: torch.Tensor, qweight: torch.Tensor, qscales: tor
     return q
 
 
+def row_ssq(x: torch.Tensor) -> torch.Tensor:
+    """x [rows, hidden] -> fp32 [ceil(hidden / 128), rows]: the sum of squares of every 128-column tile of every row,
+    the RMSNorm statistics awq_gemv_rmsnorm reads."""
+    dev = _dev(x)
+    rows, hidden = x.shape
+    ssq = torch.empty((hidden + 127) // 128, rows, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_row_ssq(x.data_ptr(), ssq.data_ptr(), rows, hidden, _lib.dtype_id(x.dtype), _stream()))
+    return ssq
+
+
+def _gemv_ws(dev, M, N, K):
+    stream = _stream()
+    ws = _lib.workspace(dev, stream, _lib.lib().awq_gemv_workspace_bytes(M, N, K))
+    return (None if ws is None else ws.data_ptr()), (0 if ws is None else ws.numel()), stream
+
+
+def awq_gemv_add_residual(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor,
+                          residual: torch.Tensor, ssq: torch.Tensor) -> None:
+    """residual [M <= 64, N] += x @ W IN PLACE (rounded like a linear followed by an addition); ssq [N / 128, M]
+    receives the tile sums of squares of the new residual."""
+    dev = _dev(x, qweight, qscales, qzeros, residual, ssq)
+    M, K = x.shape
+    N = qscales.shape[1]
+    g = K // qscales.shape[0]
+    assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    assert residual.shape == (M, N) and residual.dtype == x.dtype
+    assert ssq.shape == (N // 128, M) and ssq.dtype == torch.float32 and N % 128 == 0
+    with torch.cuda.device(dev):
+        ws, ws_bytes, stream = _gemv_ws(dev, M, N, K)
+        _lib.check(_lib.lib().awq_gemv_add_residual(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(),
+                                                    qzeros.data_ptr(), residual.data_ptr(), ssq.data_ptr(), M, N, K, g,
+                                                    _lib.dtype_id(x.dtype), ws, ws_bytes, stream))
+
+
+def awq_gemv_rmsnorm(x: torch.Tensor, ssq: torch.Tensor, norm_weight: torch.Tensor, eps: float, qweight: torch.Tensor,
+                     qscales: torch.Tensor, qzeros: torch.Tensor, gated: bool = False) -> torch.Tensor:
+    """(RMSNorm(x) * norm_weight) @ W for the residual stream x [M <= 64, K] with its statistics ssq [K / 128, M];
+    gated: interleaved gate|up buffers, returns SiLU(gate) * up [M, N / 2]."""
+    dev = _dev(x, ssq, norm_weight, qweight, qscales, qzeros)
+    M, K = x.shape
+    N = qscales.shape[1]
+    g = K // qscales.shape[0]
+    assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    assert K % 128 == 0 and ssq.shape == (K // 128, M) and ssq.dtype == torch.float32
+    assert norm_weight.shape == (K,) and norm_weight.dtype == x.dtype
+    out = torch.empty(M, N // 2 if gated else N, dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        ws, ws_bytes, stream = _gemv_ws(dev, M, N, K)
+        _lib.check(_lib.lib().awq_gemv_rmsnorm(x.data_ptr(), ssq.data_ptr(), norm_weight.data_ptr(), eps,
+                                               qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(), out.data_ptr(),
+                                               M, N, K, g, 1 if gated else 0, _lib.dtype_id(x.dtype), ws, ws_bytes, stream))
+    return out
+
+
+def awq_gemv_rmsnorm_qkv_rope_store(x: torch.Tensor, ssq: torch.Tensor, norm_weight: torch.Tensor, norm_eps: float,
+                                    qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor,
+                                    q_weight: torch.Tensor, k_weight: torch.Tensor, cos_sin: torch.Tensor,
+                                    positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor,
+                                    v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, eps: float) -> torch.Tensor:
+    """awq_gemv_qkv_rope_store on RMSNorm(x) * norm_weight, x [M <= 64, K] the residual stream, ssq [K / 128, M]."""
+    dev = _dev(x, ssq, norm_weight, qweight, qscales, qzeros, q_weight, k_weight, cos_sin, positions, slots, k_cache,
+               v_cache)
+    M, K = x.shape
+    N = qscales.shape[1]
+    g = K // qscales.shape[0]
+    hd = 128
+    assert N == (num_heads + 2 * num_kv_heads) * hd
+    assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    assert K % 128 == 0 and ssq.shape == (K // 128, M) and ssq.dtype == torch.float32
+    assert norm_weight.shape == (K,) and norm_weight.dtype == x.dtype
+    assert q_weight.shape == (hd,) and k_weight.shape == (hd,) and q_weight.dtype == x.dtype and k_weight.dtype == x.dtype
+    assert k_cache.dtype == x.dtype and v_cache.dtype == x.dtype and k_cache.shape == v_cache.shape
+    assert k_cache.dim() == 4 and k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == hd
+    assert cos_sin.dtype == torch.float32 and cos_sin.numel() % hd == 0
+    assert positions.dtype == torch.int64 and slots.dtype == torch.int64 and positions.numel() == M and slots.numel() == M
+    block_size = k_cache.shape[2]
+    num_slots = k_cache.numel() // (num_kv_heads * hd)
+    q = torch.empty(M, num_heads, hd, dtype=x.dtype, device=dev)
+    with torch.cuda.device(dev):
+        ws, ws_bytes, stream = _gemv_ws(dev, M, N, K)
+        _lib.check(_lib.lib().awq_gemv_rmsnorm_qkv_rope_store(
+            x.data_ptr(), ssq.data_ptr(), norm_weight.data_ptr(), norm_eps, qweight.data_ptr(), qscales.data_ptr(),
+            qzeros.data_ptr(), q_weight.data_ptr(), k_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(),
+            slots.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), M, N, K, g, num_heads, num_kv_heads,
+            cos_sin.numel() // hd, num_slots, block_size, eps, _lib.dtype_id(x.dtype), ws, ws_bytes, stream))
+    return q
+
+
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                            context_lens: torch.Tensor, scale: float) -> torch.Tensor:
     """q [batch, nh, hd]; caches [num_blocks, nkv, block_size, hd]; block_table int32 [batch, max_blocks];

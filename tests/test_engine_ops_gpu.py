@@ -322,3 +322,110 @@ def test_argmax_rows(dtype, rows, vocab):
     logits[0, vocab - 1] = 3.0
     logits[0, vocab // 2] = 3.0
     assert ops.argmax_rows(logits)[0].item() == vocab // 2
+
+
+def _packed(K, N, dtype, g):
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    qs = (torch.rand(K // 128, N, device="cuda", generator=g) * 0.02 + 0.001).to(dtype)
+    qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    return qw, qs, qz
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,hidden", [(1, 1024), (32, 1024), (7, 5120), (3, 8192), (5, 136)])
+def test_row_ssq(dtype, rows, hidden):
+    """Tile sums of squares against torch (fp32, a few ulps: another summation order)."""
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(rows + hidden)
+    x = torch.randn(rows, hidden, device="cuda", generator=g).to(dtype)
+    ssq = ops.row_ssq(x)
+    tiles = (hidden + 127) // 128
+    assert ssq.shape == (tiles, rows) and ssq.dtype == torch.float32
+    pad = torch.zeros(rows, tiles * 128, device="cuda")
+    pad[:, :hidden] = x.float()
+    want = pad.view(rows, tiles, 128).double().pow(2).sum(-1).t()
+    assert torch.allclose(ssq.double(), want, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,N", [(1, 2048, 1024), (32, 2048, 1024), (16, 3072, 1024), (64, 1024, 5120),
+                                   (5, 8192, 256), (33, 25600, 1024)])
+def test_gemv_add_residual_equals_unfused(dtype, M, K, N):
+    """o_proj / down_proj with the residual addition and the RMSNorm statistics in the epilogue against the GEMV
+    followed by the add + norm kernel: residual stream and statistics bit for bit."""
+    import nanoquantization_amd as nq
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(M * 7 + K + N)
+    qw, qs, qz = _packed(K, N, dtype, g)
+    x = (torch.randn(M, K, device="cuda", generator=g) * 0.3).to(dtype)
+    res = torch.randn(M, N, device="cuda", generator=g).to(dtype)
+    print(f"gemv_add_residual M={M} K={K} N={N} {dtype}", flush=True)
+    want = res.clone()
+    w = torch.ones(N, dtype=dtype, device="cuda")
+    ops.add_rmsnorm(want, nq.awq_gemm(x, qw, qs, qz, 8), w, 1e-6)     # updates `want` in place
+    got = res.clone()
+    ssq = torch.full((N // 128, M), float("nan"), device="cuda")
+    ops.awq_gemv_add_residual(x, qw, qs, qz, got, ssq)
+    assert torch.equal(got, want)
+    assert torch.equal(ssq, ops.row_ssq(want))
+    again = res.clone()
+    ssq2 = torch.empty_like(ssq)
+    ops.awq_gemv_add_residual(x, qw, qs, qz, again, ssq2)              # workspace counters were left clean
+    assert torch.equal(again, got) and torch.equal(ssq2, ssq)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,N,gated", [(1, 1024, 4096, False), (32, 1024, 6144, True), (16, 2048, 2048, True),
+                                         (64, 1024, 4096, False), (7, 5120, 1280, True), (40, 4096, 512, False)])
+def test_gemv_rmsnorm_equals_unfused(dtype, M, K, N, gated):
+    """RMSNorm in the GEMV's prologue against the norm kernel followed by the plain (or gated) GEMV: bit for bit."""
+    import nanoquantization_amd as nq
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(M * 11 + K + N)
+    qw, qs, qz = _packed(K, N, dtype, g)
+    x = torch.randn(M, K, device="cuda", generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(K, device="cuda", generator=g)).to(dtype)
+    print(f"gemv_rmsnorm M={M} K={K} N={N} gated={gated} {dtype}", flush=True)
+    h = ops.add_rmsnorm(x.clone(), None, w, 1e-6)
+    want = ops.awq_gemv_swiglu(h, qw, qs, qz) if gated else nq.awq_gemm(h, qw, qs, qz, 8)
+    got = ops.awq_gemv_rmsnorm(x, ops.row_ssq(x), w, 1e-6, qw, qs, qz, gated=gated)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,nh,nkv", [(1, 1024, 16, 8), (32, 1024, 16, 8), (64, 2048, 4, 2)])
+def test_gemv_rmsnorm_qkv_rope_store_equals_unfused(dtype, M, K, nh, nkv):
+    from nanoquantization_amd.engine import ops
+    from nanoquantization_amd.layers.rope import RoPE
+    hd, bs, max_pos, num_slots = 128, 16, 512, 256
+    N = (nh + 2 * nkv) * hd
+    g = torch.Generator(device="cuda").manual_seed(M * 17 + K + nh)
+    qw, qs, qz = _packed(K, N, dtype, g)
+    x = torch.randn(M, K, device="cuda", generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(K, device="cuda", generator=g)).to(dtype)
+    nqw = (1 + 0.1 * torch.randn(hd, device="cuda", generator=g)).to(dtype)
+    nkw = (1 + 0.1 * torch.randn(hd, device="cuda", generator=g)).to(dtype)
+    pos = torch.randint(0, max_pos, (M,), device="cuda", generator=g)
+    slots = torch.randperm(num_slots, device="cuda", generator=g)[:M]
+    rope = RoPE(hd, max_pos).cuda()
+    print(f"gemv_rmsnorm_qkv_rope_store M={M} K={K} nh={nh} nkv={nkv} {dtype}", flush=True)
+    kc = torch.zeros(num_slots // bs, nkv, bs, hd, dtype=dtype, device="cuda")
+    vc, kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(kc), torch.zeros_like(kc)
+    h = ops.add_rmsnorm(x.clone(), None, w, 1e-6)
+    q2 = ops.awq_gemv_qkv_rope_store(h, qw, qs, qz, nqw, nkw, rope.cos_sin_cache, pos, slots, kc2, vc2, nh, nkv, 1e-6)
+    q = ops.awq_gemv_rmsnorm_qkv_rope_store(x, ops.row_ssq(x), w, 1e-6, qw, qs, qz, nqw, nkw, rope.cos_sin_cache, pos,
+                                            slots, kc, vc, nh, nkv, 1e-6)
+    assert torch.equal(q, q2) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
+
+
+def test_norm_fused_entry_points_reject_unsupported():
+    from nanoquantization_amd import _lib
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(5)
+    K, N = 256, 136                                     # N is not a multiple of 128: no staged kernel
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
+    qs = torch.rand(K // 128, N, device="cuda", generator=g).half()
+    qz = torch.zeros(K // 128, N // 8, dtype=torch.int32, device="cuda")
+    x = torch.randn(4, K, device="cuda", generator=g).half()
+    with pytest.raises(_lib.AwqHipError):
+        ops.awq_gemv_rmsnorm(x, ops.row_ssq(x), torch.ones(K, dtype=torch.half, device="cuda"), 1e-6, qw, qs, qz)

@@ -223,3 +223,22 @@ def test_engine_continuous_batching():
     small = LLMEngine(model, max_batch=2, max_seq_len=64, block_size=16, num_blocks=2, use_graph=False)
     with pytest.raises(RuntimeError, match="KV cache too small"):
         small.serve([(list(range(40)), 8)])
+
+
+@pytest.mark.gpu
+def test_engine_norm_fused_decode_equals_separate_kernels():
+    """The decode step with the residual adds and RMSNorms folded into the GEMVs (five launches per block) produces
+    the tokens of the step with stand-alone add + norm kernels (seven): every fused piece returns the same bits."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import random_awq_qwen3
+    print("engine: norm-fused decode vs separate kernels", flush=True)
+    cfg = dict(TINY, hidden_size=512, head_dim=128, intermediate_size=768)
+    model = random_awq_qwen3(cfg, seed=11, std=0.05)
+    torch.manual_seed(12)
+    prompts = torch.randint(0, 512, (5, 23)).tolist()
+    outs = []
+    for fuse in (False, True):
+        eng = LLMEngine(model, max_batch=8, max_seq_len=96, block_size=16, use_graph=True, fuse_norm=fuse)
+        assert eng.norm_fused_ok == fuse
+        outs.append(eng.generate(prompts, 20))
+    assert outs[0] == outs[1]
