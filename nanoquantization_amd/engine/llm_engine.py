@@ -12,7 +12,10 @@ start-up; the checkpoint layout is untouched.
 Decode.  One step = embedding, then per block: add+RMSNorm kernel, fused q|k|v AWQ GEMV, a kernel that
 does per-head q/k RMSNorm + rotary and writes k/v into their cache slots, paged attention (flash
 decoding over the block table), o_proj GEMV, add+RMSNorm, fused gate|up GEMV, SiLU*up kernel, down GEMV
-(include/nq_engine_ops.h + include/awq_hip.h).  All per-step state lives in fixed device buffers (token
+(include/nq_engine_ops.h + include/awq_hip.h).  Where the shapes allow (head_dim 128, hidden a multiple of 128, gate|up
+interleaved) the two add+RMSNorm kernels disappear as well: the o_proj and down_proj GEMVs add into the residual
+stream and leave its RMSNorm statistics, the q|k|v and gate|up GEMVs normalise their input on the way in -- five
+launches per block, same bits.  All per-step state lives in fixed device buffers (token
 ids, positions, active mask, block table, step counter, output tokens) and the step advances that
 state itself, so it is captured once in a HIP graph and replayed with no host work between steps.
 
