@@ -285,6 +285,7 @@ def main():
                 "decode_ms_per_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
                 "prefill_s": round(st["prefill_s"], 4),
                 "prefill_tok_per_s": round(B * P / st["prefill_s"], 1),
+                "launches_per_block": 5 if eng.norm_fused_ok else 7,
             }
             del eng, model
             torch.cuda.empty_cache()

@@ -240,5 +240,7 @@ def test_engine_norm_fused_decode_equals_separate_kernels():
     for fuse in (False, True):
         eng = LLMEngine(model, max_batch=8, max_seq_len=96, block_size=16, use_graph=True, fuse_norm=fuse)
         assert eng.norm_fused_ok == fuse
-        outs.append(eng.generate(prompts, 20))
+        # the static batch, then the same engine under continuous batching with ragged requests
+        reqs = [(p[: 5 + 3 * i], 6 + i) for i, p in enumerate(prompts)]
+        outs.append((eng.generate(prompts, 20), eng.serve(reqs)))
     assert outs[0] == outs[1]
