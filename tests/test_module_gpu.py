@@ -62,3 +62,23 @@ def test_state_dict_roundtrip_keeps_outputs():
     mb2 = mb2.to("cuda")
     assert mb2.bias.dtype == torch.bfloat16
     assert (mb(x).float() - mb2(x).float()).abs().max().item() <= 2.0 ** -8 * mb.bias.abs().max().item() + 2e-3
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_forward_empty_and_boundary_row_counts(bias):
+    """No rows at all, and the row counts where the dispatch changes kernel (16/17 one m-tile vs row blocks, 64/65
+    GEMV vs GEMM, 1023/1024 fused vs two-pass): shape, dtype and the fp32 oracle at every one of them."""
+    K, N, g = 512, 384, 128
+    m = _module(K, N, g, torch.bfloat16, bias, seed=3)
+    for shape in [(0, K), (2, 0, K)]:
+        y = m(torch.zeros(*shape, dtype=torch.bfloat16, device="cuda"))
+        assert y.shape == tuple(shape[:-1]) + (N,) and y.dtype == torch.bfloat16 and y.numel() == 0
+    qw, qz, qs = m.qweight.cpu().numpy(), m.qzeros.cpu().numpy(), to_bits(m.qscales)
+    b = m.bias.float().cpu().numpy() if bias else None
+    for M in (16, 17, 64, 65, 1023, 1024):
+        print(f"forward boundary M={M} bias={bias}", flush=True)
+        torch.manual_seed(M)
+        x = torch.randn(M, K).to(torch.bfloat16).cuda()
+        ref = o.linear_fp32(to_bits(x), qw, qz, qs, "bf16", b)
+        err = o.max_rel_err(m(x).float().cpu().numpy(), ref)
+        assert err <= 6e-3, (M, err)
