@@ -1303,9 +1303,9 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
         if (allow_shared_chunk && M > 16 && N % 512 == 0 && N >= 5120 &&
-            K * N >= (M > 32 ? (50ll << 20) : (100ll << 20))) {
-            // 17..64 rows on the largest weights (from sweeps: Qwen3-32B MLP and, above 32 rows, its fused
-            // q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
+            K * N >= (M > 32 ? (50ll << 20) : 95000000ll)) {
+            // 17..64 rows on the largest weights (from sweeps: the fused gate|up of Qwen3-8B and the MLP of
+            // Qwen3-14B/32B and, above 32 rows, the 32B fused q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
             // one workgroup per CU exists, four chunks per split at least.  Below these sizes re-reading the
             // weights once per block of 16 rows (mostly from cache) is faster than the shared chunk's second pass.
             v = M > 32 ? kWideM4 : kWideM2;
@@ -1319,10 +1319,29 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             const int64_t cap = chunks < 64 ? (chunks / 2 < 10 ? chunks / 2 : 10) : 32;
             if (s > cap) s = cap;
             s = balance_splits(chunks, s, 4, cap);
-        } else if (tiles * row_blocks < 200) {
-            s = cdiv(200, tiles * row_blocks);   // about 200 workgroups
-            if (s > chunks / 4) s = chunks / 4;
-            s = balance_splits(chunks, s, 4, chunks / 4);
+        } else {
+            // 5..64 rows.  A CU streams at a fixed rate whatever the number of workgroups on it, so the launch lasts
+            // as long as the CU with the most bytes: at least about 200 workgroups, and a count that fills whole
+            // rounds of the 256 CUs (272 column tiles unsplit = two rounds, the second almost empty: 48.9 us
+            // against 34.9 us cut four ways, 5120 x 34816 at 16 rows).  Each further split costs a tail
+            // (publish, fetch, add) that grows with the rows of a block, hence the penalty: at 5120 x 25600 five
+            // splits win at 8 rows (22.9 against 24.4 us) and lose at 16 (27.4 against 24.7).
+            const int64_t wgs = tiles * row_blocks;
+            const int64_t cap = chunks / 4 > 1 ? chunks / 4 : 1;
+            int64_t s0 = wgs < 200 ? cdiv(200, wgs) : 1;
+            if (s0 > cap) s0 = cap;
+            const int64_t hi = s0 + 5 < cap ? s0 + 5 : cap;
+            double best_score = -1.0;
+            for (int64_t c = s0; c <= hi; ++c) {
+                const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
+                const double eff_wave = (double)chunks / (double)(splits * 4 * cdiv(cps, 4));
+                const double eff_cu = (double)(wgs * splits) / (double)(256 * cdiv(wgs * splits, 256));
+                const double score = eff_wave * eff_cu - 0.05 * (double)(M < 16 ? M : 16) / 16.0 * (double)(c - s0);
+                if (score > best_score + 1e-9) {
+                    best_score = score;
+                    s = c;
+                }
+            }
         }
         if (s < 1) s = 1;
         *variant = v;
