@@ -1482,12 +1482,15 @@ extern "C" size_t awq_gemv_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, i
 extern "C" size_t awq_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (K < 32 || N < 8 || M < 1) return 0;
     int v, s;
-    // the caller does not pass the group size here: cover both data paths
-    awq::pick_gemv(M, N, K, 128, &v, &s);
-    const size_t a = awq::gemv_ws_bytes(M, N, K, v, s);
-    awq::pick_gemv(M, N, K, 32, &v, &s);
-    const size_t b = awq::gemv_ws_bytes(M, N, K, v, s);
-    return a > b ? a : b;
+    // the caller passes neither the group size nor the entry point: cover both data paths, and the staged path
+    // with and without the shared-chunk kernel (the fused forms never take it)
+    size_t need = 0;
+    for (int form = 0; form < 3; ++form) {
+        awq::pick_gemv(M, N, K, form == 2 ? 32 : 128, &v, &s, form != 1);
+        const size_t b = awq::gemv_ws_bytes(M, N, K, v, s);
+        if (b > need) need = b;
+    }
+    return need;
 }
 
 extern "C" int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void* qscales,

@@ -429,3 +429,35 @@ def test_norm_fused_entry_points_reject_unsupported():
     x = torch.randn(4, K, device="cuda", generator=g).half()
     with pytest.raises(_lib.AwqHipError):
         ops.awq_gemv_rmsnorm(x, ops.row_ssq(x), torch.ones(K, dtype=torch.half, device="cuda"), 1e-6, qw, qs, qz)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_fused_forms_on_largest_decode_shapes(dtype):
+    """Qwen3-32B widths at 64 rows, where the plain GEMV runs the shared-chunk kernel (another summation order) and
+    the fused forms stay on the row-block kernel: results within one rounding step of the separate kernels, the
+    statistics exactly those of the residual that was stored."""
+    import nanoquantization_amd as nq
+    from nanoquantization_amd.engine import ops
+    M = 64
+    g = torch.Generator(device="cuda").manual_seed(64)
+    # down_proj 25600 -> 5120 with the residual epilogue
+    K, N = 25600, 5120
+    qw, qs, qz = _packed(K, N, dtype, g)
+    x = (torch.randn(M, K, device="cuda", generator=g) * 0.1).to(dtype)
+    res = torch.randn(M, N, device="cuda", generator=g).to(dtype)
+    print(f"norm-fused forms at 32B widths {dtype}", flush=True)
+    want = res.clone()
+    ops.add_rmsnorm(want, nq.awq_gemm(x, qw, qs, qz, 8), torch.ones(N, dtype=dtype, device="cuda"), 1e-6)
+    got = res.clone()
+    ssq = torch.empty(N // 128, M, device="cuda")
+    ops.awq_gemv_add_residual(x, qw, qs, qz, got, ssq)
+    _close(got, want.float(), dtype, what="residual")
+    assert torch.equal(ssq, ops.row_ssq(got))
+    # fused gate|up 5120 -> 2 x 25600 with the RMSNorm prologue
+    K, N = 5120, 51200
+    qw, qs, qz = _packed(K, N, dtype, g)
+    xr = torch.randn(M, K, device="cuda", generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(K, device="cuda", generator=g)).to(dtype)
+    want = ops.awq_gemv_swiglu(ops.add_rmsnorm(xr.clone(), None, w, 1e-6), qw, qs, qz)
+    got = ops.awq_gemv_rmsnorm(xr, ops.row_ssq(xr), w, 1e-6, qw, qs, qz, gated=True)
+    _close(got, want.float(), dtype, what="gated product")
