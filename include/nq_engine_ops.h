@@ -86,6 +86,17 @@ int nq_silu_mul_interleaved(const void* gate_up, void* out, int64_t rows, int64_
  * (nanoquantization/models/qwen3_quantized.py:312-314). */
 int nq_argmax_rows(const void* logits, int64_t* out, int64_t rows, int64_t vocab, int dtype, void* stream);
 
+/* Bookkeeping of a decode step over the paged cache (the reference has no generation loop; one launch each instead of
+ * a dozen elementwise ones).  `active` is one byte per row (torch.bool).
+ * nq_decode_prepare: slots[r] = active[r] ? block_table[r][positions[r] / block_size] * block_size +
+ *   positions[r] % block_size : -1 (the slot convention of nq_qk_norm_rope_store), context_lens[r] = positions[r] + 1.
+ * nq_decode_advance: out_log[step[0]][r] = next_tokens[r] (skipped when step[0] is outside [0, out_rows)),
+ *   ids[r] = next_tokens[r], positions[r] += active[r], step[0] += 1. */
+int nq_decode_prepare(const int64_t* positions, const uint8_t* active, const int32_t* block_table, int64_t* slots,
+                      int32_t* context_lens, int64_t rows, int64_t max_blocks, int64_t block_size, void* stream);
+int nq_decode_advance(const int64_t* next_tokens, const uint8_t* active, int64_t* out_log, int64_t* ids,
+                      int64_t* positions, int64_t* step, int64_t rows, int64_t out_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

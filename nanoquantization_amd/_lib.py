@@ -62,6 +62,8 @@ SYMBOLS = {
     "nq_silu_mul": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "nq_silu_mul_interleaved": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "nq_argmax_rows": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "nq_decode_prepare": (_int, [_vp] * 5 + [_i64] * 3 + [_vp]),
+    "nq_decode_advance": (_int, [_vp] * 6 + [_i64] * 2 + [_vp]),
 }
 
 

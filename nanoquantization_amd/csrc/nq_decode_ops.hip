@@ -737,6 +737,42 @@ int launch_attn_g(int G, const void* q, const void* kc, const void* vc, const in
     return AWQ_ERR_UNSUPPORTED;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Bookkeeping of a decode step over the paged cache, one launch each instead of a dozen elementwise ones.
+// prepare: the cache slot and the context length of the token each row feeds at its position.
+__global__ __launch_bounds__(256) void decode_prepare_kernel(const int64_t* __restrict__ pos,
+                                                            const uint8_t* __restrict__ active,
+                                                            const int32_t* __restrict__ table,
+                                                            int64_t* __restrict__ slots, int32_t* __restrict__ ctx,
+                                                            int rows, int max_blocks, int block_size) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    int64_t p = pos[r];
+    p = p < 0 ? 0 : p;
+    int64_t blk = p / block_size;
+    blk = blk >= max_blocks ? max_blocks - 1 : blk;
+    slots[r] = active[r] ? (int64_t)table[(int64_t)r * max_blocks + blk] * block_size + p % block_size : -1;
+    ctx[r] = (int32_t)(p + 1);
+}
+
+// advance: the sampled tokens become row step[0] of the output log and the next step's input; active rows move on
+// one position; the step counter goes up.  One workgroup, so that every thread has read the counter before it changes.
+__global__ __launch_bounds__(1024) void decode_advance_kernel(const int64_t* __restrict__ next,
+                                                             const uint8_t* __restrict__ active,
+                                                             int64_t* __restrict__ out, int64_t* __restrict__ ids,
+                                                             int64_t* __restrict__ pos, int64_t* __restrict__ step,
+                                                             int rows, int64_t out_rows) {
+    const int64_t s = step[0];
+    __syncthreads();
+    for (int r = threadIdx.x; r < rows; r += blockDim.x) {
+        const int64_t t = next[r];
+        if (s >= 0 && s < out_rows) out[s * rows + r] = t;
+        ids[r] = t;
+        if (active[r]) pos[r] += 1;
+    }
+    if (threadIdx.x == 0) step[0] = s + 1;
+}
+
 }  // namespace
 }  // namespace awq
 
@@ -916,6 +952,33 @@ extern "C" int nq_argmax_rows(const void* logits, int64_t* out, int64_t rows, in
         argmax_rows_kernel<F16><<<dim3((unsigned)rows), dim3(1024), 0, st>>>((const uint16_t*)logits, out, (int)vocab);
     else
         argmax_rows_kernel<BF16><<<dim3((unsigned)rows), dim3(1024), 0, st>>>((const uint16_t*)logits, out, (int)vocab);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" int nq_decode_prepare(const int64_t* positions, const uint8_t* active, const int32_t* block_table,
+                                 int64_t* slots, int32_t* context_lens, int64_t rows, int64_t max_blocks,
+                                 int64_t block_size, void* stream) {
+    const char* fn = "nq_decode_prepare";
+    if (!positions || !active || !block_table || !slots || !context_lens) return bad(fn, "null pointer argument");
+    if (rows <= 0 || max_blocks <= 0 || block_size <= 0 || rows > 0x7fffffff || max_blocks > 0x7fffffff ||
+        block_size > 0x7fffffff)
+        return bad(fn, "rows, max_blocks and block_size must be positive 31-bit counts");
+    (void)hipGetLastError();
+    decode_prepare_kernel<<<dim3((unsigned)cdiv(rows, 256)), dim3(256), 0, (hipStream_t)stream>>>(
+        positions, active, block_table, slots, context_lens, (int)rows, (int)max_blocks, (int)block_size);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
+}
+
+extern "C" int nq_decode_advance(const int64_t* next_tokens, const uint8_t* active, int64_t* out_log, int64_t* ids,
+                                 int64_t* positions, int64_t* step, int64_t rows, int64_t out_rows, void* stream) {
+    const char* fn = "nq_decode_advance";
+    if (!next_tokens || !active || !out_log || !ids || !positions || !step) return bad(fn, "null pointer argument");
+    if (rows <= 0 || rows > 0x7fffffff || out_rows <= 0) return bad(fn, "rows and out_rows must be positive");
+    (void)hipGetLastError();
+    decode_advance_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>(next_tokens, active, out_log, ids, positions,
+                                                                         step, (int)rows, out_rows);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }

@@ -156,10 +156,8 @@ class LLMEngine:
     def _decode_step(self) -> None:
         m, bs, eps = self.model.model, self.block_size, self.eps
         pos = self.s_pos
-        blk = self.s_table.gather(1, (pos // bs).unsqueeze(1)).squeeze(1).long()
-        # idle rows read row 0's table but write nothing: slot -1 is skipped by the kernel
-        slots = torch.where(self.s_active, blk * bs + pos % bs, torch.full_like(pos, -1))
-        ctx = (pos + 1).to(torch.int32)
+        # idle rows read row 0's table but write nothing: slot -1 is skipped by the kernels
+        slots, ctx = ops.decode_prepare(pos, self.s_active, self.s_table, bs)
         x = m.embed_tokens(self.s_ids)                                   # residual stream [B, hidden]
         delta = None
         nl = len(m.layers)
@@ -215,10 +213,8 @@ class LLMEngine:
 
     def _finish_step(self, h: torch.Tensor) -> None:
         nxt = ops.argmax_rows(self.model.lm_head(h))
-        self.s_out.index_copy_(0, self.s_step, nxt.unsqueeze(0))
-        self.s_ids.copy_(nxt)
-        self.s_pos.add_(self.s_active.to(torch.long))               # idle rows stay where they are
-        self.s_step.add_(1)
+        # log the tokens, feed them back, move the active rows on (idle rows stay where they are), count the step
+        ops.decode_advance(nxt, self.s_active, self.s_out, self.s_ids, self.s_pos, self.s_step)
 
     def _state(self):
         return [self.s_ids, self.s_pos, self.s_step]

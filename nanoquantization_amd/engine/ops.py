@@ -242,6 +242,36 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def decode_prepare(positions: torch.Tensor, active: torch.Tensor, block_table: torch.Tensor, block_size: int):
+    """positions int64 [rows], active bool [rows], block_table int32 [rows, max_blocks] -> (slots int64 [rows] with -1
+    for idle rows, context_lens int32 [rows] = positions + 1)."""
+    dev = _dev(positions, active, block_table)
+    rows = positions.numel()
+    assert positions.dtype == torch.int64 and active.dtype == torch.bool and block_table.dtype == torch.int32
+    assert active.numel() == rows and block_table.dim() == 2 and block_table.shape[0] == rows
+    slots = torch.empty(rows, dtype=torch.int64, device=dev)
+    ctx = torch.empty(rows, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_decode_prepare(positions.data_ptr(), active.data_ptr(), block_table.data_ptr(),
+                                                slots.data_ptr(), ctx.data_ptr(), rows, block_table.shape[1], block_size,
+                                                _stream()))
+    return slots, ctx
+
+
+def decode_advance(next_tokens: torch.Tensor, active: torch.Tensor, out_log: torch.Tensor, ids: torch.Tensor,
+                   positions: torch.Tensor, step: torch.Tensor) -> None:
+    """IN PLACE: out_log[step[0]] = next_tokens, ids = next_tokens, positions += active, step += 1."""
+    dev = _dev(next_tokens, active, out_log, ids, positions, step)
+    rows = next_tokens.numel()
+    assert all(t.dtype == torch.int64 for t in (next_tokens, out_log, ids, positions, step)) and active.dtype == torch.bool
+    assert out_log.dim() == 2 and out_log.shape[1] == rows and ids.numel() == rows and positions.numel() == rows
+    assert active.numel() == rows and step.numel() == 1
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_decode_advance(next_tokens.data_ptr(), active.data_ptr(), out_log.data_ptr(),
+                                                ids.data_ptr(), positions.data_ptr(), step.data_ptr(), rows,
+                                                out_log.shape[0], _stream()))
+
+
 def interleave_gate_up(gate, up):
     """Packed buffers (qweight, qscales, qzeros) of the gate and the up projection -> one set with the word
     columns interleaved (word 2t = gate word t, word 2t+1 = up word t), the layout awq_gemv_swiglu takes."""

@@ -461,3 +461,28 @@ def test_norm_fused_forms_on_largest_decode_shapes(dtype):
     want = ops.awq_gemv_swiglu(ops.add_rmsnorm(xr.clone(), None, w, 1e-6), qw, qs, qz)
     got = ops.awq_gemv_rmsnorm(xr, ops.row_ssq(xr), w, 1e-6, qw, qs, qz, gated=True)
     _close(got, want.float(), dtype, what="gated product")
+
+
+def test_decode_prepare_and_advance():
+    """The step's bookkeeping kernels against the torch expressions they stand in for."""
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator().manual_seed(9)
+    rows, max_blocks, bs = 37, 6, 16
+    pos = torch.randint(0, max_blocks * bs, (rows,), generator=g).cuda()
+    active = (torch.rand(rows, generator=g) > 0.3).cuda()
+    table = torch.randint(0, 500, (rows, max_blocks), generator=g).to(torch.int32).cuda()
+    slots, ctx = ops.decode_prepare(pos, active, table, bs)
+    blk = table.gather(1, (pos // bs).unsqueeze(1)).squeeze(1).long()
+    assert torch.equal(slots, torch.where(active, blk * bs + pos % bs, torch.full_like(pos, -1)))
+    assert torch.equal(ctx, (pos + 1).to(torch.int32))
+    out = torch.full((5, rows), -7, dtype=torch.long, device="cuda")
+    ids = torch.zeros(rows, dtype=torch.long, device="cuda")
+    step = torch.tensor([3], device="cuda")
+    nxt = torch.randint(0, 1000, (rows,), generator=g).cuda()
+    pos0 = pos.clone()
+    ops.decode_advance(nxt, active, out, ids, pos, step)
+    assert torch.equal(out[3], nxt) and (out[[0, 1, 2, 4]] == -7).all()
+    assert torch.equal(ids, nxt) and torch.equal(pos, pos0 + active.long()) and step.item() == 4
+    ops.decode_advance(nxt, active, out, ids, pos, step)
+    ops.decode_advance(nxt, active, out, ids, pos, step)          # step 5 is past the log: nothing is written there
+    assert step.item() == 6 and torch.equal(out[4], nxt) and torch.equal(pos, pos0 + 3 * active.long())
