@@ -32,6 +32,10 @@ int nq_add_rmsnorm(void* residual, const void* delta, const void* weight, void* 
  * stream that no awq_gemv_add_residual has produced (the embedding output of a decode step).  hidden % 8 == 0,
  * hidden <= 8192.  The mean of squares of RMSNorm.rms_norm, nanoquantization/layers/norm.py:18-32. */
 int nq_row_ssq(const void* x, float* ssq, int64_t rows, int64_t hidden, int dtype, void* stream);
+/* The same with the embedding lookup in front: x_out[r] = table[ids[r]] (ids clamped to [0, table_rows)), ssq of x_out.
+ * Qwen3QuantizedModel.forward's embed_tokens, nanoquantization/models/qwen3_quantized.py:259-273. */
+int nq_embed_row_ssq(const int64_t* ids, const void* table, void* x_out, float* ssq, int64_t rows, int64_t hidden,
+                     int64_t table_rows, int dtype, void* stream);
 
 /* qkv [rows, (num_heads + 2*num_kv_heads) * head_dim] is the output of the q|k|v projections
  * side by side.  Every q and k head is RMS-normalised (q_weight / k_weight, [head_dim]) and rotated

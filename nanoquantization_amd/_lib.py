@@ -56,6 +56,7 @@ SYMBOLS = {
     # include/nq_engine_ops.h
     "nq_add_rmsnorm": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_float, _int, _vp]),
     "nq_row_ssq": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "nq_embed_row_ssq": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp]),
     "nq_qk_norm_rope_store": (_int, [_vp] * 10 + [_i64] * 7 + [ctypes.c_float, _int, _vp]),
     "nq_paged_attention_workspace_bytes": (_sz, [_i64] * 5),
     "nq_paged_attention_decode": (_int, [_vp] * 6 + [_i64] * 7 + [ctypes.c_float, _int, _vp, _sz, _vp]),

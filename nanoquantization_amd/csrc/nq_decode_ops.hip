@@ -104,14 +104,29 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(uint16_t* __r
 
 // ssq[tile][row] = sum of squares of x[row, 128 tile .. 128 tile + 127]: the statistics an AWQ GEMV with an
 // RMSNorm prologue reads, for a residual stream that no GEMV with a residual epilogue has produced yet.
+// With `ids` the row is gathered from a table first (row ids[r] of `x`, clamped to the table) and copied to x_out:
+// the embedding lookup of a decode step and its statistics in one launch.
 template <typename T>
 __global__ __launch_bounds__(kNormThreads) void row_ssq_kernel(const uint16_t* __restrict__ x, float* __restrict__ ssq,
-                                                              int rows, int hidden) {
+                                                              int rows, int hidden, const int64_t* __restrict__ ids,
+                                                              int64_t table_rows, uint16_t* __restrict__ x_out) {
     __shared__ float s_tile[kNormTiles];
     float v[kNormPasses][8];
-    row_load_ssq<T>(const_cast<uint16_t*>(x), nullptr, (int64_t)blockIdx.x * hidden, hidden, v, s_tile);
+    int64_t src = blockIdx.x;
+    if (ids) {
+        src = ids[blockIdx.x];
+        src = src < 0 ? 0 : (src >= table_rows ? table_rows - 1 : src);
+    }
+    row_load_ssq<T>(const_cast<uint16_t*>(x), nullptr, src * hidden, hidden, v, s_tile);
     const int tiles = (hidden + 127) >> 7;
     if ((int)threadIdx.x < tiles) ssq[(size_t)threadIdx.x * rows + blockIdx.x] = s_tile[threadIdx.x];
+    if (x_out) {
+#pragma unroll
+        for (int p = 0; p < kNormPasses; ++p) {
+            const int i = (p * kNormThreads + threadIdx.x) * 8;
+            if (i < hidden) *reinterpret_cast<u32x4*>(x_out + (int64_t)blockIdx.x * hidden + i) = pack8<T>(v[p]);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -802,8 +817,24 @@ extern "C" int nq_add_rmsnorm(void* residual, const void* delta, const void* wei
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }
 
+static int row_ssq_entry(const char* fn, const void* x, float* ssq, int64_t rows, int64_t hidden, const int64_t* ids,
+                         int64_t table_rows, void* x_out, int dtype, void* stream);
+
 extern "C" int nq_row_ssq(const void* x, float* ssq, int64_t rows, int64_t hidden, int dtype, void* stream) {
-    const char* fn = "nq_row_ssq";
+    return row_ssq_entry("nq_row_ssq", x, ssq, rows, hidden, nullptr, 0, nullptr, dtype, stream);
+}
+
+extern "C" int nq_embed_row_ssq(const int64_t* ids, const void* table, void* x_out, float* ssq, int64_t rows,
+                                int64_t hidden, int64_t table_rows, int dtype, void* stream) {
+    const char* fn = "nq_embed_row_ssq";
+    if (!ids || !x_out) return bad(fn, "null pointer argument");
+    if (!aligned16(x_out)) return bad(fn, "x_out must be 16-byte aligned");
+    if (table_rows <= 0) return bad(fn, "table_rows must be positive");
+    return row_ssq_entry(fn, table, ssq, rows, hidden, ids, table_rows, x_out, dtype, stream);
+}
+
+static int row_ssq_entry(const char* fn, const void* x, float* ssq, int64_t rows, int64_t hidden, const int64_t* ids,
+                         int64_t table_rows, void* x_out, int dtype, void* stream) {
     if (!x || !ssq) return bad(fn, "null pointer argument");
     if (!aligned16(x) || (reinterpret_cast<uintptr_t>(ssq) & 3u)) return bad(fn, "x must be 16-byte, ssq 4-byte aligned");
     if (dtype != AWQ_F16 && dtype != AWQ_BF16) return bad(fn, "dtype must be AWQ_F16 or AWQ_BF16");
@@ -815,9 +846,11 @@ extern "C" int nq_row_ssq(const void* x, float* ssq, int64_t rows, int64_t hidde
     hipStream_t st = (hipStream_t)stream;
     (void)hipGetLastError();
     if (dtype == AWQ_F16)
-        row_ssq_kernel<F16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>((const uint16_t*)x, ssq, (int)rows, (int)hidden);
+        row_ssq_kernel<F16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>((const uint16_t*)x, ssq, (int)rows, (int)hidden,
+                                                                                ids, table_rows, (uint16_t*)x_out);
     else
-        row_ssq_kernel<BF16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>((const uint16_t*)x, ssq, (int)rows, (int)hidden);
+        row_ssq_kernel<BF16><<<dim3((unsigned)rows), dim3(kNormThreads), 0, st>>>((const uint16_t*)x, ssq, (int)rows, (int)hidden,
+                                                                                 ids, table_rows, (uint16_t*)x_out);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? AWQ_OK : hip_fail(fn, e);
 }

@@ -158,13 +158,11 @@ class LLMEngine:
         pos = self.s_pos
         # idle rows read row 0's table but write nothing: slot -1 is skipped by the kernels
         slots, ctx = ops.decode_prepare(pos, self.s_active, self.s_table, bs)
-        x = m.embed_tokens(self.s_ids)                                   # residual stream [B, hidden]
-        delta = None
         nl = len(m.layers)
         if self.norm_fused_ok:
             # five launches per block: the o_proj and down_proj GEMVs add into the residual stream and leave its
             # RMSNorm statistics, the q|k|v and gate|up GEMVs normalise their input on the way in
-            ssq = ops.row_ssq(x)
+            x, ssq = ops.embed_row_ssq(self.s_ids, m.embed_tokens.weight)   # residual stream [B, hidden]
             for li, layer in enumerate(m.layers):
                 attn, lin, mlp = layer.self_attn, self.qkv[li], layer.mlp
                 prefetch_hint(attn.o_proj.qweight, attn.o_proj.qscales)
@@ -183,6 +181,8 @@ class LLMEngine:
                 ops.awq_gemv_add_residual(act, mlp.down_proj.qweight, mlp.down_proj.qscales, mlp.down_proj.qzeros, x, ssq)
             self._finish_step(ops.add_rmsnorm(x, None, m.norm.weight, m.norm.eps))
             return
+        x = m.embed_tokens(self.s_ids)                                   # residual stream [B, hidden]
+        delta = None
         for li, layer in enumerate(m.layers):
             attn = layer.self_attn
             gu = self.gate_up_il[li][:2] if self.swiglu_ok else (self.gate_up[li].qweight, self.gate_up[li].qscales)

@@ -115,6 +115,19 @@ def row_ssq(x: torch.Tensor) -> torch.Tensor:
     return ssq
 
 
+def embed_row_ssq(ids: torch.Tensor, table: torch.Tensor):
+    """ids int64 [rows], table [vocab, hidden] -> (x [rows, hidden] = table[ids], its row_ssq)."""
+    dev = _dev(ids, table)
+    rows, (vocab, hidden) = ids.numel(), table.shape
+    assert ids.dtype == torch.int64
+    x = torch.empty(rows, hidden, dtype=table.dtype, device=dev)
+    ssq = torch.empty((hidden + 127) // 128, rows, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().nq_embed_row_ssq(ids.data_ptr(), table.data_ptr(), x.data_ptr(), ssq.data_ptr(), rows, hidden,
+                                               vocab, _lib.dtype_id(table.dtype), _stream()))
+    return x, ssq
+
+
 def _gemv_ws(dev, M, N, K):
     stream = _stream()
     ws = _lib.workspace(dev, stream, _lib.lib().awq_gemv_workspace_bytes(M, N, K))

@@ -486,3 +486,13 @@ def test_decode_prepare_and_advance():
     ops.decode_advance(nxt, active, out, ids, pos, step)
     ops.decode_advance(nxt, active, out, ids, pos, step)          # step 5 is past the log: nothing is written there
     assert step.item() == 6 and torch.equal(out[4], nxt) and torch.equal(pos, pos0 + 3 * active.long())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_row_ssq(dtype):
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(21)
+    table = torch.randn(1000, 1024, device="cuda", generator=g).to(dtype)
+    ids = torch.randint(0, 1000, (33,), device="cuda", generator=g)
+    x, ssq = ops.embed_row_ssq(ids, table)
+    assert torch.equal(x, table[ids]) and torch.equal(ssq, ops.row_ssq(table[ids].contiguous()))
