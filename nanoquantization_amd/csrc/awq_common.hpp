@@ -135,6 +135,11 @@ __device__ __forceinline__ float mul_round(float a, float b) {
     asm("" : "+v"(p));
     return T::to_f32(T::from_f32(p));
 }
+// The same barrier for any fp32 value about to be rounded to T: the value is an fp32 result first.
+__device__ __forceinline__ float as_f32_result(float v) {
+    asm("" : "+v"(v));
+    return v;
+}
 
 // Sum of squares of one 128-column tile of a row, 8 consecutive values per lane, 16 lanes (an aligned group) per
 // tile: the lane's 8 squares in column order by fused multiply-add, then the lanes by xor 8, 4, 2, 1.  Every

@@ -285,11 +285,7 @@ __device__ __forceinline__ void qkv_rope_store(const float (&out)[8], int m, siz
     const float* cs = qe.cos_sin + pos * 128;
     const f32x4 c0 = *reinterpret_cast<const f32x4*>(cs + i0), c1 = *reinterpret_cast<const f32x4*>(cs + i0 + 4);
     const f32x4 s0 = *reinterpret_cast<const f32x4*>(cs + 64 + i0), s1 = *reinterpret_cast<const f32x4*>(cs + 64 + i0 + 4);
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) ss += a[e] * a[e];
-#pragma unroll
-    for (int o = 8; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
+    const float ss = tile_ssq(a);
     const float r = rsqrtf(ss / 128.f + qe.eps);
     const bool first = dc < 8;
     uint32_t packed[4];
@@ -297,11 +293,12 @@ __device__ __forceinline__ void qkv_rope_store(const float (&out)[8], int m, siz
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const float wf = T::to_f32((uint16_t)((e & 1) ? wraw[e >> 1] >> 16 : wraw[e >> 1] & 0xFFFFu));
-        const float xn = T::to_f32(T::from_f32(T::to_f32(T::from_f32(a[e] * r)) * wf));
+        const float xn = T::to_f32(T::from_f32(mul_round<T>(a[e], r) * wf));
         const float other = __shfl_xor(xn, 8);
         const float cc = e < 4 ? c0[e] : c1[e - 4], sn = e < 4 ? s0[e] : s1[e - 4];
         const float x1 = first ? xn : other, x2 = first ? other : xn;
-        y[e] = first ? __fsub_rn(__fmul_rn(x1, cc), __fmul_rn(x2, sn)) : __fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cc));
+        y[e] = as_f32_result(first ? __fsub_rn(__fmul_rn(x1, cc), __fmul_rn(x2, sn))
+                                   : __fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cc)));
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) packed[i] = T::pack2(y[2 * i], y[2 * i + 1]);

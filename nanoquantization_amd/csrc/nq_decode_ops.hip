@@ -214,8 +214,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
         if (i < half) {
             const float x1 = round_to<T>(round_to<T>(a[p] * r) * w1[p]);
             const float x2 = round_to<T>(round_to<T>(b[p] * r) * w2[p]);
-            const uint16_t y1 = T::from_f32(__fsub_rn(__fmul_rn(x1, cc[p]), __fmul_rn(x2, sn[p])));
-            const uint16_t y2 = T::from_f32(__fadd_rn(__fmul_rn(x1, sn[p]), __fmul_rn(x2, cc[p])));
+            const uint16_t y1 = T::from_f32(as_f32_result(__fsub_rn(__fmul_rn(x1, cc[p]), __fmul_rn(x2, sn[p]))));
+            const uint16_t y2 = T::from_f32(as_f32_result(__fadd_rn(__fmul_rn(x1, sn[p]), __fmul_rn(x2, cc[p]))));
             dst[i] = y1;
             dst[i + half] = y2;
             if (dst2) {
@@ -267,22 +267,25 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_vec_kernel(
     const float* cs = cos_sin + pos * HD;
     const f32x4 c0 = *reinterpret_cast<const f32x4*>(cs + i0), c1 = *reinterpret_cast<const f32x4*>(cs + i0 + 4);
     const f32x4 s0 = *reinterpret_cast<const f32x4*>(cs + HALF + i0), s1 = *reinterpret_cast<const f32x4*>(cs + HALF + i0 + 4);
+    // the summation order and rounding points of the q|k|v GEMV's fused epilogue (head_dim 128: tile_ssq), so that
+    // both routes give the same bits
     float ss = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) ss += a[e] * a[e];
+    for (int e = 0; e < 8; ++e) ss = __builtin_fmaf(a[e], a[e], ss);
 #pragma unroll
     for (int o = LPH / 2; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
     const float r = rsqrtf(ss / (float)HD + eps);
     float xn[8], y[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) xn[e] = round_to<T>(round_to<T>(a[e] * r) * wf[e]);
+    for (int e = 0; e < 8; ++e) xn[e] = round_to<T>(mul_round<T>(a[e], r) * wf[e]);
     const bool first = dc < LPH / 2;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const float other = __shfl_xor(xn[e], LPH / 2);
         const float cc = e < 4 ? c0[e] : c1[e - 4], sn = e < 4 ? s0[e] : s1[e - 4];
         const float x1 = first ? xn[e] : other, x2 = first ? other : xn[e];
-        y[e] = first ? __fsub_rn(__fmul_rn(x1, cc), __fmul_rn(x2, sn)) : __fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cc));
+        y[e] = as_f32_result(first ? __fsub_rn(__fmul_rn(x1, cc), __fmul_rn(x2, sn))
+                                   : __fadd_rn(__fmul_rn(x1, sn), __fmul_rn(x2, cc)));
     }
     if (!live || !(is_q || is_k)) return;
     const u32x4 packed = pack8<T>(y);

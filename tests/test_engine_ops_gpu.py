@@ -96,8 +96,8 @@ def test_qk_norm_rope_store(dtype, nh, nkv, hd):
                                         (40, 5120, 64, 8), (16, 2048, 8, 8)])
 def test_gemv_qkv_rope_store_equals_unfused(dtype, M, K, nh, nkv):
     """Projection + q/k norm + rotary + cache write in one launch against the GEMV followed by the stand-alone
-    kernel: v (a plain copy of the projection) bit for bit; q and k within one rounding step (the per-head sum of
-    squares is added up in another order)."""
+    kernel: bit for bit (same summation order and rounding points), except where the plain projection runs another
+    kernel with another summation order."""
     import nanoquantization_amd as nq
     from nanoquantization_amd.engine import ops
     from nanoquantization_amd.layers.rope import RoPE
@@ -124,11 +124,13 @@ def test_gemv_qkv_rope_store_equals_unfused(dtype, M, K, nh, nkv):
     q2 = ops.qk_norm_rope_store(nq.awq_gemm(x, qw, qs, qz, 8), nqw, nkw, rope.cos_sin_cache, pos, slots, kc2, vc2,
                                 nh, nkv, hd, 1e-6)
     if M > 32 and K * N >= 50 << 20:
-        _close(vc, vc2.float(), dtype, what="v cache")   # the plain projection runs the shared-chunk kernel here: another sum order
+        # the plain projection runs the shared-chunk kernel here: another sum order
+        _close(vc, vc2.float(), dtype, what="v cache")
+        _close(q, q2.float(), dtype, what="q")
+        _close(kc, kc2.float(), dtype, what="k cache")
     else:
         assert torch.equal(vc, vc2), "v is the projection itself"
-    _close(q, q2.float(), dtype, what="q")
-    _close(kc, kc2.float(), dtype, what="k cache")
+        assert torch.equal(q, q2) and torch.equal(kc, kc2)
     assert torch.equal(q, ops.awq_gemv_qkv_rope_store(x, qw, qs, qz, nqw, nkw, rope.cos_sin_cache, pos, slots,
                                                       torch.zeros_like(kc), torch.zeros_like(vc), nh, nkv, 1e-6))
 
