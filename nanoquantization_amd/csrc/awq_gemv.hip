@@ -413,18 +413,24 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
         if (splits == 1 && wk < NQ)
             rv_pre = residual_load(y, m_base + 4 * kb + wk, N, (size_t)wv_col * 8, m_base + 4 * kb + wk < M && col_ok);
     }
+    // rows m_base + 4*kb + r with r >= r_lim exist for no kb: with fewer than 4 rows their slots are neither
+    // written nor summed (a quarter of the LDS traffic at one row)
+    const int r_lim = M - m_base < 4 ? M - m_base : 4;
     if constexpr (WK > 1) {
         float* mine = red + (size_t)wave * (NF * 4 * 64);
 #pragma unroll
         for (int v = 0; v < V; ++v)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
+                if (r < r_lim) {
 #pragma unroll
-                for (int c = 0; c < 8; ++c) mine[((v * 4 + r) * 8 + c) * 64 + lane] = acc[v * 8 + c][r];
+                    for (int c = 0; c < 8; ++c) mine[((v * 4 + r) * 8 + c) * 64 + lane] = acc[v * 8 + c][r];
+                }
         __syncthreads();
     }
     for (int q = wk; q < NQ; q += WK) {
         const int v = q >> 2, r = q & 3;
+        if (r >= r_lim) continue;   // uniform
         const int m = m_base + 4 * kb + r;
         float out[8];
         if constexpr (WK > 1) {
