@@ -152,6 +152,53 @@ class LLMEngine:
         h = ops.add_rmsnorm(last, dlast, m.norm.weight, m.norm.eps)
         return ops.argmax_rows(self.model.lm_head(h))
 
+    @torch.no_grad()
+    def _prefill_ragged(self, prompts: List[List[int]], tables: List[List[int]]) -> torch.Tensor:
+        """Prompts of any lengths in one pass: every per-token operation (norms, AWQ linears, rotary, cache write)
+        runs once over the concatenated tokens, the causal attention once per prompt over its own slice.  Returns the
+        next token of every prompt [len(prompts)]."""
+        m, bs, eps = self.model.model, self.block_size, self.eps
+        dev = self.device
+        lens = [len(p) for p in prompts]
+        starts = [0]
+        for n in lens:
+            starts.append(starts[-1] + n)
+        total = starts[-1]
+        ids = torch.tensor([t for p in prompts for t in p], dtype=torch.long, device=dev)
+        pos_flat = torch.cat([torch.arange(n, device=dev) for n in lens]).contiguous()
+        slot_list = []
+        for n, tbl in zip(lens, tables):
+            t = torch.tensor(tbl[: (n + bs - 1) // bs], device=dev)
+            p = torch.arange(n, device=dev)
+            slot_list.append(t[p // bs] * bs + p % bs)
+        slots = torch.cat(slot_list).contiguous()
+        gqa = self.nh != self.nkv
+        kvw = self.nkv * self.hd
+        x = m.embed_tokens(ids)                                          # residual stream [total, hidden]
+        delta = None
+        for li, layer in enumerate(m.layers):
+            attn = layer.self_attn
+            h = ops.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps)
+            qkv = self.qkv[li](h)
+            q, k = ops.qk_norm_rope_store(qkv, attn.q_norm.weight, attn.k_norm.weight, attn.rope.cos_sin_cache,
+                                          pos_flat, slots, self.cache.k[li], self.cache.v[li], self.nh, self.nkv,
+                                          self.hd, attn.q_norm.eps, dense_k=True)
+            v = qkv[:, -kvw:].view(total, self.nkv, self.hd)
+            o = torch.empty(total, self.nh * self.hd, dtype=self.dtype, device=dev)
+            for a, n in zip(starts, lens):
+                oi = F.scaled_dot_product_attention(q[a:a + n].transpose(0, 1).unsqueeze(0),
+                                                    k[a:a + n].transpose(0, 1).unsqueeze(0),
+                                                    v[a:a + n].transpose(0, 1).unsqueeze(0),
+                                                    is_causal=True, enable_gqa=gqa)
+                o[a:a + n] = oi[0].transpose(0, 1).reshape(n, self.nh * self.hd)
+            h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
+            act = (ops.awq_linear_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
+                   else ops.silu_mul(self.gate_up[li](h)))
+            delta = layer.mlp.down_proj(act)
+        last = torch.tensor([a + n - 1 for a, n in zip(starts, lens)], device=dev)
+        h = ops.add_rmsnorm(x[last].contiguous(), delta[last].contiguous(), m.norm.weight, m.norm.eps)
+        return ops.argmax_rows(self.model.lm_head(h))
+
     # ---- decode: one token per sequence, attention over the paged cache --------------------------
     def _decode_step(self) -> None:
         m, bs, eps = self.model.model, self.block_size, self.eps
@@ -287,11 +334,18 @@ class LLMEngine:
 
     # ---- continuous batching ---------------------------------------------------------------------------
     @torch.no_grad()
-    def serve(self, requests, eos_token_id: Optional[int] = None, stats: Optional[dict] = None) -> List[List[int]]:
+    def serve(self, requests, eos_token_id: Optional[int] = None, stats: Optional[dict] = None,
+              batch_prefill: bool = False, max_prefill_tokens: int = 8192) -> List[List[int]]:
         """requests: sequence of (prompt token ids, max_new_tokens), any lengths.  Returns the greedy continuation
         of each request, in request order (cut after `eos_token_id` if one is given).  Without an end-of-sequence
         token the host reads tokens back only when the output buffer fills up or at the end; with one it reads
-        them after every step."""
+        them after every step.
+
+        By default every admitted request is prefilled on its own, so its tokens do not depend on what else is
+        queued or running (decode rows are independent as well).  `batch_prefill` prefills all requests admitted at
+        the same moment in one pass (up to `max_prefill_tokens` prompt tokens): fewer, larger launches, but the row
+        count of the prefill linears -- and with it their kernel and summation order -- then depends on the
+        company a request arrives in."""
         import time
         from collections import deque
         bs = self.block_size
@@ -307,7 +361,7 @@ class LLMEngine:
         step_log = []                     # per decode step since the last read-back: [(row, request index)]
         self.s_active.zero_(); self.s_pos.zero_(); self.s_ids.zero_(); self.s_table.zero_(); self.s_step.zero_()
         torch.cuda.synchronize()
-        t_start, n_steps, n_prefill = time.perf_counter(), 0, 0
+        t_start, n_steps, n_prefill, n_prefill_calls = time.perf_counter(), 0, 0, 0
 
         def retire(row):
             _, _, blocks = running.pop(row)
@@ -336,34 +390,50 @@ class LLMEngine:
         try:
             while waiting or running:
                 # admit while a row and the blocks for the whole request are free
-                while waiting and free_rows:
+                admitted = []                 # (request index, blocks), prefilled together if batch_prefill
+                tokens_admitted = 0
+                while waiting and len(admitted) < len(free_rows):
                     ri = waiting[0]
                     prompt, max_new = requests[ri]
                     need = (len(prompt) + max_new + bs - 1) // bs
                     if need > len(self.cache.free):
-                        if not running:
+                        if not running and not admitted:
                             raise RuntimeError(f"KV cache too small for request {ri}: {need} blocks wanted, "
                                                f"{len(self.cache.free)} exist free with nothing running")
                         break
+                    if admitted and (not batch_prefill or tokens_admitted + len(prompt) > max_prefill_tokens):
+                        break
                     waiting.popleft()
-                    blocks = self.cache.allocate(need)
+                    admitted.append((ri, self.cache.allocate(need)))
+                    tokens_admitted += len(prompt)
+                if admitted:
                     try:
-                        ids = torch.tensor([prompt], dtype=torch.long, device=self.device)
-                        tok = int(self._prefill(ids, [blocks])[0])
+                        if len(admitted) == 1:
+                            ids = torch.tensor([requests[admitted[0][0]][0]], dtype=torch.long, device=self.device)
+                            toks = self._prefill(ids, [admitted[0][1]]).tolist()
+                        else:
+                            toks = self._prefill_ragged([requests[ri][0] for ri, _ in admitted],
+                                                        [b for _, b in admitted]).tolist()
                     except Exception:
-                        self.cache.release(blocks)
+                        for _, blocks in admitted:
+                            self.cache.release(blocks)
                         raise
-                    n_prefill += 1
-                    out[ri].append(tok)
-                    if max_new == 1 or tok == eos_token_id:
-                        self.cache.release(blocks)
-                        continue
-                    row = free_rows.pop()
-                    running[row] = [ri, max_new - 1, blocks]
-                    self.s_table[row] = torch.tensor(blocks + [0] * (self.max_blocks - need), dtype=torch.int32)
-                    self.s_ids[row] = tok
-                    self.s_pos[row] = len(prompt)
-                    self.s_active[row] = True
+                    n_prefill += len(admitted)
+                    n_prefill_calls += 1
+                    for (ri, blocks), tok in zip(admitted, toks):
+                        prompt, max_new = requests[ri]
+                        out[ri].append(tok)
+                        if max_new == 1 or tok == eos_token_id:
+                            self.cache.release(blocks)
+                            continue
+                        row = free_rows.pop()
+                        running[row] = [ri, max_new - 1, blocks]
+                        self.s_table[row] = torch.tensor(blocks + [0] * (self.max_blocks - len(blocks)), dtype=torch.int32)
+                        self.s_ids[row] = tok
+                        self.s_pos[row] = len(prompt)
+                        self.s_active[row] = True
+                    if waiting and free_rows and len(admitted) > 0 and not batch_prefill:
+                        continue              # one prefill per pass: admit the next request before decoding
                 if not running:
                     continue
                 self._run_decode()
@@ -385,6 +455,6 @@ class LLMEngine:
         if stats is not None:
             torch.cuda.synchronize()
             stats.update(wall_s=time.perf_counter() - t_start, decode_steps=n_steps, prefills=n_prefill,
-                         tokens=sum(len(o) for o in out))
+                         prefill_calls=n_prefill_calls, tokens=sum(len(o) for o in out))
         return out
 

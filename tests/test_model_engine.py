@@ -198,19 +198,29 @@ def test_engine_continuous_batching():
     assert [len(o) for o in got] == budgets
     assert len(eng.cache.free) == total_blocks and st["prefills"] == len(reqs)
     assert st["decode_steps"] < sum(b - 1 for b in budgets), "requests must share decode steps"
-    for (prompt, _), cont in zip(reqs, got):
-        seq = torch.tensor([prompt + cont], device="cuda")
-        pos = torch.arange(seq.shape[1], device="cuda").unsqueeze(0)
-        logits = model.lm_head(model(seq, pos)).float()[0, len(prompt) - 1:-1]
-        chosen = torch.tensor(cont, device="cuda")
-        gap = logits.max(-1).values - logits.gather(-1, chosen.unsqueeze(-1)).squeeze(-1)
-        scale = logits.abs().max().item()
-        assert gap.max().item() <= 2e-2 * scale
-        top2 = logits.topk(2, dim=-1).values
-        clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
-        assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
+    def check_against_recompute(conts):
+        for (prompt, _), cont in zip(reqs, conts):
+            seq = torch.tensor([prompt + cont], device="cuda")
+            pos = torch.arange(seq.shape[1], device="cuda").unsqueeze(0)
+            logits = model.lm_head(model(seq, pos)).float()[0, len(prompt) - 1:-1]
+            chosen = torch.tensor(cont, device="cuda")
+            gap = logits.max(-1).values - logits.gather(-1, chosen.unsqueeze(-1)).squeeze(-1)
+            scale = logits.abs().max().item()
+            assert gap.max().item() <= 2e-2 * scale
+            top2 = logits.topk(2, dim=-1).values
+            clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
+            assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
+
+    check_against_recompute(got)
     # the same requests again (the captured graph and the freed blocks are reused) give the same tokens
     assert eng.serve(reqs) == got
+    # requests admitted together prefilled in one ragged pass: fewer prefill launches, same check
+    stb = {}
+    gotb = eng.serve(reqs, stats=stb, batch_prefill=True)
+    assert [len(o) for o in gotb] == budgets and stb["prefills"] == len(reqs) and stb["prefill_calls"] < len(reqs)
+    check_against_recompute(gotb)
+    assert len(eng.cache.free) == total_blocks
+    assert eng.serve(reqs, batch_prefill=True) == gotb
     # end-of-sequence: pick a token that some request emits mid-way and check the cut
     ri = max(range(len(got)), key=lambda i: len(got[i]))
     eos = got[ri][len(got[ri]) // 2]
