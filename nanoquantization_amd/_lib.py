@@ -104,6 +104,47 @@ def dtype_id(dtype: torch.dtype) -> int:
     raise AwqHipError(f"qscales dtype must be float16 or bfloat16, got {dtype}")
 
 
+# Host-side shortcuts for the launch path (a decode-size launch takes ~5 us on the GPU; the wrappers around it
+# should not take three times that).
+class _NoContext:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_CONTEXT = _NoContext()
+
+
+def on_device(device: torch.device):
+    """Context manager that makes `device` current; free when it already is."""
+    idx = device.index
+    if idx is None or idx == torch._C._cuda_getDevice():
+        return _NO_CONTEXT
+    return torch.cuda.device(device)
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    """The raw hipStream_t of torch's current stream on `device`."""
+    idx = device.index
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice() if idx is None else idx)
+
+
+_ws_bytes_cache: dict[tuple, int] = {}
+
+
+def workspace_bytes(entry: str, M: int, N: int, K: int, extra: tuple = ()) -> int:
+    """`<entry>_workspace_bytes(M, N, K, *extra)` of the library, remembered per shape."""
+    key = (entry, M, N, K, extra)
+    n = _ws_bytes_cache.get(key)
+    if n is None:
+        n = getattr(lib(), entry + "_workspace_bytes")(M, N, K, *extra)
+        if len(_ws_bytes_cache) < 65536:
+            _ws_bytes_cache[key] = n
+    return n
+
+
 # One zero-initialised split-K workspace per (device, stream).  The kernels leave
 # it zeroed, and calls on one stream are ordered, so it is shared by every layer.
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}

@@ -23,8 +23,8 @@ def _dev(*ts: torch.Tensor) -> torch.device:
     return dev
 
 
-def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+def _stream(dev: torch.device) -> int:
+    return _lib.current_stream_ptr(dev)
 
 
 def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float) -> torch.Tensor:
@@ -34,10 +34,10 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     assert weight.shape == (hidden,) and weight.dtype == residual.dtype
     assert delta is None or (delta.shape == residual.shape and delta.dtype == residual.dtype)
     y = torch.empty_like(residual)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().nq_add_rmsnorm(residual.data_ptr(), None if delta is None else delta.data_ptr(),
                                              weight.data_ptr(), y.data_ptr(), rows, hidden, eps,
-                                             _lib.dtype_id(residual.dtype), _stream()))
+                                             _lib.dtype_id(residual.dtype), _stream(dev)))
     return y
 
 
@@ -60,12 +60,12 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torc
     num_slots = k_cache.numel() // (num_kv_heads * head_dim)
     q = torch.empty(rows, num_heads, head_dim, dtype=qkv.dtype, device=dev)
     k = torch.empty(rows, num_kv_heads, head_dim, dtype=qkv.dtype, device=dev) if dense_k else None
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().nq_qk_norm_rope_store(
             qkv.data_ptr(), q_weight.data_ptr(), k_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(),
             slots.data_ptr(), q.data_ptr(), None if k is None else k.data_ptr(), k_cache.data_ptr(),
             v_cache.data_ptr(), rows, num_heads, num_kv_heads,
-            head_dim, cos_sin.numel() // head_dim, num_slots, block_size, eps, _lib.dtype_id(qkv.dtype), _stream()))
+            head_dim, cos_sin.numel() // head_dim, num_slots, block_size, eps, _lib.dtype_id(qkv.dtype), _stream(dev)))
     return (q, k) if dense_k else q
 
 
@@ -91,8 +91,8 @@ def awq_gemv_qkv_rope_store(x: torch.Tensor, qweight: torch.Tensor, qscales: tor
     num_slots = k_cache.numel() // (num_kv_heads * hd)
     q = torch.empty(M, num_heads, hd, dtype=x.dtype, device=dev)
     L = _lib.lib()
-    with torch.cuda.device(dev):
-        stream = _stream()
+    with _lib.on_device(dev):
+        stream = _stream(dev)
         nbytes = L.awq_gemv_workspace_bytes(M, N, K)
         ws = _lib.workspace(dev, stream, nbytes)
         _lib.check(L.awq_gemv_qkv_rope_store(
@@ -110,8 +110,8 @@ def row_ssq(x: torch.Tensor) -> torch.Tensor:
     dev = _dev(x)
     rows, hidden = x.shape
     ssq = torch.empty((hidden + 127) // 128, rows, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        _lib.check(_lib.lib().nq_row_ssq(x.data_ptr(), ssq.data_ptr(), rows, hidden, _lib.dtype_id(x.dtype), _stream()))
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().nq_row_ssq(x.data_ptr(), ssq.data_ptr(), rows, hidden, _lib.dtype_id(x.dtype), _stream(dev)))
     return ssq
 
 
@@ -122,14 +122,14 @@ def embed_row_ssq(ids: torch.Tensor, table: torch.Tensor):
     assert ids.dtype == torch.int64
     x = torch.empty(rows, hidden, dtype=table.dtype, device=dev)
     ssq = torch.empty((hidden + 127) // 128, rows, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().nq_embed_row_ssq(ids.data_ptr(), table.data_ptr(), x.data_ptr(), ssq.data_ptr(), rows, hidden,
-                                               vocab, _lib.dtype_id(table.dtype), _stream()))
+                                               vocab, _lib.dtype_id(table.dtype), _stream(dev)))
     return x, ssq
 
 
 def _gemv_ws(dev, M, N, K):
-    stream = _stream()
+    stream = _stream(dev)
     ws = _lib.workspace(dev, stream, _lib.lib().awq_gemv_workspace_bytes(M, N, K))
     return (None if ws is None else ws.data_ptr()), (0 if ws is None else ws.numel()), stream
 
@@ -145,7 +145,7 @@ def awq_gemv_add_residual(x: torch.Tensor, qweight: torch.Tensor, qscales: torch
     assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
     assert residual.shape == (M, N) and residual.dtype == x.dtype
     assert ssq.shape == (N // 128, M) and ssq.dtype == torch.float32 and N % 128 == 0
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         ws, ws_bytes, stream = _gemv_ws(dev, M, N, K)
         _lib.check(_lib.lib().awq_gemv_add_residual(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(),
                                                     qzeros.data_ptr(), residual.data_ptr(), ssq.data_ptr(), M, N, K, g,
@@ -164,7 +164,7 @@ def awq_gemv_rmsnorm(x: torch.Tensor, ssq: torch.Tensor, norm_weight: torch.Tens
     assert K % 128 == 0 and ssq.shape == (K // 128, M) and ssq.dtype == torch.float32
     assert norm_weight.shape == (K,) and norm_weight.dtype == x.dtype
     out = torch.empty(M, N // 2 if gated else N, dtype=x.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         ws, ws_bytes, stream = _gemv_ws(dev, M, N, K)
         _lib.check(_lib.lib().awq_gemv_rmsnorm(x.data_ptr(), ssq.data_ptr(), norm_weight.data_ptr(), eps,
                                                qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(), out.data_ptr(),
@@ -196,7 +196,7 @@ def awq_gemv_rmsnorm_qkv_rope_store(x: torch.Tensor, ssq: torch.Tensor, norm_wei
     block_size = k_cache.shape[2]
     num_slots = k_cache.numel() // (num_kv_heads * hd)
     q = torch.empty(M, num_heads, hd, dtype=x.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         ws, ws_bytes, stream = _gemv_ws(dev, M, N, K)
         _lib.check(_lib.lib().awq_gemv_rmsnorm_qkv_rope_store(
             x.data_ptr(), ssq.data_ptr(), norm_weight.data_ptr(), norm_eps, qweight.data_ptr(), qscales.data_ptr(),
@@ -219,13 +219,13 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     max_blocks = block_table.shape[1]
     out = torch.empty(batch, nh * hd, dtype=q.dtype, device=dev)
     L = _lib.lib()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         nbytes = L.nq_paged_attention_workspace_bytes(batch, nh, nkv, hd, block_size * max_blocks)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
         _lib.check(L.nq_paged_attention_decode(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), context_lens.data_ptr(),
             out.data_ptr(), batch, nh, nkv, hd, block_size, max_blocks, num_blocks, scale, _lib.dtype_id(q.dtype),
-            None if ws is None else ws.data_ptr(), nbytes, _stream()))
+            None if ws is None else ws.data_ptr(), nbytes, _stream(dev)))
     return out
 
 
@@ -238,8 +238,8 @@ def silu_mul(gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
     assert two == 2 * inter and gate_up.is_contiguous()
     out = torch.empty(rows, inter, dtype=gate_up.dtype, device=dev)
     fn = _lib.lib().nq_silu_mul_interleaved if interleaved else _lib.lib().nq_silu_mul
-    with torch.cuda.device(dev):
-        _lib.check(fn(gate_up.data_ptr(), out.data_ptr(), rows, inter, _lib.dtype_id(gate_up.dtype), _stream()))
+    with _lib.on_device(dev):
+        _lib.check(fn(gate_up.data_ptr(), out.data_ptr(), rows, inter, _lib.dtype_id(gate_up.dtype), _stream(dev)))
     return out
 
 
@@ -249,9 +249,9 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     rows, vocab = logits.shape
     assert logits.is_contiguous()
     out = torch.empty(rows, dtype=torch.int64, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().nq_argmax_rows(logits.data_ptr(), out.data_ptr(), rows, vocab,
-                                             _lib.dtype_id(logits.dtype), _stream()))
+                                             _lib.dtype_id(logits.dtype), _stream(dev)))
     return out
 
 
@@ -264,10 +264,10 @@ def decode_prepare(positions: torch.Tensor, active: torch.Tensor, block_table: t
     assert active.numel() == rows and block_table.dim() == 2 and block_table.shape[0] == rows
     slots = torch.empty(rows, dtype=torch.int64, device=dev)
     ctx = torch.empty(rows, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().nq_decode_prepare(positions.data_ptr(), active.data_ptr(), block_table.data_ptr(),
                                                 slots.data_ptr(), ctx.data_ptr(), rows, block_table.shape[1], block_size,
-                                                _stream()))
+                                                _stream(dev)))
     return slots, ctx
 
 
@@ -279,10 +279,10 @@ def decode_advance(next_tokens: torch.Tensor, active: torch.Tensor, out_log: tor
     assert all(t.dtype == torch.int64 for t in (next_tokens, out_log, ids, positions, step)) and active.dtype == torch.bool
     assert out_log.dim() == 2 and out_log.shape[1] == rows and ids.numel() == rows and positions.numel() == rows
     assert active.numel() == rows and step.numel() == 1
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().nq_decode_advance(next_tokens.data_ptr(), active.data_ptr(), out_log.data_ptr(),
                                                 ids.data_ptr(), positions.data_ptr(), step.data_ptr(), rows,
-                                                out_log.shape[0], _stream()))
+                                                out_log.shape[0], _stream(dev)))
 
 
 def interleave_gate_up(gate, up):
@@ -311,8 +311,8 @@ def awq_linear_swiglu(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Ten
         return silu_mul(_gemm._linear("awq_linear", x, qweight, qscales, qzeros, None), interleaved=True)
     out = torch.empty(M, N // 2, dtype=x.dtype, device=dev)
     L = _lib.lib()
-    with torch.cuda.device(dev):
-        stream = _stream()
+    with _lib.on_device(dev):
+        stream = _stream(dev)
         nbytes = L.awq_linear_swiglu_workspace_bytes(M, N, K)
         ws = _lib.workspace(dev, stream, nbytes)
         _lib.check(L.awq_linear_swiglu(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(),
@@ -330,8 +330,8 @@ def awq_gemv_swiglu(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tenso
     assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
     out = torch.empty(M, N // 2, dtype=x.dtype, device=dev)
     L = _lib.lib()
-    with torch.cuda.device(dev):
-        stream = _stream()
+    with _lib.on_device(dev):
+        stream = _stream(dev)
         nbytes = L.awq_gemv_workspace_bytes(M, N, K)
         ws = _lib.workspace(dev, stream, nbytes)
         _lib.check(L.awq_gemv_swiglu(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(),

@@ -62,8 +62,8 @@ def awq_dequantize(
     dev = _require_device(qweight, qscales, qzeros)
     qweight, qscales, qzeros = qweight.contiguous(), qscales.contiguous(), qzeros.contiguous()
     out = torch.empty(K, N, dtype=qscales.dtype, device=dev)
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _lib.on_device(dev):
+        stream = _lib.current_stream_ptr(dev)
         _lib.check(_lib.lib().awq_dequantize(_ptr(qweight), _ptr(qscales), _ptr(qzeros), _ptr(out),
                                              K, N, g, _lib.dtype_id(qscales.dtype), stream))
     return out
@@ -82,8 +82,8 @@ def awq_dequantize_transposed(qweight: torch.Tensor, qscales: torch.Tensor, qzer
     dev = _require_device(qweight, qscales, qzeros)
     qweight, qscales, qzeros = qweight.contiguous(), qscales.contiguous(), qzeros.contiguous()
     out = torch.empty(N, K, dtype=qscales.dtype, device=dev)
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _lib.on_device(dev):
+        stream = _lib.current_stream_ptr(dev)
         _lib.check(_lib.lib().awq_dequantize_transposed(_ptr(qweight), _ptr(qscales), _ptr(qzeros), _ptr(out),
                                                         K, N, g, _lib.dtype_id(qscales.dtype), stream))
     return out
@@ -101,8 +101,9 @@ def _linear(entry: str, x, qweight, qscales, qzeros, bias, extra=()):
     dt = qscales.dtype
     if x.dtype != dt:  # the reference casts x to the output dtype on load (layers/gemm.py:259)
         x = x.to(dt)
-    x, qweight, qscales, qzeros = x.contiguous(), qweight.contiguous(), qscales.contiguous(), qzeros.contiguous()
-    if bias is not None:
+    if not (x.is_contiguous() and qweight.is_contiguous() and qscales.is_contiguous() and qzeros.is_contiguous()):
+        x, qweight, qscales, qzeros = x.contiguous(), qweight.contiguous(), qscales.contiguous(), qzeros.contiguous()
+    if bias is not None and (bias.dtype != dt or bias.device != dev or not bias.is_contiguous()):
         bias = bias.to(device=dev, dtype=dt).contiguous()
     if entry == "awq_linear" and _two_pass_ok(M, K, g):
         wt = awq_dequantize_transposed(qweight, qscales, qzeros)
@@ -114,16 +115,15 @@ def _linear(entry: str, x, qweight, qscales, qzeros, bias, extra=()):
     if M == 0:
         return out
     L = _lib.lib()
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream().cuda_stream
-        if extra:
-            nbytes = getattr(L, entry + "_workspace_bytes")(M, N, K, *extra)
-        else:
-            nbytes = getattr(L, entry + "_workspace_bytes")(M, N, K)
-        ws = _lib.workspace(dev, stream, nbytes)
-        _lib.check(getattr(L, entry)(_ptr(x), _ptr(qweight), _ptr(qscales), _ptr(qzeros), _ptr(bias),
-                                     _ptr(out), M, N, K, g, _lib.dtype_id(dt), _ptr(ws),
-                                     0 if ws is None else ws.numel(), stream, *extra))
+    with _lib.on_device(dev):
+        stream = _lib.current_stream_ptr(dev)
+        nbytes = _lib.workspace_bytes(entry, M, N, K, tuple(extra))
+        ws = _lib.workspace(dev, stream, nbytes) if nbytes else None
+        status = getattr(L, entry)(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(), _ptr(bias),
+                                   out.data_ptr(), M, N, K, g, _lib.dtype_id(dt), _ptr(ws),
+                                   0 if ws is None else ws.numel(), stream, *extra)
+        if status:
+            _lib.check(status)
     return out
 
 
@@ -257,13 +257,17 @@ class WQLinear_GEMM(nn.Module):
         awq_linear.qzeros = pack_awq(zeros.to(torch.int32))
         return awq_linear
 
-    @torch.no_grad()
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        # One regime switch inside the library: split-K GEMV for <= 16 tokens, fused dequant + MFMA GEMM above; the
+        # bias is added in the kernel epilogue.  The output is a fresh tensor outside autograd, as under the
+        # reference's @torch.no_grad (layers/gemm.py:552); buffers are fetched from the module's dictionary directly
+        # (nn.Module.__getattr__ costs more than the rest of this function).
+        buf = self._buffers
+        bias = buf["bias"] if "bias" in buf else self.bias
+        if x.dim() == 2:
+            return _linear("awq_linear", x, buf["qweight"], buf["qscales"], buf["qzeros"], bias)
         out_shape = x.shape[:-1] + (self.out_features,)
-        x2 = x.reshape(-1, x.shape[-1])
-        # one regime switch inside the library: split-K GEMV for <= 16 tokens,
-        # fused dequant + MFMA GEMM above; the bias is added in the kernel epilogue
-        out = _linear("awq_linear", x2, self.qweight, self.qscales, self.qzeros, self.bias)
+        out = _linear("awq_linear", x.reshape(-1, x.shape[-1]), buf["qweight"], buf["qscales"], buf["qzeros"], bias)
         return out.reshape(out_shape)
 
     def extra_repr(self) -> str:
