@@ -172,7 +172,8 @@ int awq_gemm(const void* x, const int32_t* qweight, const void* qscales, const i
 
 /* The whole forward of one AWQ linear: picks the regime from M (awq_gemv for
  * M <= 16, and up to 64 where it takes the shape, awq_gemm above) and applies the bias.
- * Replaces WQLinear_GEMM.forward, nanoquantization/layers/gemm.py:552-567
+ * A K that is a multiple of 32 but not of 64 (which awq_gemm does not take) is served by
+ * awq_gemv in blocks of 16 rows.  Replaces WQLinear_GEMM.forward, nanoquantization/layers/gemm.py:552-567
  * (the reshape of x/y to 2-D stays with the caller). */
 int awq_linear(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
                const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,

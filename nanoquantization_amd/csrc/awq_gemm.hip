@@ -422,8 +422,12 @@ extern "C" int awq_gemm(const void* x, const int32_t* qweight, const void* qscal
 
 extern "C" size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     // the regime depends on the group size, which this query does not get: cover both
-    const size_t a = M <= 64 ? awq_gemv_workspace_bytes(M, N, K) : 0;
+    size_t a = M <= 64 ? awq_gemv_workspace_bytes(M, N, K) : 0;
     const size_t b = M > 16 ? awq_gemm_workspace_bytes(M, N, K) : 0;
+    if (M > 16 && K % awq::kBK != 0) {   // served by the GEMV in blocks of 16 rows
+        const size_t c = awq_gemv_workspace_bytes(16, N, K);
+        a = a > c ? a : c;
+    }
     return a > b ? a : b;
 }
 
@@ -459,6 +463,21 @@ extern "C" int awq_linear(const void* x, const int32_t* qweight, const void* qsc
     if (M >= 1 && ((M <= 16 && group_size % 32 == 0) || (M <= 64 && staged)))
         return awq_gemv(x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, workspace,
                         workspace_bytes, stream);
+    if (M > 16 && K % awq::kBK != 0 && K % 32 == 0 && group_size > 0 && group_size % 32 == 0 && K % group_size == 0 &&
+        N > 0 && x && y) {
+        // a K the MFMA GEMM's 64-row steps do not divide (the reference takes any multiple of 32,
+        // layers/gemm.py:268): the GEMV, 16 rows at a time -- no real model has such a width, so only
+        // the result matters here
+        const size_t esz = 2;
+        for (int64_t m0 = 0; m0 < M; m0 += 16) {
+            const int64_t rows = M - m0 < 16 ? M - m0 : 16;
+            const int rc = awq_gemv(static_cast<const char*>(x) + (size_t)m0 * K * esz, qweight, qscales, qzeros, bias,
+                                    static_cast<char*>(y) + (size_t)m0 * N * esz, rows, N, K, group_size, dtype,
+                                    workspace, workspace_bytes, stream);
+            if (rc != AWQ_OK) return rc;
+        }
+        return AWQ_OK;
+    }
     return awq_gemm(x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, workspace,
                     workspace_bytes, stream);
 }

@@ -188,3 +188,19 @@ def test_gemm_largest_shapes_properties(M, K, N):
     assert err <= TIGHT["bf16"], err
     sub = nq.awq_gemm(x[rows].contiguous(), qw, sc, qz, 8).float()          # another kernel / tile shape
     assert ((sub - ref).abs().max() / ref.abs().max()).item() <= TIGHT["bf16"]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,K,N,g", [(48, 288, 512, 32), (200, 224, 384, 32), (65, 544, 1280, 32), (32, 32, 256, 32)])
+def test_linear_k_not_a_multiple_of_64(dtype, M, K, N, g):
+    """K = 32 * odd (the reference admits any multiple of its 32-row K block) above 16 rows: awq_linear serves it
+    with the GEMV, 16 rows at a time."""
+    from nanoquantization_amd.layers import gemm as gemm_layer
+    print(f"linear K%64!=0 M={M} K={K} N={N} g={g} {dtype}", flush=True)
+    p = make_case(K, N, g, dtype, seed=M + K)
+    xb = make_x(M, K, dtype, seed=M)
+    bias = np.random.default_rng(M).standard_normal(N).astype(np.float32)
+    bias_bits = o.to_bits16(bias, dtype)
+    y = gemm_layer._linear("awq_linear", to_dev(xb, dtype), to_dev(p["qweight"]), to_dev(p["qscales"], dtype),
+                           to_dev(p["qzeros"]), to_dev(bias_bits, dtype))
+    _check(y, xb, p, dtype, o.from_bits16(bias_bits, dtype))
