@@ -780,9 +780,12 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
         const int slot = h * 16 + dsl;
         wsrc[h] = (uint32_t)((slot & 3) * 8 + (slot >> 2)) * (uint32_t)words + (uint32_t)(tile * 16 + dq * 4);
     }
-    // x: one DMA instruction per step; lane = m * 4 + k-block
-    const bool x_lane = (lane >> 2) < M;
-    const uint32_t xsrc = (uint32_t)(x_lane ? lane >> 2 : 0) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
+    // x: up to 4 rows in one DMA instruction per chunk, lane = m * 16 + (step * 4 + k-block), LDS layout
+    // [m][step][k-block]; more rows in one instruction per step, lane = m * 4 + k-block, layout [step][m][k-block]
+    const bool x_few = M <= 4;
+    const bool x_lane = x_few ? (lane >> 4) < M : (lane >> 2) < M;
+    const uint32_t xsrc = x_few ? (uint32_t)(x_lane ? lane >> 4 : 0) * (uint32_t)K + (uint32_t)(lane & 15) * 8u
+                                : (uint32_t)(x_lane ? lane >> 2 : 0) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
     const bool zs_lane = lane < 16;
     const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
 
@@ -798,10 +801,14 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
                                                  16, 0, 0);
         }
         if (x_lane) {
+            if (x_few) {
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + row0 + xsrc), AWQ_LPTR(stage + x_off), 16, 0, 0);
+            } else {
 #pragma unroll
-            for (int s = 0; s < CH; ++s)
-                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc),
-                                                 AWQ_LPTR(stage + x_off + s * 64 * M), 16, 0, 0);
+                for (int s = 0; s < CH; ++s)
+                    __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc),
+                                                     AWQ_LPTR(stage + x_off + s * 64 * M), 16, 0, 0);
+            }
         }
         if (zs_lane) {
             const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
@@ -814,7 +821,8 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
 
     // compute-lane read offsets inside the staging buffer (bytes)
     const uint32_t* w_rd = reinterpret_cast<const uint32_t*>(stage + (kb * 16 + j) * 4);   // + (s*512 + r*64) words
-    const int x_rd_off = x_off + (min(j, M - 1) * 4 + kb) * 16;                            // + s * 64 * M
+    const int x_rd_off = x_off + (x_few ? min(j, M - 1) * 16 + kb : min(j, M - 1) * 4 + kb) * 16;   // + s * x_rd_step
+    const int x_rd_step = x_few ? 64 : 64 * M;
     const int z_rd_off = zs_off + j * 4;
     const int s_rd_off = zs_off + 64 + j * 16;
 
@@ -853,7 +861,7 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
         for (int s = 0; s < CH; ++s) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) d.w[s][r] = w_rd[s * 512 + r * 64];
-            d.xa[s][0] = *reinterpret_cast<const u32x4*>(stage + x_rd_off + s * 64 * M);
+            d.xa[s][0] = *reinterpret_cast<const u32x4*>(stage + x_rd_off + s * x_rd_step);
         }
         d.zw = *reinterpret_cast<const uint32_t*>(stage + z_rd_off);
         d.sv[0] = *reinterpret_cast<const u32x4*>(stage + s_rd_off);
