@@ -387,6 +387,16 @@ extern "C" const char* awq_gemm_variant_name(int variant) {
     return (variant >= 0 && variant < awq::kNumGemmVariants) ? awq::kGemmVariants[variant].name : "";
 }
 
+extern "C" int awq_gemm_plan(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
+    if (!variant || !split_k || M < 1 || N < 8 || N % 8 != 0 || K < awq::kBK || K % awq::kBK != 0) {
+        awq::set_error("awq_gemm_plan: not a shape awq_gemm takes (M=%lld N=%lld K=%lld)", (long long)M, (long long)N,
+                       (long long)K);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    awq::pick_gemm(M, N, K, variant, split_k);
+    return AWQ_OK;
+}
+
 extern "C" size_t awq_gemm_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant,
                                               int split_k) {
     if (variant < 0 || variant >= awq::kNumGemmVariants || split_k < 1 || K < awq::kBK || N < 8 || M < 1)

@@ -1484,6 +1484,21 @@ extern "C" const char* awq_gemv_variant_name(int variant) {
     return (variant >= 0 && variant < awq::kNumGemvVariants) ? awq::kGemvVariants[variant].name : "";
 }
 
+extern "C" int awq_gemv_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, int* variant, int* split_k) {
+    if (!variant || !split_k || M < 1 || M > 64 || N < 8 || N % 8 != 0 || K < 32 || group_size < 32 ||
+        group_size % 32 != 0 || K % group_size != 0) {
+        awq::set_error("awq_gemv_plan: not a shape awq_gemv takes (M=%lld N=%lld K=%lld g=%lld)", (long long)M,
+                       (long long)N, (long long)K, (long long)group_size);
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    awq::pick_gemv(M, N, K, group_size, variant, split_k);
+    if (M > 16 && *variant < awq::kFirstDmaVariant) {
+        awq::set_error("awq_gemv_plan: rows 17..64 need the staged path (N %% 128 == 0, group_size %% 128 == 0)");
+        return AWQ_ERR_UNSUPPORTED;
+    }
+    return AWQ_OK;
+}
+
 extern "C" size_t awq_gemv_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant,
                                               int split_k) {
     if (variant < 0 || variant >= awq::kNumGemvVariants || split_k < 1 || K < 32 || N < 8 || M < 1) return 0;

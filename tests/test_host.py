@@ -131,3 +131,63 @@ def test_product_does_not_import_oracle():
             if f.endswith((".py", ".hip", ".hpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+def _plan(fn, *args):
+    v, s = ctypes.c_int(-1), ctypes.c_int(-1)
+    rc = fn(*args, ctypes.byref(v), ctypes.byref(s))
+    return rc, v.value, s.value
+
+
+def test_dispatch_plans_are_consistent():
+    """Host-only: for a sweep of shapes, the variant and K split the library would pick are valid for the shape, fit
+    the workspace it asks for, and follow the documented rules (no device call is made)."""
+    _ensure_built()
+    L = _lib.lib()
+    gemv_names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
+    gemm_names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
+    shapes = [(1024, 2048), (1024, 1024), (2048, 1024), (1024, 3072), (3072, 1024), (4096, 12288), (12288, 4096),
+              (5120, 25600), (25600, 5120), (5120, 10240), (8192, 5120), (5120, 34816), (4096, 24576), (128, 128),
+              (256, 8), (1024, 1032), (3072, 136)]
+    for K, N in shapes:
+        for M in (1, 2, 4, 5, 8, 16, 17, 32, 33, 48, 64):
+            for g in (128, 32):
+                rc, v, s = _plan(L.awq_gemv_plan, M, N, K, g)
+                staged_ok = N % 128 == 0 and g % 128 == 0
+                if M > 16 and not staged_ok:
+                    assert rc != 0, (M, N, K, g)
+                    continue
+                assert rc == 0 and 0 <= v < len(gemv_names) and s >= 1, (M, N, K, g, rc, v, s)
+                name = gemv_names[v]
+                chunks = max(K // 128, 1)
+                assert s <= chunks, (name, s, chunks)
+                if name.startswith(("dma", "wide")):
+                    assert staged_ok
+                else:
+                    assert M <= 16
+                if name.startswith("wide"):
+                    assert M > 16 and N % 512 == 0 and K * N >= 50 << 20
+                    assert N // 512 * s <= 256 + N // 512            # about one workgroup per CU
+                if not staged_ok:
+                    assert not name.startswith(("dma", "wide"))
+                if g == 128:   # awq_gemv_workspace_bytes takes no group size: it must cover this plan
+                    assert L.awq_gemv_ex_workspace_bytes(M, N, K, v, s) <= L.awq_gemv_workspace_bytes(M, N, K)
+                    assert L.awq_gemv_workspace_bytes(M, N, K) <= L.awq_linear_workspace_bytes(M, N, K)
+        for M in (17, 64, 65, 128, 129, 512, 1000, 2048, 8192):
+            if K % 64:
+                continue
+            rc, v, s = _plan(L.awq_gemm_plan, M, N, K)
+            assert rc == 0 and 0 <= v < len(gemm_names) and 1 <= s <= 16, (M, N, K, rc, v, s)
+            assert s <= max(K // 64 // 8, 1)                         # at least 8 K steps per split
+            assert (gemm_names[v].startswith("256x256")) == (M > 128)
+            assert L.awq_gemm_ex_workspace_bytes(M, N, K, v, s) == L.awq_gemm_workspace_bytes(M, N, K)
+            assert L.awq_gemm_workspace_bytes(M, N, K) <= L.awq_linear_workspace_bytes(M, N, K)
+    # the whole-rounds rule for 5..64 rows: 272 column tiles are cut so that the workgroups fill the 256 CUs evenly
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 5120, 128)
+    assert rc == 0 and gemv_names[v] == "dma1x4" and s >= 3
+    wgs = 34816 // 128 * s
+    assert wgs / (256 * -(-wgs // 256)) >= 0.8
+    # shapes awq_gemv does not take are refused by the plan as well
+    assert _plan(L.awq_gemv_plan, 65, 1024, 1024, 128)[0] != 0
+    assert _plan(L.awq_gemv_plan, 4, 1024, 1000, 128)[0] != 0
+    assert _plan(L.awq_gemm_plan, 64, 1024, 96)[0] != 0
