@@ -191,3 +191,30 @@ def test_dispatch_plans_are_consistent():
     assert _plan(L.awq_gemv_plan, 65, 1024, 1024, 128)[0] != 0
     assert _plan(L.awq_gemv_plan, 4, 1024, 1000, 128)[0] != 0
     assert _plan(L.awq_gemm_plan, 64, 1024, 96)[0] != 0
+
+
+def test_every_entry_point_validates_before_touching_a_device():
+    """Called with null pointers, every status-returning entry point reports an error (and says which function) without
+    any device call: this runs on a machine with no GPU."""
+    _ensure_built()
+    L = _lib.lib()
+    checked = 0
+    for name, (res, args) in _lib.SYMBOLS.items():
+        if res is not ctypes.c_int or not args or name == "awq_prefetch_hint":   # NULL clears the pending hints
+            continue
+        vals = []
+        for a in args:
+            if a is ctypes.c_float:
+                vals.append(1e-6)
+            elif a in (ctypes.c_int64, ctypes.c_size_t):
+                vals.append(128)
+            elif a is ctypes.c_int:
+                vals.append(0)
+            else:
+                vals.append(None)
+        rc = getattr(L, name)(*vals)
+        msg = L.awq_hip_last_error().decode()
+        assert rc != 0 and msg.split(":")[0] in (name, "awq_gemm", "awq_gemv"), (name, rc, msg)
+        checked += 1
+    assert checked >= 25
+    assert L.awq_prefetch_hint(None, 0) == 0
