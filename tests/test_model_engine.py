@@ -254,3 +254,19 @@ def test_engine_norm_fused_decode_equals_separate_kernels():
         reqs = [(p[: 5 + 3 * i], 6 + i) for i, p in enumerate(prompts)]
         outs.append((eng.generate(prompts, 20), eng.serve(reqs)))
     assert outs[0] == outs[1]
+
+
+def test_paged_kv_cache_block_bookkeeping():
+    """Host logic of the cache: blocks are handed out once, come back on release, exhaustion raises (CPU)."""
+    from nanoquantization_amd.engine.llm_engine import PagedKVCache
+    c = PagedKVCache(num_layers=2, num_blocks=6, block_size=4, num_kv_heads=2, head_dim=8, dtype=torch.bfloat16,
+                     device=torch.device("cpu"))
+    assert c.k.shape == (2, 6, 2, 4, 8) and c.v.shape == c.k.shape
+    a = c.allocate(4)
+    b = c.allocate(2)
+    assert sorted(a + b) == list(range(6)) and len(c.free) == 0
+    with pytest.raises(RuntimeError, match="KV cache exhausted"):
+        c.allocate(1)
+    c.release(a)
+    assert sorted(c.free) == sorted(a)
+    assert sorted(c.allocate(3) + c.free) == sorted(a)
