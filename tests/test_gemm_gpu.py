@@ -204,3 +204,36 @@ def test_linear_k_not_a_multiple_of_64(dtype, M, K, N, g):
     y = gemm_layer._linear("awq_linear", to_dev(xb, dtype), to_dev(p["qweight"]), to_dev(p["qscales"], dtype),
                            to_dev(p["qzeros"]), to_dev(bias_bits, dtype))
     _check(y, xb, p, dtype, o.from_bits16(bias_bits, dtype))
+
+
+def test_linear_random_shapes_default_dispatch():
+    """Seeded sweep over odd shape combinations (row counts either side of every dispatch boundary, K = group x small
+    and large factors, N with and without whole 128-column tiles, three group sizes, optional bias): whatever kernel
+    the default dispatch picks must meet the tight error bound and be bit-stable run to run."""
+    import random
+    from nanoquantization_amd.layers import gemm as gemm_layer
+    rnd = random.Random(1234)
+    cases = 0
+    while cases < 60:
+        tdt = rnd.choice([torch.float16, torch.bfloat16])
+        g = rnd.choice([128, 128, 128, 64, 32])
+        K = g * rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 16, 17, 24, 31, 32, 40, 48, 64, 100])
+        N = 8 * rnd.choice([1, 3, 16, 17, 32, 48, 64, 96, 128, 136, 160, 256, 272, 384, 512, 640, 1000, 1024, 1280])
+        M = rnd.choice([1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 24, 31, 32, 33, 48, 63, 64, 65, 100, 128, 129, 200, 256, 300, 1024, 1100])
+        if K % 32 or K * N * max(M, 64) > 2e10:
+            continue
+        cases += 1
+        gen = torch.Generator(device="cuda").manual_seed(cases)
+        qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+        qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+        qs = (torch.rand(K // g, N, device="cuda", generator=gen) * 0.02 + 0.001).to(tdt)
+        x = torch.randn(M, K, device="cuda", generator=gen).to(tdt)
+        bias = torch.randn(N, device="cuda", generator=gen).to(tdt) if rnd.random() < 0.3 else None
+        print(f"random linear {cases}: M={M} K={K} N={N} g={g} {tdt} bias={bias is not None}", flush=True)
+        y = gemm_layer._linear("awq_linear", x, qw, qs, qz, bias)
+        ref = x.float() @ nq.awq_dequantize(qw, qs, qz).float()
+        if bias is not None:
+            ref = ref + bias.float()
+        err = ((y.float() - ref).abs().max() / ref.abs().max().clamp_min(1e-6)).item()
+        assert err <= (1.5e-3 if tdt == torch.float16 else 6e-3), err
+        assert torch.equal(y, gemm_layer._linear("awq_linear", x, qw, qs, qz, bias))
