@@ -1314,7 +1314,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
         if (allow_shared_chunk && M > 16 && N % 512 == 0 && N >= 5120 &&
-            K * N >= (M > 32 ? (50ll << 20) : 95000000ll)) {
+            K * N >= (M > 48 ? (50ll << 20) : (M > 32 ? 64000000ll : 95000000ll))) {
             // 17..64 rows on the largest weights (from sweeps: the fused gate|up of Qwen3-8B and the MLP of
             // Qwen3-14B/32B and, above 32 rows, the 32B fused q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
             // one workgroup per CU exists, four chunks per split at least.  Below these sizes re-reading the
