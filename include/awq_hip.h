@@ -153,13 +153,19 @@ int awq_gemv_rmsnorm_qkv_rope_store(const void* x, const float* ssq, const void*
                                     int64_t num_slots, int64_t block_size, float eps, int dtype, void* workspace,
                                     size_t workspace_bytes, void* stream);
 
-/* Optional hint for latency-bound decode loops: the next awq_gemv / awq_linear / awq_gemv_swiglu call of
- * the calling thread that takes the staged GEMV path and leaves compute units idle also launches a few
- * spare workgroups that read [ptr, ptr + bytes) -- meant to be the packed qweight of the launch AFTER it --
- * so that that launch finds its weights in the 256 MB Infinity Cache instead of HBM.  Up to four regions
- * (qweight, qscales, qzeros ...) can be pending; all are consumed (or dropped) by that one call; they never
- * change results.  ptr must be 128-byte aligned, NULL clears the pending hints.  No reference counterpart (the reference launches each linear on its own). */
+/* Optional hint for latency-bound decode loops: names a region [ptr, ptr + bytes) -- meant to be the packed
+ * qweight of the launch AFTER the next one -- that the next linear call of the calling thread (any awq_gemv*,
+ * awq_gemm*, awq_linear* entry point) may pull into the 256 MB Infinity Cache.  That call takes every pending
+ * region on entry, before it checks its arguments: if it runs the one-tile staged GEMV and leaves compute units
+ * idle it launches a few spare workgroups that read the regions; any other kernel, and any error return, drops
+ * them.  Hints therefore never outlive the next linear call and never change results.  Up to four regions
+ * (qweight, qscales, qzeros ...) can be pending; further ones are ignored.  ptr must be 128-byte aligned and stay
+ * mapped until that next call's kernel has run; NULL clears the pending hints.  No reference counterpart (the
+ * reference launches each linear on its own). */
 int awq_prefetch_hint(const void* ptr, size_t bytes);
+/* Number of regions pending on the calling thread (0..4); host-only, for callers and tests that want to see the
+ * rule above at work.  No reference counterpart. */
+int awq_prefetch_pending(void);
 
 /* Prefill regime, any M >= 1 (meant for M > 16): fused dequant + MFMA GEMM,
  * y = x @ dequant(W) (+ bias), W rounded to dtype exactly as the reference

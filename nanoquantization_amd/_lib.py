@@ -43,6 +43,7 @@ SYMBOLS = {
     "awq_gemv_rmsnorm_qkv_rope_store": (_int, [_vp, _vp, _vp, ctypes.c_float] + [_vp] * 11 + [_i64] * 9 +
                                         [ctypes.c_float, _int, _vp, _sz, _vp]),
     "awq_prefetch_hint": (_int, [_vp, _sz]),
+    "awq_prefetch_pending": (_int, []),
     "awq_gemm": (_int, _LINEAR_ARGS),
     "awq_linear": (_int, _LINEAR_ARGS),
     "awq_gemv_plan": (_int, [_i64, _i64, _i64, _i64, ctypes.POINTER(_int), ctypes.POINTER(_int)]),
@@ -149,16 +150,23 @@ def workspace_bytes(entry: str, M: int, N: int, K: int, extra: tuple = ()) -> in
 
 # One zero-initialised split-K workspace per (device, stream).  The kernels leave
 # it zeroed, and calls on one stream are ordered, so it is shared by every layer.
+# A workspace is never freed: a HIP graph captured while it was current keeps its
+# address in its kernel arguments, so when a larger one is needed the old tensor is
+# retired, not released (its memory must not be handed to anyone else, and its
+# arrival counters must stay zero between replays).
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
+_retired_workspaces: list[torch.Tensor] = []
 
 
-def workspace(device: torch.device, stream_ptr: int, nbytes: int) -> torch.Tensor | None:
+def workspace(device: torch.device, stream_ptr: int, nbytes: int, _alloc=None) -> torch.Tensor | None:
     if nbytes == 0:
         return None
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            _retired_workspaces.append(ws)
         size = max(nbytes, 8 << 20)
-        ws = torch.zeros(size, dtype=torch.uint8, device=device)
+        ws = (_alloc or torch.zeros)(size, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws

@@ -307,6 +307,10 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
                          void* stream, int variant, int split_k, int act = 0) {
+    // prefetch hints pending on this thread were meant for this call; the GEMM fills the chip, so they are dropped
+    // (before any check: an error return must not leave them for an unrelated later launch)
+    PrefetchRegions dropped;
+    take_prefetch_hint(&dropped);
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
     if (K % kBK != 0 || !(g % 64 == 0 || (64 % g == 0 && g % 8 == 0))) {

@@ -1168,7 +1168,7 @@ template <typename T, int WK>
 static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const void* qscales,
                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                                   int g, void* workspace, int split_k, hipStream_t stream, int act,
-                                  const GemvFusion& fu = GemvFusion{}) {
+                                  PrefetchRegions pf, const GemvFusion& fu = GemvFusion{}) {
     const int groups = N / 128;
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
@@ -1198,9 +1198,7 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
         }
     }
     (void)hipGetLastError();  // do not report an earlier, unrelated failure as this launch's
-    // pending prefetch hints ride on this launch when the compute grid leaves CUs idle
-    PrefetchRegions pf;
-    take_prefetch_hint(&pf);
+    // the caller's pending prefetch hints ride on this launch when the compute grid leaves CUs idle
     long long pf_bytes = 0;
     for (int r = 0; r < pf.count; ++r) pf_bytes += pf.bytes[r];
     int pf_wgs = 0;
@@ -1255,8 +1253,6 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
         raised = true;
     }
     (void)hipGetLastError();
-    PrefetchRegions pf;
-    take_prefetch_hint(&pf);   // this kernel fills the chip; a pending hint is dropped
     hipLaunchKernelGGL(kern, dim3(groups, splits), dim3(512), lds, stream,
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
@@ -1377,6 +1373,10 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
                          void* stream, int variant, int split_k, int act = 0,
                          const GemvFusion& fu = GemvFusion{}) {
+    // Pending prefetch hints belong to this call whatever becomes of it: they are taken before any check, ride on
+    // the one-tile staged launch, and are dropped by every other kernel and by every error return.
+    PrefetchRegions pf;
+    take_prefetch_hint(&pf);
     int rc = check_linear_args(fn, x, qweight, qscales, qzeros, y, M, N, K, g, dtype);
     if (rc != AWQ_OK) return rc;
     if (act && (variant < kFirstDmaVariant || bias)) {
@@ -1452,12 +1452,12 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                     : launch_gemv_wide<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
             break;
         case kDma1x4:
-            e = f16 ? launch_gemv_dma<F16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu)
-                    : launch_gemv_dma<BF16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu);
+            e = f16 ? launch_gemv_dma<F16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, pf, fu)
+                    : launch_gemv_dma<BF16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, pf, fu);
             break;
         case kDma1x8:
-            e = f16 ? launch_gemv_dma<F16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu)
-                    : launch_gemv_dma<BF16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu);
+            e = f16 ? launch_gemv_dma<F16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, pf, fu)
+                    : launch_gemv_dma<BF16, 8>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, pf, fu);
             break;
         default: {
             // register path; group sizes 32/64/96...: one 32-row step per chunk, always with the next chunk prefetched
@@ -1530,15 +1530,22 @@ extern "C" int awq_gemv_swiglu(const void* x, const int32_t* qweight, const void
 }
 
 namespace awq {
+// error return of an entry point that has not reached gemv_dispatch: pending prefetch hints go with it
+static int fail_drop(int rc) {
+    PrefetchRegions dropped;
+    take_prefetch_hint(&dropped);
+    return rc;
+}
+
 static int make_norm_prologue(const char* fn, const float* ssq, const void* norm_weight, float norm_eps, int64_t M,
                               NormPrologue* np) {
     if (!ssq || !norm_weight) {
         set_error("%s: null pointer argument", fn);
-        return AWQ_ERR_INVALID_ARG;
+        return fail_drop(AWQ_ERR_INVALID_ARG);
     }
     if ((reinterpret_cast<uintptr_t>(norm_weight) & 15u) || (reinterpret_cast<uintptr_t>(ssq) & 3u)) {
         set_error("%s: the norm weight must be 16-byte aligned, the sums of squares 4-byte aligned", fn);
-        return AWQ_ERR_INVALID_ARG;
+        return fail_drop(AWQ_ERR_INVALID_ARG);
     }
     np->weight = reinterpret_cast<const uint16_t*>(norm_weight);
     np->ssq = ssq;
@@ -1556,20 +1563,20 @@ static int qkv_rope_store_entry(const char* fn, const void* x, const NormPrologu
                                 void* stream) {
     if (!q_weight || !k_weight || !cos_sin || !positions || !slots || !q_out || !k_cache || !v_cache) {
         set_error("%s: null pointer argument", fn);
-        return AWQ_ERR_INVALID_ARG;
+        return fail_drop(AWQ_ERR_INVALID_ARG);
     }
     if ((reinterpret_cast<uintptr_t>(q_weight) | reinterpret_cast<uintptr_t>(k_weight) |
          reinterpret_cast<uintptr_t>(cos_sin) | reinterpret_cast<uintptr_t>(q_out) |
          reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15u) {
         set_error("%s: every tensor must be 16-byte aligned", fn);
-        return AWQ_ERR_INVALID_ARG;
+        return fail_drop(AWQ_ERR_INVALID_ARG);
     }
     if (num_heads <= 0 || num_kv_heads <= 0 || N != (num_heads + 2 * num_kv_heads) * 128 || max_positions <= 0 ||
         max_positions > 0x7fffffff || block_size <= 0 || block_size > 0x7fffffff || num_slots <= 0 ||
         num_slots % block_size != 0) {
         set_error("%s: needs head_dim 128 (N == (num_heads + 2 * num_kv_heads) * 128), positive max_positions and "
                   "block_size, and num_slots a multiple of block_size", fn);
-        return AWQ_ERR_INVALID_ARG;
+        return fail_drop(AWQ_ERR_INVALID_ARG);
     }
     QkvEpilogue qe;
     qe.q_weight = reinterpret_cast<const uint16_t*>(q_weight);
@@ -1650,7 +1657,7 @@ extern "C" int awq_gemv_add_residual(const void* x, const int32_t* qweight, cons
     const char* fn = "awq_gemv_add_residual";
     if (!ssq || (reinterpret_cast<uintptr_t>(ssq) & 3u)) {
         awq::set_error("%s: ssq must be a 4-byte aligned device pointer", fn);
-        return AWQ_ERR_INVALID_ARG;
+        return awq::fail_drop(AWQ_ERR_INVALID_ARG);
     }
     awq::ResidEpilogue re;
     re.ssq = ssq;

@@ -77,15 +77,14 @@ extern "C" int awq_prefetch_hint(const void* ptr, size_t bytes) {
         awq::set_error("awq_prefetch_hint: the region must start on a 128-byte boundary");
         return AWQ_ERR_INVALID_ARG;
     }
-    if (awq::g_pf.count == awq::kMaxPrefetchRegions) {
-        awq::set_error("awq_prefetch_hint: at most %d regions can be pending", awq::kMaxPrefetchRegions);
-        return AWQ_ERR_INVALID_ARG;
-    }
+    if (awq::g_pf.count == awq::kMaxPrefetchRegions) return AWQ_OK;   // a hint is optional: further regions are ignored
     awq::g_pf.ptr[awq::g_pf.count] = static_cast<const char*>(ptr);
     awq::g_pf.bytes[awq::g_pf.count] = (long long)bytes;
     ++awq::g_pf.count;
     return AWQ_OK;
 }
+
+extern "C" int awq_prefetch_pending(void) { return awq::g_pf.count; }
 
 extern "C" int awq_hip_version(void) { return 100; }
 

@@ -28,9 +28,14 @@ How each function is pinned (see tests/test_oracle.py):
   * dequant: brute-force scalar loop, fp16/bf16 rounding checked against torch's
     own conversions, equality with quantize_minmax's x_dq where it must hold.
   * linear_fp32: reduces to a library matmul on the dequantised matrix.
-  * linear_splitk_ref: "parity unpinned" -- the reference's Triton kernel
-    cannot run without a GPU and its test holds no stored vectors; used only to
-    report how far the reference's own schedule sits from the fp32 oracle.
+  * linear_splitk_ref: what the schedule's arithmetic fixes -- one split of
+    one block is the rounded fp32 product; a one-hot x returns one row of the
+    dequantised weight for every split count (each K row owned by exactly one
+    split); a scalar pure-Python walk of the kernel's own pointer arithmetic
+    (pid_k * BLOCK_K start, stride BLOCK_K * SPLIT_K, per-split rounding, sum,
+    final rounding) on integer-valued data where every fp32 sum is exact and
+    the 16-bit roundings are active -- a contiguous (wrong) block assignment
+    gives different bits on the same data.
 
 bf16 values are carried as uint16 bit patterns (numpy has no bfloat16).
 """
@@ -229,7 +234,7 @@ def linear_splitk_ref(x_bits, qweight, qzeros, qscales_bits, dtype: str, split_k
     """The reference kernel's rounding schedule (gemm.py:217,313-326,378): split s
     owns K-blocks s, s+S, s+2S, ... of `block_k` rows; fp32 accumulate inside a
     split; each partial rounded to `dtype`; partials summed and rounded to `dtype`.
-    Returns uint16 bits [M, N].  PARITY UNPINNED (no stored reference vectors)."""
+    Returns uint16 bits [M, N]."""
     x = from_bits16(x_bits, dtype)
     w = dequant_f32(qweight, qzeros, qscales_bits, dtype)
     K = w.shape[0]

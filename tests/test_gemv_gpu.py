@@ -207,7 +207,8 @@ def test_prefetch_hint_never_changes_results():
         ref = nq.awq_gemm(xd, *dev, 8)
         nq.prefetch_hint(other, dev[1], dev[2])
         got = nq.awq_gemm(xd, *dev, 8)
-        again = nq.awq_gemm(xd, *dev, 8)           # the hint was consumed
+        assert L.awq_prefetch_pending() == 0       # the hint was consumed
+        again = nq.awq_gemm(xd, *dev, 8)
         torch.cuda.synchronize()
         assert torch.equal(got, ref) and torch.equal(again, ref)
     assert L.awq_prefetch_hint(ctypes.c_void_p(64), 1024) == 1      # not 128-byte aligned
@@ -215,5 +216,6 @@ def test_prefetch_hint_never_changes_results():
     buf = torch.zeros(1024, dtype=torch.uint8, device="cuda")
     for _ in range(4):
         assert L.awq_prefetch_hint(buf.data_ptr(), 1024) == 0
-    assert L.awq_prefetch_hint(buf.data_ptr(), 1024) == 1           # a fifth pending region is refused
-    assert L.awq_prefetch_hint(None, 0) == 0
+    assert L.awq_prefetch_hint(buf.data_ptr(), 1024) == 0           # a fifth region is ignored, not an error
+    assert L.awq_prefetch_pending() == 4
+    assert L.awq_prefetch_hint(None, 0) == 0 and L.awq_prefetch_pending() == 0

@@ -218,3 +218,40 @@ def test_every_entry_point_validates_before_touching_a_device():
         checked += 1
     assert checked >= 25
     assert L.awq_prefetch_hint(None, 0) == 0
+
+
+def test_prefetch_hints_never_outlive_the_next_linear_call():
+    """Hints are taken on entry of every linear entry point, before argument checks: a failing call (null pointers:
+    no device needed) clears them, and a full queue ignores further regions instead of failing."""
+    _ensure_built()
+    L = _lib.lib()
+    assert L.awq_prefetch_hint(None, 0) == 0
+    fake = ctypes.c_void_p(1 << 20)   # never dereferenced on the host
+    for entry in ("awq_gemv", "awq_gemm", "awq_linear", "awq_gemv_swiglu", "awq_linear_swiglu", "awq_gemv_ex",
+                  "awq_gemm_ex", "awq_gemv_add_residual", "awq_gemv_rmsnorm"):
+        for _ in range(6):
+            assert L.awq_prefetch_hint(fake, 4096) == 0
+        assert L.awq_prefetch_pending() == 4
+        res, args = _lib.SYMBOLS[entry]
+        vals = [1e-6 if a is ctypes.c_float else 128 if a in (ctypes.c_int64, ctypes.c_size_t) else 0
+                if a is ctypes.c_int else None for a in args]
+        assert getattr(L, entry)(*vals) != 0
+        assert L.awq_prefetch_pending() == 0, entry
+
+
+def test_superseded_workspaces_stay_alive():
+    """A workspace that a captured graph may still point to is retired, never freed, when a larger one replaces it
+    (bookkeeping only: allocation on the CPU through the test hook)."""
+    dev = torch.device("cpu", 0)
+    alloc = lambda n, dtype, device: torch.zeros(n, dtype=dtype)   # noqa: E731
+    key_stream = 0x5eed
+    before = len(_lib._retired_workspaces)
+    a = _lib.workspace(dev, key_stream, 1 << 10, _alloc=alloc)
+    assert a.numel() == 8 << 20 and _lib.workspace(dev, key_stream, 4 << 20, _alloc=alloc) is a
+    b = _lib.workspace(dev, key_stream, 9 << 20, _alloc=alloc)
+    assert b is not a and b.numel() == 9 << 20
+    assert len(_lib._retired_workspaces) == before + 1 and _lib._retired_workspaces[-1] is a
+    assert _lib.workspace(dev, key_stream, 1 << 10, _alloc=alloc) is b
+    assert _lib.workspace(dev, key_stream, 0) is None
+    del _lib._workspaces[(0, key_stream)]
+    _lib._retired_workspaces.pop()

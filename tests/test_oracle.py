@@ -245,3 +245,88 @@ def test_packed_weight_bytes_table():
     assert o.packed_weight_bytes(1024, 3072) == 1634304
     assert o.packed_weight_bytes(4096, 12288) == 26148864
     assert o.packed_weight_bytes(5120, 25600) == 68096000
+
+
+# ---- linear_splitk_ref: the reference's own split-K rounding schedule ---------------------------------------------
+def _exact_case(dtype, K=512, N=16, M=4, seed=5):
+    """Integer-valued x and power-of-two scales: every fp32 partial sum is an exact integer (no dependence on the
+    summation order) large enough that the roundings to 16 bits change it."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, size=(K, N))
+    z = rng.integers(0, 16, size=(K // 128, N))
+    qweight, qzeros = o.pack_awq(q), o.pack_awq(z)
+    scales = o.to_bits16(np.full((K // 128, N), 1.0, np.float32), dtype)
+    x = rng.integers(-128, 129, size=(M, K)).astype(np.float32)
+    return o.to_bits16(x, dtype), qweight, qzeros, scales
+
+
+def _splitk_scalar_walk(x_bits, qweight, qzeros, scales, dtype, split_k, block_k, contiguous=False):
+    """Scalar walk of nanoquantization/layers/gemm.py:217,251-326,378: program pid_k starts at row pid_k * BLOCK_K,
+    takes BLOCK_K rows, then jumps BLOCK_K * SPLIT_K rows, cdiv(K, BLOCK_K * SPLIT_K) times, rows past K masked; the
+    fp32 accumulator is stored rounded to the output type and the partials are summed and rounded once more."""
+    x = o.from_bits16(x_bits, dtype)
+    w = o.dequant_f32(qweight, qzeros, scales, dtype)
+    M, K = x.shape
+    N = w.shape[1]
+    out = np.zeros((M, N), np.float32)
+    iters = -(-K // (block_k * split_k))
+    for m in range(M):
+        for n in range(N):
+            total = np.float32(0.0)
+            for pid_k in range(split_k):
+                acc = np.float32(0.0)
+                start = pid_k * (iters * block_k) if contiguous else pid_k * block_k
+                for it in range(iters):
+                    for kk in range(block_k):
+                        k = start + kk
+                        if k < K:
+                            acc = np.float32(acc + np.float32(x[m, k] * w[k, n]))
+                    start += block_k if contiguous else block_k * split_k
+                total = np.float32(total + o.to_dtype_f32(np.array([acc], np.float32), dtype)[0])
+            out[m, n] = total
+    return o.to_bits16(out, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_splitk_ref_matches_scalar_walk_of_the_kernel_schedule(dtype):
+    xb, qw, qz, sc = _exact_case(dtype)
+    for split_k, block_k in ((8, 32), (4, 32), (2, 64), (8, 16)):
+        got = o.linear_splitk_ref(xb, qw, qz, sc, dtype, split_k, block_k)
+        want = _splitk_scalar_walk(xb, qw, qz, sc, dtype, split_k, block_k)
+        assert np.array_equal(got, want), (split_k, block_k)
+    # the data discriminates: partial roundings are active, and a contiguous assignment of K blocks to splits
+    # (a plausible slip) gives other bits
+    one = o.linear_splitk_ref(xb, qw, qz, sc, dtype, 1, 512)
+    assert not np.array_equal(o.linear_splitk_ref(xb, qw, qz, sc, dtype, 8, 32), one)
+    wrong = _splitk_scalar_walk(xb, qw, qz, sc, dtype, 8, 32, contiguous=True)
+    assert not np.array_equal(o.linear_splitk_ref(xb, qw, qz, sc, dtype, 8, 32), wrong)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_splitk_ref_closed_forms(dtype):
+    from conftest import make_case, make_x
+    # one split of one block = the fp32 product rounded once (exact data: no summation-order freedom)
+    xb, qw, qz, sc = _exact_case(dtype, seed=9)
+    x, w = o.from_bits16(xb, dtype), o.dequant_f32(qw, qz, sc, dtype)
+    assert np.array_equal(o.linear_splitk_ref(xb, qw, qz, sc, dtype, 1, 512), o.to_bits16(x @ w, dtype))
+    # one-hot activations return one row of the dequantised weight, bit for bit, whatever the split count: every K
+    # row is owned by exactly one split, the other partials are zero
+    p = make_case(256, 64, 128, dtype, seed=21)
+    wbits = o.dequant(p["qweight"], p["qzeros"], p["qscales"], dtype)
+    rows = [0, 31, 32, 100, 223, 255]
+    eye = np.zeros((len(rows), 256), np.float32)
+    eye[np.arange(len(rows)), rows] = 1.0
+    for split_k in (1, 2, 4, 8):
+        got = o.linear_splitk_ref(o.to_bits16(eye, dtype), p["qweight"], p["qzeros"], p["qscales"], dtype, split_k, 32)
+        assert np.array_equal(got & 0x7FFF, wbits[rows] & 0x7FFF) and np.array_equal(got, np.where(
+            (wbits[rows] & 0x7FFF) == 0, got, wbits[rows]))     # equal up to the sign of zero
+    # more splits than blocks: the surplus splits own nothing
+    xr = make_x(2, 256, dtype, seed=3)
+    a = o.linear_splitk_ref(xr, p["qweight"], p["qzeros"], p["qscales"], dtype, 8, 32)
+    b = o.linear_splitk_ref(xr, p["qweight"], p["qzeros"], p["qscales"], dtype, 16, 32)
+    assert a.shape == b.shape == (2, 64)
+    # linearity that survives the roundings: scaling x by 2 scales y by 2 exactly
+    x2 = o.to_bits16(o.from_bits16(xr, dtype) * 2.0, dtype)
+    y1 = o.from_bits16(a, dtype)
+    y2 = o.from_bits16(o.linear_splitk_ref(x2, p["qweight"], p["qzeros"], p["qscales"], dtype, 8, 32), dtype)
+    assert np.array_equal(y2, 2.0 * y1)
