@@ -214,39 +214,26 @@ def main():
                                  "cases": large}
 
         # ---------------- extra: prefill GEMM, cfg3 -----------------------------------------------------
-        # (a) the fused dequant + MFMA kernel of this library at every M; (b) what awq_linear does by default:
-        # the same kernel below 1024 rows, transposed dequantise + the dense library matmul from there on
-        from nanoquantization_amd.layers import gemm as gemm_layer
+        # the fused dequant + MFMA kernel: what awq_linear / WQLinear_GEMM.forward run at these row counts
         bdt = torch.bfloat16
-        fused, default = {}, {}
+        fused = {}
         for (K, N) in ((4096, 12288), (12288, 4096)):
             w = rand_packed(K, N, bdt, dev)
             for M in (512, 2048, 8192):
                 x = torch.randn(M, K, device=dev).to(bdt)
                 fn = lambda: [nq.awq_gemm(x, *w, 8) for _ in range(4)]
-                for table, min_rows in ((fused, 1 << 62), (default, gemm_layer.TWO_PASS_MIN_ROWS)):
-                    keep, gemm_layer.TWO_PASS_MIN_ROWS = gemm_layer.TWO_PASS_MIN_ROWS, min_rows
-                    try:
-                        us = time_graph(fn, 5, 1) * 1e3 / 4
-                    finally:
-                        gemm_layer.TWO_PASS_MIN_ROWS = keep
-                    tf = 2.0 * M * N * K / us / 1e6
-                    table[f"M{M}_{K}x{N}"] = {"us": round(us, 1), "TFLOPs": round(tf, 1),
-                                               "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4)}
+                us = time_graph(fn, 5, 1) * 1e3 / 4
+                tf = 2.0 * M * N * K / us / 1e6
+                fused[f"M{M}_{K}x{N}"] = {"us": round(us, 1), "TFLOPs": round(tf, 1),
+                                          "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4)}
             del w
         bestf = max(v["TFLOPs"] for v in fused.values())
-        bestd = max(v["TFLOPs"] for v in default.values())
         out["roofline_prefill"] = {
             "kernel": "awq::gemm_pipe_kernel<BF16,2,4>", "bound": "mfma", "achieved": bestf,
             "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": bestf / MFMA_PEAK_TFLOPS,
-            "workload": "cfg3: Qwen3-8B MLP shapes, bf16, M in {512,2048,8192}; the fused dequant + MFMA kernel",
-            "cases": fused,
-            "default_dispatch": {
-                "kernels": "below 1024 rows the fused kernel; from 1024 rows awq::dequant_transpose_kernel "
-                           "(weight -> [N, K] in the activation type, 0.52 B read + 2 B written per weight) + the "
-                           "dense library matmul x @ wt^T (torch.matmul -> hipBLASLt), the reference's own large-M "
-                           "structure (layers/gemm.py:558-561) with a transposed weight",
-                "achieved": bestd, "frac": bestd / MFMA_PEAK_TFLOPS, "cases": default}}
+            "workload": "cfg3: Qwen3-8B MLP shapes, bf16, M in {512,2048,8192}; the fused dequant + MFMA kernel "
+                        "(default dispatch at every M)",
+            "cases": fused}
 
         # ---------------- extra: dequantise kernel ------------------------------------------------------
         K, N = 4096, 12288

@@ -135,6 +135,12 @@ __device__ __forceinline__ float mul_round(float a, float b) {
     asm("" : "+v"(p));
     return T::to_f32(T::from_f32(p));
 }
+// acc + bias with the reference's two rounding points: the product is rounded to T first, then `out.add_(bias)`
+// adds in fp32 and rounds again (nanoquantization/layers/gemm.py:561-566).  The caller rounds the returned sum to T.
+template <typename T>
+__device__ __forceinline__ float add_bias(float acc, float b) {
+    return T::to_f32(T::from_f32(acc)) + b;
+}
 // The same barrier for any fp32 value about to be rounded to T: the value is an fp32 result first.
 __device__ __forceinline__ float as_f32_result(float v) {
     asm("" : "+v"(v));

@@ -78,14 +78,14 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[TM][TN], const uint1
         for (int b = 0; b < TN; ++b) {
             const int n = n0 + wn0 + b * 32 + li;
             if (n >= N) continue;
-            float bv = 0.f;
-            if (direct && bias) bv = T::to_f32(bias[n]);
+            const bool has_bias = direct && bias;
+            const float bv = has_bias ? T::to_f32(bias[n]) : 0.f;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm0 + a * 32 + (v >> 2) * 8 + kb2 * 4 + (v & 3);
                 if (m >= M) continue;
                 if (direct)
-                    y[(size_t)m * N + n] = T::from_f32(acc[a][b][v] + bv);
+                    y[(size_t)m * N + n] = T::from_f32(has_bias ? add_bias<T>(acc[a][b][v], bv) : acc[a][b][v]);
                 else
                     partials[((size_t)split * M + m) * N + n] = acc[a][b][v];   // 32 lanes = one 128-byte line
             }
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
         const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + nn);
 #pragma unroll
         for (int c = 0; c < 8; ++c)
-            out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
+            out[c] = add_bias<T>(out[c], T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu))));
     }
     u32x4 o;
 #pragma unroll

@@ -323,7 +323,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
             for (int b = 0; b < TN; ++b)
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    stage[((v >> 2) * 8 + kb2 * 4 + (v & 3)) * PITCH + b * 32 + li] = T::from_f32(acc[a][b][v] + bv[b]);
+                    stage[((v >> 2) * 8 + kb2 * 4 + (v & 3)) * PITCH + b * 32 + li] =
+                        T::from_f32(bias ? add_bias<T>(acc[a][b][v], bv[b]) : acc[a][b][v]);
 #pragma unroll
             for (int j = 0; j < 32 / RPP; ++j) {
                 const int row = RPP * j + lane / LPR, chunk = lane % LPR;
@@ -437,7 +438,7 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __re
         const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + n);
 #pragma unroll
         for (int c = 0; c < 8; ++c)
-            out[c] += T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
+            out[c] = add_bias<T>(out[c], T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu))));
     }
     u32x4 o;
 #pragma unroll

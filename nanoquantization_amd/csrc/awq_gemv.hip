@@ -470,7 +470,7 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
                     const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
 #pragma unroll
                     for (int c = 0; c < 8; ++c)
-                        out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
+                        out[c] = add_bias<T>(out[c], T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu))));
                 }
                 u32x4 o;
 #pragma unroll
@@ -545,7 +545,7 @@ __device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int spli
             const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
 #pragma unroll
             for (int c = 0; c < 8; ++c)
-                out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
+                out[c] = add_bias<T>(out[c], T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu))));
         }
         u32x4 o;
 #pragma unroll
@@ -1092,7 +1092,7 @@ __global__ __launch_bounds__(256) void gemv_wide_reduce_kernel(const float* __re
         const u32x4 bv = *reinterpret_cast<const u32x4*>(bias + n0);
 #pragma unroll
         for (int c = 0; c < 8; ++c)
-            out[c] += T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu)));
+            out[c] = add_bias<T>(out[c], T::to_f32((uint16_t)((c & 1) ? (bv[c >> 1] >> 16) : (bv[c >> 1] & 0xFFFFu))));
     }
     u32x4 o;
 #pragma unroll

@@ -299,16 +299,12 @@ def interleave_gate_up(gate, up):
 
 
 def awq_linear_swiglu(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor) -> torch.Tensor:
-    """x [M, K] (any M) and interleaved gate|up buffers [K, 2*inter/8] -> SiLU(x @ Wgate) * (x @ Wup) [M, inter].
-    From layers.gemm.TWO_PASS_MIN_ROWS rows on: the plain product on the two-pass path, then the gate as its own pass."""
+    """x [M, K] (any M) and interleaved gate|up buffers [K, 2*inter/8] -> SiLU(x @ Wgate) * (x @ Wup) [M, inter]."""
     dev = _dev(x, qweight, qscales, qzeros)
     M, K = x.shape
     N = qscales.shape[1]
     g = K // qscales.shape[0]
     assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
-    from ..layers import gemm as _gemm
-    if _gemm._two_pass_ok(M, K, g):
-        return silu_mul(_gemm._linear("awq_linear", x, qweight, qscales, qzeros, None), interleaved=True)
     out = torch.empty(M, N // 2, dtype=x.dtype, device=dev)
     L = _lib.lib()
     with _lib.on_device(dev):

@@ -69,15 +69,10 @@ def awq_dequantize(
     return out
 
 
-# From this many rows on, awq_linear takes the reference's own large-M structure (layers/gemm.py:558-561:
-# dequantise, then a dense library matmul) -- with the weight written transposed, the layout the library runs
-# fastest on.  Measured on MI355X at 4096 x 12288, bf16: 8192 rows 1.45 PFLOP/s against 1.0-1.1 for the fused
-# kernel (the 30 us dequantise pass included), 2048 rows 1.08 against 0.9, 512 rows a tie.
-TWO_PASS_MIN_ROWS = 1024
-
-
 def awq_dequantize_transposed(qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor) -> torch.Tensor:
-    """Packed int4 -> [N, K] weight (k-contiguous rows) in qscales.dtype: awq_dequantize(...).t(), bit for bit."""
+    """Packed int4 -> [N, K] weight (k-contiguous rows) in qscales.dtype: awq_dequantize(...).t(), bit for bit.
+    A free-standing utility (the layout dense GEMM libraries like best); the linear itself never materialises the
+    weight: every M runs the fused dequant + MFMA kernel."""
     K, N, g = _check_packed(qweight, qscales, qzeros)
     dev = _require_device(qweight, qscales, qzeros)
     qweight, qscales, qzeros = qweight.contiguous(), qscales.contiguous(), qzeros.contiguous()
@@ -87,10 +82,6 @@ def awq_dequantize_transposed(qweight: torch.Tensor, qscales: torch.Tensor, qzer
         _lib.check(_lib.lib().awq_dequantize_transposed(_ptr(qweight), _ptr(qscales), _ptr(qzeros), _ptr(out),
                                                         K, N, g, _lib.dtype_id(qscales.dtype), stream))
     return out
-
-
-def _two_pass_ok(M: int, K: int, g: int) -> bool:
-    return M >= TWO_PASS_MIN_ROWS and K % 64 == 0 and (g % 64 == 0 or (64 % g == 0 and g % 8 == 0))
 
 
 def _linear(entry: str, x, qweight, qscales, qzeros, bias, extra=()):
@@ -105,12 +96,6 @@ def _linear(entry: str, x, qweight, qscales, qzeros, bias, extra=()):
         x, qweight, qscales, qzeros = x.contiguous(), qweight.contiguous(), qscales.contiguous(), qzeros.contiguous()
     if bias is not None and (bias.dtype != dt or bias.device != dev or not bias.is_contiguous()):
         bias = bias.to(device=dev, dtype=dt).contiguous()
-    if entry == "awq_linear" and _two_pass_ok(M, K, g):
-        wt = awq_dequantize_transposed(qweight, qscales, qzeros)
-        out = torch.matmul(x, wt.t())
-        if bias is not None:
-            out.add_(bias)          # as the reference does, layers/gemm.py:565-566
-        return out
     out = torch.empty(M, N, dtype=dt, device=dev)
     if M == 0:
         return out
@@ -264,6 +249,14 @@ class WQLinear_GEMM(nn.Module):
         # (nn.Module.__getattr__ costs more than the rest of this function).
         buf = self._buffers
         bias = buf["bias"] if "bias" in buf else self.bias
+        if bias is not None and bias.dtype != buf["qscales"].dtype:
+            # the bias buffer is bf16 whatever the output type (layers/gemm.py:435-443): convert once, not per call
+            key = (bias.data_ptr(), bias._version, buf["qscales"].dtype, bias.device)
+            cached = self.__dict__.get("_bias_cast")
+            if cached is None or cached[0] != key:
+                cached = (key, bias.to(buf["qscales"].dtype))
+                self.__dict__["_bias_cast"] = cached
+            bias = cached[1]
         if x.dim() == 2:
             return _linear("awq_linear", x, buf["qweight"], buf["qscales"], buf["qzeros"], bias)
         out_shape = x.shape[:-1] + (self.out_features,)

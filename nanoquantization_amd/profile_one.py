@@ -1,7 +1,6 @@
 """Launch one AWQ linear of a given shape a few times, for a profiler or counter collection to look at:
 
     python3 -m nanoquantization_amd.profile_one linear K N M [--dtype bf16|f16] [--iters 6] [--group-size 128]
-    python3 -m nanoquantization_amd.profile_one fused  K N M ...     # the fused kernels also from 1024 rows on
     python3 -m nanoquantization_amd.profile_one dequant K N 0 ...
     python3 -m nanoquantization_amd.profile_one copy K N 0 ...       # device copy of the packed weight (counter calibration)
 
@@ -15,7 +14,7 @@ import torch
 
 def main() -> None:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("kind", choices=["linear", "fused", "dequant", "copy"])
+    ap.add_argument("kind", choices=["linear", "dequant", "copy"])
     ap.add_argument("K", type=int)
     ap.add_argument("N", type=int)
     ap.add_argument("M", type=int)
@@ -24,7 +23,6 @@ def main() -> None:
     ap.add_argument("--group-size", type=int, default=128)
     a = ap.parse_args()
     import nanoquantization_amd as nq
-    from nanoquantization_amd.layers import gemm as gemm_layer
     dev, g = torch.device("cuda:0"), a.group_size
     tdt = torch.bfloat16 if a.dtype == "bf16" else torch.float16
     gen = torch.Generator(device=dev).manual_seed(a.K + a.N)
@@ -32,9 +30,7 @@ def main() -> None:
     qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (a.K // g, a.N // 8), dtype=torch.int32, device=dev, generator=gen)
     qs = (torch.rand(a.K // g, a.N, device=dev, generator=gen) * 0.02 + 0.001).to(tdt)
     x = torch.randn(max(a.M, 1), a.K, device=dev, generator=gen).to(tdt)
-    if a.kind == "fused":
-        gemm_layer.TWO_PASS_MIN_ROWS = 1 << 62
-    fn = {"linear": lambda: nq.awq_gemm(x, qw, qs, qz, 8), "fused": lambda: nq.awq_gemm(x, qw, qs, qz, 8),
+    fn = {"linear": lambda: nq.awq_gemm(x, qw, qs, qz, 8),
           "dequant": lambda: nq.awq_dequantize(qw, qs, qz), "copy": lambda: qw.clone()}[a.kind]
     for _ in range(a.iters):
         fn()

@@ -133,11 +133,12 @@ def test_dequantize_transposed_bit_exact(dtype, K, N, g):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("M,K,N,g", [(1024, 1024, 1032, 128), (1500, 512, 2048, 64), (2048, 256, 264, 32)])
-def test_linear_two_pass_large_m(dtype, M, K, N, g):
-    # 1024 rows and more: transposed dequantise + the dense library matmul (the reference's large-M structure,
-    # layers/gemm.py:558-561), against the fp32 oracle, with and without bias, and against the fused kernel
+def test_linear_large_m_equals_dequantise_then_matmul(dtype, M, K, N, g):
+    # 1024 rows and more, the regime of the reference's awq_dequantize + torch.matmul (layers/gemm.py:558-561): the
+    # default dispatch (fused kernel) against the fp32 oracle, with and without bias, against the forced whole-tile
+    # variant, and against that two-step structure built from awq_dequantize_transposed + a dense matmul
     from nanoquantization_amd.layers.gemm import _linear
-    print(f"two-pass linear {dtype} M={M} K={K} N={N} g={g}", flush=True)
+    print(f"large-M linear {dtype} M={M} K={K} N={N} g={g}", flush=True)
     p = make_case(K, N, g, dtype, seed=M + N)
     xb = make_x(M, K, dtype, seed=M)
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
@@ -150,8 +151,10 @@ def test_linear_two_pass_large_m(dtype, M, K, N, g):
     L = _lib.lib()
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
     fused = awq_gemm_variant(xd, *dev, names.index("256x256p"), 1)
-    err = (y.float() - fused.float()).abs().max().item() / fused.float().abs().max().item()
-    assert err <= (2e-3 if dtype == "f16" else 1.6e-2), err     # both round an fp32 sum of the same products once
+    two_step = torch.matmul(xd, nq.awq_dequantize_transposed(*dev).t())
+    for other in (fused, two_step):
+        err = (y.float() - other.float()).abs().max().item() / other.float().abs().max().item()
+        assert err <= (2e-3 if dtype == "f16" else 1.6e-2), err     # both round an fp32 sum of the same products once
 
 
 def test_gemm_prefill_full_size_bf16():
@@ -164,28 +167,43 @@ def test_gemm_prefill_full_size_bf16():
     _check(y, xb, p, "bf16")
 
 
-@pytest.mark.parametrize("M,K,N", [(8192, 4096, 12288), (8192, 12288, 4096), (4096, 8192, 5120), (300, 5120, 25600)])
+@pytest.mark.parametrize("M,K,N", [(8192, 4096, 12288), (8192, 12288, 4096), (2048, 4096, 12288), (2048, 12288, 4096),
+                                   (512, 12288, 4096), (4096, 8192, 5120), (300, 5120, 25600)])
 def test_gemm_largest_shapes_properties(M, K, N):
-    """The largest prefill shapes (Qwen3-8B MLP at M = 8192, Qwen3-32B o_proj at a 4096-token prefill and gate/up
-    at a ragged M), too big for the CPU oracle: checked through size-independent properties.  (1) rows sampled
-    across every workgroup tile equal the same rows pushed through the kernel alone (a row's result does not
-    depend on M or on its tile) -- and those small calls are checked against the fp32 matmul of the dequantised,
-    bit-exact weight; (2) the kernel is run-to-run bit-stable; (3) zero rows give exact zeros."""
+    """The prefill shapes at their real sizes (Qwen3-8B MLP at M = 512 / 2048 / 8192, Qwen3-32B o_proj at a 4096-token
+    prefill and gate/up at a ragged M), too big for the CPU oracle: checked through size-independent properties, on
+    the default dispatch and on the pipelined fused kernel forced in both of its forms (every tile whole; the tiles
+    of the last round cut along K with the plan's split).  (1) rows sampled across every workgroup tile equal the
+    fp32 matmul of those rows with the dequantised weight (itself bit-exact against the oracle); (2) the same rows
+    pushed through alone (another tile shape) agree too; (3) run-to-run bit-stable; (4) a zero row gives exact zeros."""
     print(f"gemm properties M={M} K={K} N={N} bf16", flush=True)
+    L = _lib.lib()
+    names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
+    import ctypes
+    v, sp = ctypes.c_int(), ctypes.c_int()
+    assert L.awq_gemm_plan(M, N, K, ctypes.byref(v), ctypes.byref(sp)) == 0
     g = torch.Generator(device="cuda").manual_seed(M + K)
     qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
     qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, N // 8), dtype=torch.int32, device="cuda", generator=g)
     sc = (torch.rand(K // 128, N, device="cuda", generator=g) * 0.01 + 0.002).to(torch.bfloat16)
     x = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
     x[5] = 0
-    y = nq.awq_gemm(x, qw, sc, qz, 8)
-    assert torch.equal(y, nq.awq_gemm(x, qw, sc, qz, 8))
-    assert torch.count_nonzero(y[5]) == 0
     rows = torch.arange(3, M, max(1, M // 61), device="cuda")[:64]          # one or two rows of every 256-row tile
     w = nq.awq_dequantize(qw, sc, qz).float()
     ref = x[rows].float() @ w
-    err = ((y[rows].float() - ref).abs().max() / ref.abs().max()).item()
-    assert err <= TIGHT["bf16"], err
+    runs = [("default " + names[v.value] + f" split {sp.value}", lambda: nq.awq_gemm(x, qw, sc, qz, 8)),
+            ("256x256p split 1", lambda: awq_gemm_variant(x, qw, sc, qz, names.index("256x256p"), 1)),
+            (f"256x256pt split {max(sp.value, 2)}",
+             lambda: awq_gemm_variant(x, qw, sc, qz, names.index("256x256pt"), max(sp.value, 2)))]
+    for what, run in runs:
+        print(f"  {what}", flush=True)
+        y = run()
+        torch.cuda.synchronize()
+        assert torch.equal(y, run()), what
+        assert torch.count_nonzero(y[5]) == 0, what
+        err = ((y[rows].float() - ref).abs().max() / ref.abs().max()).item()
+        assert err <= TIGHT["bf16"], (what, err)
+        del y
     sub = nq.awq_gemm(x[rows].contiguous(), qw, sc, qz, 8).float()          # another kernel / tile shape
     assert ((sub - ref).abs().max() / ref.abs().max()).item() <= TIGHT["bf16"]
 

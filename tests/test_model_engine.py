@@ -256,6 +256,91 @@ def test_engine_norm_fused_decode_equals_separate_kernels():
     assert outs[0] == outs[1]
 
 
+def _teacher_forced_check(model, prompts, got, rows=None):
+    """The engine's own continuation pushed through the full-recompute forward (the reference semantics: no cache):
+    every chosen token is that forward's argmax up to the 16-bit noise of a near-tie, and exactly it wherever the
+    logits are not near-tied.  `rows` limits the recompute to some sequences."""
+    rows = list(range(len(prompts))) if rows is None else rows
+    plen = len(prompts[0])
+    seqs = torch.tensor([prompts[r] + got[r] for r in rows], device="cuda")
+    pos = torch.arange(seqs.shape[1], device="cuda").unsqueeze(0)
+    hidden = model(seqs, pos)[:, plen - 1:-1]
+    logits = model.lm_head(hidden).float()
+    chosen = torch.tensor([got[r] for r in rows], device="cuda")
+    gap = logits.max(-1).values - logits.gather(-1, chosen.unsqueeze(-1)).squeeze(-1)
+    scale = logits.abs().max().item()
+    assert gap.max().item() <= 2e-2 * scale, (gap.max().item(), scale)
+    top2 = logits.topk(2, dim=-1).values
+    clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
+    assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
+    return clear.float().mean().item()
+
+
+@pytest.mark.gpu
+def test_engine_full_qwen3_0p6b_architecture_batch_32():
+    """The whole Qwen3-0.6B architecture (28 blocks, hidden 1024, 16 q / 8 kv heads, intermediate 3072, vocabulary
+    151,936, tied head) at batch 32 with 96-token prompts: the graph-captured decode step with every fused GEMV form,
+    against the full-recompute forward."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_0P6B, random_awq_qwen3
+    print("engine: Qwen3-0.6B architecture, 28 layers, batch 32", flush=True)
+    cfg = dict(QWEN3_0P6B, max_position_embeddings=1024)
+    model = random_awq_qwen3(cfg, seed=21, std=0.02)
+    torch.manual_seed(22)
+    plen, new = 96, 6
+    prompts = torch.randint(0, cfg["vocab_size"], (32, plen)).tolist()
+    eng = LLMEngine(model, max_batch=32, max_seq_len=128, block_size=64, use_graph=True)
+    assert eng.norm_fused_ok and eng.qkv_fused_ok and eng.swiglu_ok
+    got = eng.generate(prompts, new)
+    assert len(got) == 32 and all(len(g) == new for g in got)
+    _teacher_forced_check(model, prompts, got)
+    assert eng.generate(prompts, new) == got
+
+
+@pytest.mark.gpu
+def test_engine_qwen3_32b_widths_batch_64_context_2048():
+    """Two blocks at the Qwen3-32B widths with 64 sequences of 2,048 cached tokens each: the decode shapes of the
+    largest configuration (64-row GEMVs on the shared-chunk kernel, paged attention over 32 blocks per sequence with 8
+    query heads per kv head), a 131,072-token batched prefill through the fused GEMM, against the recompute forward
+    on a sample of the sequences."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+    print("engine: Qwen3-32B widths, 2 layers, batch 64, context 2048", flush=True)
+    cfg = dict(QWEN3_32B, num_hidden_layers=2, max_position_embeddings=4096)
+    model = random_awq_qwen3(cfg, seed=23, std=0.02)
+    torch.manual_seed(24)
+    plen, new = 2048, 4
+    prompts = torch.randint(0, cfg["vocab_size"], (64, plen)).tolist()
+    eng = LLMEngine(model, max_batch=64, max_seq_len=plen + 64, block_size=64, use_graph=True)
+    got = eng.generate(prompts, new)
+    assert len(got) == 64 and all(len(g) == new for g in got)
+    _teacher_forced_check(model, prompts, got, rows=[0, 13, 31, 63])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("group_size,max_batch", [(64, 4), (128, 65), (32, 3)])
+def test_engine_shapes_outside_the_fused_decode_forms(group_size, max_batch):
+    """Group sizes 32 / 64 and widths that are not multiples of 128 (the register-path GEMV, no q|k|v / gate|up / norm
+    fusion), and more than 64 batch rows (the decode linears on the MFMA GEMM): the engine issues its prefetch hints
+    before every linear whatever kernel takes it; nothing may be left pending or fail."""
+    from nanoquantization_amd import _lib
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import random_awq_qwen3
+    print(f"engine: group size {group_size}, max_batch {max_batch}", flush=True)
+    cfg = TINY if group_size == 128 else dict(TINY, hidden_size=192, total_num_heads=3, total_num_kv_heads=1,
+                                              head_dim=64, intermediate_size=320)
+    model = random_awq_qwen3(cfg, seed=31, std=0.05, group_size=group_size)
+    torch.manual_seed(32)
+    n = min(max_batch, 5)
+    prompts = torch.randint(0, 512, (n, 21)).tolist()
+    for use_graph in (False, True):
+        eng = LLMEngine(model, max_batch=max_batch, max_seq_len=64, block_size=16, use_graph=use_graph)
+        assert not eng.norm_fused_ok and not eng.qkv_fused_ok
+        got = eng.generate(prompts, 8)
+        assert _lib.lib().awq_prefetch_pending() == 0
+        assert _teacher_forced_check(model, prompts, got) > 0.5
+
+
 def test_paged_kv_cache_block_bookkeeping():
     """Host logic of the cache: blocks are handed out once, come back on release, exhaustion raises (CPU)."""
     from nanoquantization_amd.engine.llm_engine import PagedKVCache

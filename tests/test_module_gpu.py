@@ -67,7 +67,7 @@ def test_state_dict_roundtrip_keeps_outputs():
 @pytest.mark.parametrize("bias", [False, True])
 def test_forward_empty_and_boundary_row_counts(bias):
     """No rows at all, and the row counts where the dispatch changes kernel (16/17 one m-tile vs row blocks, 64/65
-    GEMV vs GEMM, 1023/1024 fused vs two-pass): shape, dtype and the fp32 oracle at every one of them."""
+    GEMV vs GEMM, 1023/1024 where the reference's own structure changes): shape, dtype and the fp32 oracle at every one of them."""
     K, N, g = 512, 384, 128
     m = _module(K, N, g, torch.bfloat16, bias, seed=3)
     for shape in [(0, K), (2, 0, K)]:
