@@ -15,6 +15,8 @@ from oracle import awq_oracle as o
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-2
+# with a bias the reference rounds twice (the product, then out.add_(bias), layers/gemm.py:561-566): one more half ulp
+BIAS_STEP = {"f16": 2.0 ** -11, "bf16": 2.0 ** -8}
 TIGHT = {"f16": 1.5e-3, "bf16": 6e-3}   # output rounding alone is 2^-11 / 2^-8 of the value
 
 QWEN3_0P6B = [(1024, 2048), (1024, 1024), (2048, 1024), (1024, 3072), (3072, 1024)]
@@ -24,7 +26,8 @@ def _check(y, xb, p, dtype, bias=None):
     ref = o.linear_fp32(xb, p["qweight"], p["qzeros"], p["qscales"], dtype, bias)
     err = o.max_rel_err(o.from_bits16(to_bits(y), dtype), ref)
     assert err <= TOL, f"max rel err {err}"
-    assert err <= TIGHT[dtype], f"max rel err {err} (inside the 1e-2 bound but worse than rounding explains)"
+    assert err <= TIGHT[dtype] + BIAS_STEP[dtype] * (bias is not None), \
+        f"max rel err {err} (inside the 1e-2 bound but worse than rounding explains)"
     return err
 
 

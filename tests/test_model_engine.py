@@ -327,7 +327,7 @@ def test_engine_shapes_outside_the_fused_decode_forms(group_size, max_batch):
     from nanoquantization_amd.engine import LLMEngine
     from nanoquantization_amd.models.random_init import random_awq_qwen3
     print(f"engine: group size {group_size}, max_batch {max_batch}", flush=True)
-    cfg = TINY if group_size == 128 else dict(TINY, hidden_size=192, total_num_heads=3, total_num_kv_heads=1,
+    cfg = TINY if group_size == 128 else dict(TINY, hidden_size=192, total_num_heads=4, total_num_kv_heads=2,
                                               head_dim=64, intermediate_size=320)
     model = random_awq_qwen3(cfg, seed=31, std=0.05, group_size=group_size)
     torch.manual_seed(32)
