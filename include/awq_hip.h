@@ -87,6 +87,21 @@ int awq_gemv(const void* x, const int32_t* qweight, const void* qscales, const i
              const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
              int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* awq_gemv for callers that cannot allocate device memory or bring a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): same arguments without the workspace, same kernels, same bits.
+ * The split-K scratch (arrival counters + fp32 partials) is a static device array of
+ * awq_gemv_static_scratch_bytes() = 16 KiB + 16 MiB inside the library, held by every GPU the library runs on until
+ * the process ends; its address is looked up once per device on the first call there.  The call allocates nothing
+ * (no hipMalloc / hipFree, no allocating library routine).  A problem whose split-K plan needs more scratch than
+ * that (awq_gemv_workspace_bytes(M, N, K) tells) is refused with AWQ_ERR_UNSUPPORTED: every 1..16-row shape of the
+ * Qwen3 family fits, 64-row calls on the widest MLP weights do not.  All calls on one GPU share the array: calls that
+ * overlap in time on one GPU (two streams, two threads) race; calls ordered on one stream do not.  The counters are
+ * zero at load and every launch leaves them zero.  It has no counterpart in the reference. */
+size_t awq_gemv_static_scratch_bytes(void);
+int awq_gemv_static(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                    const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size, int dtype,
+                    void* stream);
+
 /* awq_gemv with the gate/up epilogue of the MLP fused in.  The packed buffers hold the gate and the up
  * projection interleaved word by word along N: packed word column 2t = the 8 gate columns 8t..8t+7,
  * word column 2t+1 = the up columns of the same outputs (qzeros and qscales alike), N = 2 * intermediate.

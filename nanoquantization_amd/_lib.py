@@ -34,6 +34,8 @@ SYMBOLS = {
     "awq_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "awq_linear_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "awq_gemv": (_int, _LINEAR_ARGS),
+    "awq_gemv_static_scratch_bytes": (_sz, []),
+    "awq_gemv_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "awq_gemv_swiglu": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "awq_linear_swiglu": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "awq_linear_swiglu_workspace_bytes": (_sz, [_i64, _i64, _i64]),

@@ -42,6 +42,8 @@
 // in split order, so results are bit-stable run to run.
 #include <type_traits>
 
+#include <mutex>
+
 #include "awq_common.hpp"
 
 namespace awq {
@@ -1677,6 +1679,69 @@ extern "C" int awq_gemv_ex(const void* x, const int32_t* qweight, const void* qs
     return awq::gemv_dispatch("awq_gemv_ex", x, qweight, qscales, qzeros, bias, y, M, N, K,
                               group_size, dtype, workspace, workspace_bytes, stream, variant,
                               split_k);
+}
+
+// ---- awq_gemv without any allocation: the split-K scratch is a static device array ----------------------------
+// Zero at load, and every launch leaves its arrival counters at zero again (the last workgroup of a tile resets its
+// counter), so the counters need no clearing between calls; the partials are written before they are read.
+namespace awq {
+constexpr size_t kStaticScratchBytes = kCounterBytes + ((size_t)16 << 20);
+constexpr int kMaxScratchDevices = 64;
+}  // namespace awq
+static __device__ __align__(256) unsigned char scratch[awq::kStaticScratchBytes];
+
+namespace awq {
+// Device address of `scratch` on the current device, looked up once per device (every device has its own copy of
+// the array at its own address); nullptr with the error text set on failure.
+static void* static_scratch_ptr(const char* fn) {
+    static void* ptrs[kMaxScratchDevices] = {};
+    static std::mutex mu;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        hip_fail(fn, e);
+        return nullptr;
+    }
+    if (dev < 0 || dev >= kMaxScratchDevices) {
+        set_error("%s: device index %d outside 0..%d", fn, dev, kMaxScratchDevices - 1);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            hip_fail(fn, e != hipSuccess ? e : hipErrorInvalidSymbol);
+            return nullptr;
+        }
+        ptrs[dev] = p;
+    }
+    return ptrs[dev];
+}
+}  // namespace awq
+
+extern "C" size_t awq_gemv_static_scratch_bytes(void) { return awq::kStaticScratchBytes; }
+
+extern "C" int awq_gemv_static(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                               const void* bias, void* y, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                               int dtype, void* stream) {
+    const char* fn = "awq_gemv_static";
+    int v = 0, s = 1;
+    if (K >= 32 && N >= 8 && group_size > 0 && M >= 1) awq::pick_gemv(M, N, K, group_size, &v, &s);
+    const size_t need = (K >= 32 && N >= 8 && M >= 1) ? awq::gemv_ws_bytes(M, N, K, v, s) : 0;
+    if (need > awq::kStaticScratchBytes) {
+        awq::set_error("%s: M=%lld N=%lld K=%lld needs %zu bytes of split-K scratch, the static buffer holds %zu; "
+                       "use awq_gemv with a caller-provided workspace", fn, (long long)M, (long long)N, (long long)K,
+                       need, awq::kStaticScratchBytes);
+        return awq::fail_drop(AWQ_ERR_UNSUPPORTED);
+    }
+    void* ws = nullptr;
+    if (need > 0) {
+        ws = awq::static_scratch_ptr(fn);
+        if (!ws) return awq::fail_drop(AWQ_ERR_HIP);
+    }
+    return awq::gemv_dispatch(fn, x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, ws,
+                              need > 0 ? awq::kStaticScratchBytes : 0, stream, v, s);
 }
 
 extern "C" int awq_gemv(const void* x, const int32_t* qweight, const void* qscales,
