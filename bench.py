@@ -12,7 +12,7 @@ restatement of the reference path on the host cores, bounded sample), and -- as 
 headline -- the same GEMV on the Qwen3-32B MLP shapes where a launch is long enough to be HBM-bound,
 the prefill GEMM TFLOP/s at the Qwen3-8B MLP shapes, the dequantise kernel, and config 1's latency.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cfg5] [--no-cpu]
 """
 from __future__ import annotations
 
@@ -52,6 +52,29 @@ def rand_packed(K, N, tdt, dev, g=G):
     qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, device=dev)
     sc = (torch.rand(K // g, N, device=dev) * 0.02 + 0.001).to(tdt)
     return qw, sc, qz
+
+
+def decode_step_bytes(model, ctx_tokens):
+    """Algorithmic HBM bytes of one decode step: every packed AWQ buffer and the dense lm_head read once, plus the
+    K and V rows of `ctx_tokens` cached tokens (summed over the batch) in every layer."""
+    from nanoquantization_amd.layers.gemm import WQLinear_GEMM
+    wbytes = 0
+    for m in model.modules():
+        if isinstance(m, WQLinear_GEMM):
+            wbytes += m.qweight.numel() * 4 + m.qzeros.numel() * 4 + m.qscales.numel() * m.qscales.element_size()
+    head = model.lm_head.weight
+    a0 = model.model.layers[0].self_attn
+    kv = ctx_tokens * len(model.model.layers) * 2 * a0.num_kv_heads * a0.head_dim * head.element_size()
+    return {"awq_weights": wbytes, "lm_head": head.numel() * head.element_size(), "kv_cache": int(kv),
+            "total": int(wbytes + head.numel() * head.element_size() + kv)}
+
+
+def step_roofline(nbytes, ms_per_step, kernel):
+    gbs = nbytes["total"] / (ms_per_step * 1e-3) / 1e9
+    return {"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_step": nbytes,
+            "note": "whole decode step (all launches of the graph), not one kernel: packed weights + lm_head + cached "
+                    "K/V of the batch, each read once, / wall time per step"}
 
 
 def time_graph(fn, steps, warmup):
@@ -97,8 +120,8 @@ def main():
     ap.add_argument("--layers", type=int, default=64, help="distinct weight copies of one block per step")
     ap.add_argument("--quick", action="store_true", help="skip the extra (non-headline) measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--cfg5", action="store_true",
-                    help="also run the Qwen3-32B-architecture section (about 75 GB of device memory, a minute)")
+    ap.add_argument("--no-cfg5", action="store_true",
+                    help="skip the Qwen3-32B-architecture section (about 90 GB of device memory, a minute)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the AWQ linear path has no multi-GPU part); "
@@ -273,6 +296,9 @@ def main():
                 "prefill_s": round(st["prefill_s"], 4),
                 "prefill_tok_per_s": round(B * P / st["prefill_s"], 1),
                 "launches_per_block": 5 if eng.norm_fused_ok else 7,
+                "roofline": step_roofline(decode_step_bytes(model, B * (P + NEW // 2)),
+                                          st["decode_s"] / st["decode_steps"] * 1e3,
+                                          "decode step: awq::gemv_dma_kernel forms + awq::paged_attn_decode"),
             }
             # the same engine under continuous batching: ragged requests, rows and cache blocks recycled
             rg = torch.Generator().manual_seed(2)
@@ -298,36 +324,56 @@ def main():
         except Exception as e:  # the headline must still be printed
             out["e2e_qwen3_0p6b"] = {"error": repr(e)}
 
-    if args.cfg5:
-        # ---------------- extra: cfg5, Qwen3-32B architecture: batch-64 decode at 2048 context, 4096-token prefill
+    if not args.quick and not args.no_cfg5:
+        # ---------------- extra: cfg5, Qwen3-32B architecture: batch-64 decode at 2048 context with a 4096-token
+        # prefill admitted in between (one serve() call), then the steady decode step on its own
         try:
             from nanoquantization_amd.engine import LLMEngine
             from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
             cfg = dict(QWEN3_32B, max_position_embeddings=8192)
             model = random_awq_qwen3(cfg, seed=0, device=dev, dtype=torch.bfloat16)
-            B, P, NEW = 64, 2048, 17
-            eng = LLMEngine(model, max_batch=B, max_seq_len=P + 64, block_size=64, use_graph=True)
-            prompts = torch.randint(0, cfg["vocab_size"], (B, P), generator=torch.Generator().manual_seed(1)).tolist()
-            eng.generate(prompts, 4)
+            B, P, NEW, LONG = 64, 2048, 24, 4096
+            eng = LLMEngine(model, max_batch=B, max_seq_len=LONG + 64, block_size=64, use_graph=True)
+            rg = torch.Generator().manual_seed(1)
+            prompts = torch.randint(0, cfg["vocab_size"], (B, P), generator=rg).tolist()
+            long_prompt = torch.randint(0, cfg["vocab_size"], (LONG,), generator=rg).tolist()
+            eng.generate(prompts[:4], 3)                  # warm-up: graph capture, workspaces
+            eng.serve([(long_prompt, 2)])                 # warm-up of the long prefill's shapes
+            # mixed run: 64 requests at 2048 tokens fill the batch (prefilled four at a time); request 0 ends after
+            # 4 tokens, which frees a row for the 4096-token request: it is prefilled while 63 rows wait at a
+            # context of ~2052, then all 64 rows decode together
+            reqs = [(p, 4 if i == 0 else NEW) for i, p in enumerate(prompts)] + [(long_prompt, 12)]
+            sv = {}
+            eng.serve(reqs, stats=sv, batch_prefill=True, max_prefill_tokens=4 * P)
+            long_pf = [p for p in sv["prefill_log"] if p[0] == LONG]
             st = {}
-            eng.generate(prompts, NEW, stats=st)
-            del eng
-            torch.cuda.empty_cache()
-            eng1 = LLMEngine(model, max_batch=1, max_seq_len=4096 + 64, block_size=64, use_graph=False)
-            one = torch.randint(0, cfg["vocab_size"], (1, 4096), generator=torch.Generator().manual_seed(2)).tolist()
-            eng1.generate(one, 2)
-            st1 = {}
-            eng1.generate(one, 2, stats=st1)
+            eng.generate(prompts, 17, stats=st)           # the steady decode step alone, batch 64 at 2048..2064
+            ms_step = st["decode_s"] / st["decode_steps"] * 1e3
             out["cfg5_qwen3_32b"] = {
-                "workload": "Qwen3-32B architecture (64 layers, hidden 5120, 64 q / 8 kv heads, intermediate 25600), random AWQ "
-                            "g=128 weights, bf16: batch 64 decode at 2048 context; one 4096-token prefill",
+                "workload": "Qwen3-32B architecture (64 layers, hidden 5120, 64 q / 8 kv heads, intermediate 25600), random "
+                            "AWQ g=128 weights, bf16, paged KV (block 64).  mixed: one serve() of 64 requests x 2048-token "
+                            "prompts (24 new tokens; one of them 4) plus a 4096-token request admitted when the first row "
+                            "frees, i.e. prefilled between decode steps of the other 63 rows.  steady: generate() of 64 x "
+                            "2048 prompts, 16 timed decode steps",
+                "mixed": {
+                    "wall_s": round(sv["wall_s"], 3), "generated_tokens": sv["tokens"],
+                    "generated_tok_per_s": round(sv["tokens"] / sv["wall_s"], 1),
+                    "decode_steps": sv["decode_steps"], "decode_s": round(sv["decode_s"], 4),
+                    "decode_ms_per_step": round(sv["decode_s"] / max(1, sv["decode_steps"]) * 1e3, 2),
+                    "prefill_calls": sv["prefill_calls"], "prefill_s": round(sv["prefill_s"], 4),
+                    "batch_prefill_tok_per_s": round(sum(p[0] for p in sv["prefill_log"] if p[0] != LONG)
+                                                     / max(1e-9, sum(p[3] for p in sv["prefill_log"] if p[0] != LONG)), 1),
+                    "prefill_4096_s": round(long_pf[0][3], 4) if long_pf else None,
+                    "prefill_4096_tok_per_s": round(LONG / long_pf[0][3], 1) if long_pf else None,
+                    "prefill_4096_after_decode_steps": long_pf[0][2] if long_pf else None,
+                },
                 "decode_tok_per_s": round(B * st["decode_steps"] / st["decode_s"], 1),
-                "decode_ms_per_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 2),
-                "batch_prefill_tok_per_s": round(B * P / st["prefill_s"], 1),
-                "prefill_4096_s": round(st1["prefill_s"], 4),
-                "prefill_4096_tok_per_s": round(4096 / st1["prefill_s"], 1),
+                "decode_ms_per_step": round(ms_step, 2),
+                "roofline": step_roofline(decode_step_bytes(model, B * (P + 8)), ms_step,
+                                          "decode step: awq::gemv_wide_kernel / gemv_dma_kernel forms + "
+                                          "awq::paged_attn_decode_mfma_kernel"),
             }
-            del eng1, model
+            del eng, model
             torch.cuda.empty_cache()
         except Exception as e:
             out["cfg5_qwen3_32b"] = {"error": repr(e)}

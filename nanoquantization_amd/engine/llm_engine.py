@@ -362,6 +362,7 @@ class LLMEngine:
         self.s_active.zero_(); self.s_pos.zero_(); self.s_ids.zero_(); self.s_table.zero_(); self.s_step.zero_()
         torch.cuda.synchronize()
         t_start, n_steps, n_prefill, n_prefill_calls = time.perf_counter(), 0, 0, 0
+        prefill_log = []                  # per prefill pass: (prompt tokens, requests, decode steps so far, seconds)
 
         def retire(row):
             _, _, blocks = running.pop(row)
@@ -407,6 +408,9 @@ class LLMEngine:
                     admitted.append((ri, self.cache.allocate(need)))
                     tokens_admitted += len(prompt)
                 if admitted:
+                    if stats is not None:
+                        torch.cuda.synchronize()
+                        t_pf = time.perf_counter()
                     try:
                         if len(admitted) == 1:
                             ids = torch.tensor([requests[admitted[0][0]][0]], dtype=torch.long, device=self.device)
@@ -420,6 +424,8 @@ class LLMEngine:
                         raise
                     n_prefill += len(admitted)
                     n_prefill_calls += 1
+                    if stats is not None:       # toks.tolist() above has waited for the pass
+                        prefill_log.append((tokens_admitted, len(admitted), n_steps, time.perf_counter() - t_pf))
                     for (ri, blocks), tok in zip(admitted, toks):
                         prompt, max_new = requests[ri]
                         out[ri].append(tok)
@@ -454,7 +460,10 @@ class LLMEngine:
                 retire(row)
         if stats is not None:
             torch.cuda.synchronize()
-            stats.update(wall_s=time.perf_counter() - t_start, decode_steps=n_steps, prefills=n_prefill,
-                         prefill_calls=n_prefill_calls, tokens=sum(len(o) for o in out))
+            wall = time.perf_counter() - t_start
+            prefill_s = sum(p[3] for p in prefill_log)
+            stats.update(wall_s=wall, decode_steps=n_steps, prefills=n_prefill, prefill_calls=n_prefill_calls,
+                         tokens=sum(len(o) for o in out), prefill_s=prefill_s, decode_s=wall - prefill_s,
+                         prefill_log=prefill_log)
         return out
 
