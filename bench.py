@@ -133,7 +133,7 @@ def main():
 
     from nanoquantization_amd import _lib
     import nanoquantization_amd as nq
-    if not os.path.exists(_lib.LIB_PATH):
+    if not (os.path.exists(_lib.LIB_PATH) and os.path.exists(_lib.TORCH_LIB_PATH)):
         from nanoquantization_amd.build import build
         build(verbose=False)
     _lib.lib()

@@ -1,4 +1,6 @@
-"""ctypes binding of libawq_hip.so, the C ABI declared in include/awq_hip.h.
+"""Loaders of the two shared libraries: libawq_hip.so (the C ABI declared in include/awq_hip.h and
+include/nq_engine_ops.h, bound with ctypes) and libawq_torch.so (the PyTorch operator binding over that ABI for the
+linear path: torch.ops.nanoquantization_amd.*).
 
 There is no fallback: if the library is missing or a call fails, an exception
 is raised.
@@ -93,6 +95,27 @@ def lib() -> ctypes.CDLL:
                     fn.restype, fn.argtypes = res, args
                 _lib = handle
     return _lib
+
+
+TORCH_LIB_PATH = os.path.join(PKG_DIR, "libawq_torch.so")
+_torch_ops = None
+
+
+def torch_ops():
+    """torch.ops.nanoquantization_amd: the operators of csrc/torch_binding.cpp (awq_dequantize, awq_linear,
+    awq_linear_swiglu), registered with the dispatcher by loading libawq_torch.so.  Raises if it has not been built."""
+    global _torch_ops
+    if _torch_ops is None:
+        lib()                                           # libawq_hip.so first: the binding links against it
+        with _lock:
+            if _torch_ops is None:
+                if not os.path.exists(TORCH_LIB_PATH):
+                    raise AwqHipError(
+                        f"{TORCH_LIB_PATH} is missing: build it with `python -m nanoquantization_amd.build` "
+                        "(there is no CPU or eager fallback for the AWQ kernels)")
+                torch.ops.load_library(TORCH_LIB_PATH)
+                _torch_ops = torch.ops.nanoquantization_amd
+    return _torch_ops
 
 
 def check(status: int) -> None:

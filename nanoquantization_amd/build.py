@@ -1,4 +1,5 @@
-"""Builds csrc/*.hip into nanoquantization_amd/libawq_hip.so for gfx950.
+"""Builds csrc/*.hip into nanoquantization_amd/libawq_hip.so for gfx950, and csrc/torch_binding.cpp (host code
+only: the PyTorch operator registration over the C ABI) into nanoquantization_amd/libawq_torch.so.
 
 Usage: python -m nanoquantization_amd.build
 """
@@ -13,7 +14,11 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libawq_hip.so")
 
-HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+TORCH_LIB_PATH = os.path.join(PKG_DIR, "libawq_torch.so")
+
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.environ.get("HIPCC", os.path.join(ROCM, "bin", "hipcc"))
+CXX = os.environ.get("CXX", "g++")
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
@@ -66,8 +71,33 @@ def build(verbose: bool = True) -> str:
         jobs.append(([HIPCC, *compile_flags, *EXTRA.get(os.path.basename(src), []), "-c", src, "-o", obj], obj))
     with ThreadPoolExecutor(max_workers=min(4, len(jobs))) as pool:
         list(pool.map(lambda j: _run(j[0], verbose), jobs))
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *[o for _, o in jobs], "-o", LIB_PATH], verbose)
+    with ThreadPoolExecutor(max_workers=2) as pool:
+        # the operator binding has no device code: host compiler, torch headers; it only needs the C header
+        binding = pool.submit(_run, torch_binding_compile_cmd(os.path.join(objdir, "torch_binding.o")), verbose)
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *[o for _, o in jobs], "-o", LIB_PATH], verbose)
+        binding.result()
+    _run(torch_binding_link_cmd(os.path.join(objdir, "torch_binding.o")), verbose)
     return LIB_PATH
+
+
+def _torch_dirs():
+    import torch
+    root = os.path.dirname(torch.__file__)
+    return ([os.path.join(root, "include"), os.path.join(root, "include", "torch", "csrc", "api", "include")],
+            os.path.join(root, "lib"), int(torch._C._GLIBCXX_USE_CXX11_ABI))
+
+
+def torch_binding_compile_cmd(obj: str) -> list[str]:
+    incs, _, abi = _torch_dirs()
+    return [CXX, "-O2", "-fPIC", "-std=c++17", "-w", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+            f"-D_GLIBCXX_USE_CXX11_ABI={abi}", *[f"-I{i}" for i in incs], f"-I{ROCM}/include",
+            "-c", os.path.join(CSRC, "torch_binding.cpp"), "-o", obj]
+
+
+def torch_binding_link_cmd(obj: str) -> list[str]:
+    _, libdir, _ = _torch_dirs()
+    return [CXX, "-shared", "-fPIC", obj, "-o", TORCH_LIB_PATH, f"-L{libdir}", "-ltorch", "-ltorch_cpu", "-lc10",
+            "-lc10_hip", "-ltorch_hip", f"-L{PKG_DIR}", "-lawq_hip", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{libdir}"]
 
 
 if __name__ == "__main__":

@@ -58,15 +58,10 @@ def awq_dequantize(
     block_size_y: int = 32,
 ) -> torch.Tensor:
     """Packed int4 -> [K, N] weight in qscales.dtype, bit-exact RN((q - z) * s)."""
-    K, N, g = _check_packed(qweight, qscales, qzeros)
-    dev = _require_device(qweight, qscales, qzeros)
-    qweight, qscales, qzeros = qweight.contiguous(), qscales.contiguous(), qzeros.contiguous()
-    out = torch.empty(K, N, dtype=qscales.dtype, device=dev)
-    with _lib.on_device(dev):
-        stream = _lib.current_stream_ptr(dev)
-        _lib.check(_lib.lib().awq_dequantize(_ptr(qweight), _ptr(qscales), _ptr(qzeros), _ptr(out),
-                                             K, N, g, _lib.dtype_id(qscales.dtype), stream))
-    return out
+    _check_packed(qweight, qscales, qzeros)
+    _require_device(qweight, qscales, qzeros)
+    _lib.dtype_id(qscales.dtype)
+    return _lib.torch_ops().awq_dequantize(qweight, qscales, qzeros)
 
 
 def awq_dequantize_transposed(qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor) -> torch.Tensor:
@@ -139,7 +134,11 @@ def awq_gemm(
     their own K split (the reduction is in fp32 and in a fixed order).
     """
     assert split_k_iters & (split_k_iters - 1) == 0
-    return _linear("awq_linear", x, qweight, qscales, qzeros, None)
+    K, N, g = _check_packed(qweight, qscales, qzeros)
+    assert x.dim() == 2 and x.shape[1] == K
+    _require_device(x, qweight, qscales, qzeros)
+    _lib.dtype_id(qscales.dtype)
+    return _lib.torch_ops().awq_linear(x, qweight, qscales, qzeros, None)
 
 
 def awq_gemv_variant(x, qweight, qscales, qzeros, variant: int, split_k: int, bias=None):
@@ -150,6 +149,18 @@ def awq_gemv_variant(x, qweight, qscales, qzeros, variant: int, split_k: int, bi
 def awq_gemm_variant(x, qweight, qscales, qzeros, variant: int, split_k: int, bias=None):
     """Fused dequant+MFMA GEMM with a forced tile variant and K split (tuning / tests)."""
     return _linear("awq_gemm_ex", x, qweight, qscales, qzeros, bias, (variant, split_k))
+
+
+_AWQ_LINEAR_OP = None
+
+
+def _linear_op():
+    """torch.ops.nanoquantization_amd.awq_linear (argument checks, output allocation, workspace and the launch on
+    torch's current stream all happen in the C++ binding), looked up once."""
+    global _AWQ_LINEAR_OP
+    if _AWQ_LINEAR_OP is None:
+        _AWQ_LINEAR_OP = _lib.torch_ops().awq_linear.default
+    return _AWQ_LINEAR_OP
 
 
 def pack_awq(intweight: torch.Tensor) -> torch.Tensor:
@@ -257,11 +268,14 @@ class WQLinear_GEMM(nn.Module):
                 cached = (key, bias.to(buf["qscales"].dtype))
                 self.__dict__["_bias_cast"] = cached
             bias = cached[1]
+        if x.device.type != "cuda":
+            raise _lib.AwqHipError(
+                "AWQ kernels run on a HIP device only (tensor is on %s); there is no CPU fallback" % x.device)
+        op = _AWQ_LINEAR_OP or _linear_op()
         if x.dim() == 2:
-            return _linear("awq_linear", x, buf["qweight"], buf["qscales"], buf["qzeros"], bias)
+            return op(x, buf["qweight"], buf["qscales"], buf["qzeros"], bias)
         out_shape = x.shape[:-1] + (self.out_features,)
-        out = _linear("awq_linear", x.reshape(-1, x.shape[-1]), buf["qweight"], buf["qscales"], buf["qzeros"], bias)
-        return out.reshape(out_shape)
+        return op(x.reshape(-1, x.shape[-1]), buf["qweight"], buf["qscales"], buf["qzeros"], bias).reshape(out_shape)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
