@@ -229,6 +229,59 @@ __device__ __forceinline__ void compute_chunk_bytes(const Chunk<1, CH, MT>& d, f
     }
 }
 
+// compute_chunk for one word column and one m-tile, one 32-row step at a time: the same MFMA chains and the same
+// fold, so the same bits, but a caller can start on step 0 while the rows of steps 1..3 are still on their way.
+// d[2*b + h] is the running product of byte b's low (h = 0) / high (h = 1) nibble column, dones the row sums.
+struct StepAcc {
+    f32x4 d[8];
+    f32x4 dones;
+};
+__device__ __forceinline__ void step_acc_clear(StepAcc& a) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a.d[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    a.dones = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+template <typename T>
+__device__ __forceinline__ void compute_step(const uint32_t (&w)[8], u32x4 xa, StepAcc& a, const AndOr& emb_lo,
+                                             const AndOr& emb_hi) {
+    const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
+    a.dones = T::mfma16(xa, ones, a.dones);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        u32x4 flo, fhi;
+#pragma unroll
+        for (int rp = 0; rp < 4; ++rp) {
+            const uint32_t p = __builtin_amdgcn_perm(w[2 * rp + 1], w[2 * rp],
+                                                     0x0c000c00u | (uint32_t)b | ((4u + b) << 16));
+            flo[rp] = emb_lo(Embed<T>::pre_lo(p));
+            fhi[rp] = emb_hi(Embed<T>::pre_hi(p));
+        }
+        a.d[2 * b] = T::mfma16(xa, flo, a.d[2 * b]);
+        a.d[2 * b + 1] = T::mfma16(xa, fhi, a.d[2 * b + 1]);
+    }
+}
+// kFirst: acc is known to be zero (nothing was folded into it yet) and need not be live before this call
+template <typename T, bool kFirst = false>
+__device__ __forceinline__ void fold_steps(const StepAcc& a, uint32_t zw, u32x4 sv, f32x4 (&acc)[8]) {
+    constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int c = h ? kHiCol[b] : kLoCol[b];
+            const float mul = h ? Embed<T>::kMulHi : Embed<T>::kMulLo;
+            const float off = h ? Embed<T>::kOffHi : Embed<T>::kOffLo;
+            const float zf = (float)((zw >> nibble_shift(c)) & 0xFu) * mul + off;
+            const uint32_t pair = sv[c >> 1];
+            const float sc = T::to_f32((uint16_t)((c & 1) ? (pair >> 16) : (pair & 0xFFFFu))) * (1.f / mul);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float t = sc * (a.d[2 * b + h][r] - zf * a.dones[r]);
+                acc[c][r] = kFirst ? 0.f + t : acc[c][r] + t;   // 0 + t: the bits of the running sum (a -0 becomes +0)
+            }
+        }
+}
+
 // A workgroup is WN x WK waves: wave w works on column tile (group*WN + w % WN)
 // and K sub-slice w / WN.  Sum the WK waves of each column tile through LDS
 // (fixed order), then either store y (splits == 1) or publish this split's
@@ -703,7 +756,9 @@ struct GemvExtra<kModeQkv | kModeNorm> { QkvEpilogue qe; NormPrologue np; };
 template <>
 struct GemvExtra<kModeResid> { ResidEpilogue re; };
 
-template <typename T, int WK, int MODE = 0>
+// STREAM: every wave has at most one chunk (decode-size launches) and takes it step by step as it lands; a form of
+// its own because it needs a dozen registers more than the 128 that let four waves of the other form share a SIMD.
+template <typename T, int WK, int MODE = 0, bool STREAM = false>
 __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
@@ -794,18 +849,27 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const bool zs_lane = lane < 16;
     const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
 
+    // Order of the loads of a chunk: the weights of steps 0..3 (two loads each), x, the zero words and the scales.
+    // The step-by-step form consumes them as they land and wants x first: one load for all four steps with at most 4
+    // rows, else one per step in front of that step's weights (on multi-chunk launches that order measured 7 % slower
+    // at 16 rows).
     auto issue_dma = [&](int c) {
         const int row0 = c * 128;
         uint32_t* w_lds = reinterpret_cast<uint32_t*>(stage);
+        if (STREAM && x_few && x_lane)
+            __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + row0 + xsrc), AWQ_LPTR(stage + x_off), 16, 0, 0);
 #pragma unroll
         for (int s = 0; s < CH; ++s) {
+            if (STREAM && !x_few && x_lane)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc),
+                                                 AWQ_LPTR(stage + x_off + s * 64 * M), 16, 0, 0);
             const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
 #pragma unroll
             for (int h = 0; h < 2; ++h)
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
                                                  16, 0, 0);
         }
-        if (x_lane) {
+        if (!STREAM && x_lane) {
             if (x_few) {
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + row0 + xsrc), AWQ_LPTR(stage + x_off), 16, 0, 0);
             } else {
@@ -832,8 +896,6 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const int s_rd_off = zs_off + 64 + j * 16;
 
     f32x4 acc[1][8];
-#pragma unroll
-    for (int f = 0; f < 8; ++f) acc[0][f] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     float rstd = 0.f;
     if constexpr (NORM) {   // the lane's row: 1 / rms from the tile sums, added in tile order (eight loads in flight)
@@ -851,7 +913,54 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     } else {
         if (c0 < c1) issue_dma(c0);
     }
-    for (int c = c0; c < c1; ++c) {
+    static_assert(!(STREAM && NORM), "the step-by-step form has no RMSNorm prologue");
+    int c_first = c0;
+    if constexpr (STREAM) {
+        // A wave with a single chunk (a decode-size launch: the chunk is all there is, and the loads of the eight
+        // waves of a workgroup queue up behind each other) takes it step by step as its rows land: wait for the
+        // loads of step s only -- outstanding loads are counted in issue order --, read its operands, multiply.
+        // With more chunks the next one is fetched while a whole chunk is multiplied, below.
+        if (c0 < c1) {   // the host launches this form only where a wave has one chunk at most
+            const AndOr emb_lo(Embed<T>::kMaskLo, Embed<T>::kMagicLo), emb_hi(Embed<T>::kMaskHi, Embed<T>::kMagicHi);
+            StepAcc sa;
+            step_acc_clear(sa);
+            uint32_t zw = 0;
+            u32x4 sv = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int s = 0; s < CH; ++s) {
+                // loads still allowed in flight: the later steps' (2 each, 3 with an x load per step) and zeros/scales
+                if (x_few) {
+                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
+                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+                } else {
+                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | 11);
+                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | 5);
+                }
+                if (s == 3) __builtin_amdgcn_s_waitcnt(0x0F70);
+                asm volatile("" ::: "memory");
+                uint32_t w[8];
+#pragma unroll
+                for (int r = 0; r < 8; ++r) w[r] = w_rd[s * 512 + r * 64];
+                const u32x4 xa = *reinterpret_cast<const u32x4*>(stage + x_rd_off + s * x_rd_step);
+                if (s == 3) {
+                    zw = *reinterpret_cast<const uint32_t*>(stage + z_rd_off);
+                    sv = *reinterpret_cast<const u32x4*>(stage + s_rd_off);
+                }
+                compute_step<T>(w, xa, sa, emb_lo, emb_hi);
+            }
+            fold_steps<T, true>(sa, zw, sv, acc[0]);
+            c_first = c1;
+        } else {
+#pragma unroll
+            for (int f = 0; f < 8; ++f) acc[0][f] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    } else {
+#pragma unroll
+        for (int f = 0; f < 8; ++f) acc[0][f] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int c = STREAM ? c1 : c_first; c < c1; ++c) {
         u32x4 nw[CH];
         if constexpr (NORM) {
 #pragma unroll
@@ -1194,7 +1303,10 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
                                    reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeQkv>),
                                    reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeNorm>),
                                    reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeQkv | kModeNorm>),
-                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeResid>)};
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeResid>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, 0, true>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeQkv, true>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeResid, true>)};
             for (const void* f : forms) {
                 hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
                 if (e != hipSuccess) return e;
@@ -1217,8 +1329,16 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
         pf.count = 0;
     }
     const dim3 grid(groups + pf_wgs, splits, row_blocks), block(64 * WK);
+    const bool stream_form = cps <= WK;   // one chunk per wave at most
 #define AWQ_DMA_LAUNCH(MODE, EXTRA)                                                                                \
-    hipLaunchKernelGGL((gemv_dma_kernel<T, WK, MODE>), grid, block, lds, stream,                                  \
+    AWQ_DMA_LAUNCH_FORM(MODE, false, EXTRA)
+#define AWQ_DMA_LAUNCH_S(MODE, EXTRA)                                                                              \
+    do {                                                                                                           \
+        if (stream_form) AWQ_DMA_LAUNCH_FORM(MODE, true, EXTRA);                                                   \
+        else AWQ_DMA_LAUNCH_FORM(MODE, false, EXTRA);                                                              \
+    } while (0)
+#define AWQ_DMA_LAUNCH_FORM(MODE, STREAMED, EXTRA)                                                                 \
+    hipLaunchKernelGGL((gemv_dma_kernel<T, WK, MODE, STREAMED>), grid, block, lds, stream,                        \
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),          \
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),     \
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters, \
@@ -1226,14 +1346,16 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     if (fu.qe && fu.np)
         AWQ_DMA_LAUNCH(kModeQkv | kModeNorm, (GemvExtra<kModeQkv | kModeNorm>{*fu.qe, *fu.np}));
     else if (fu.qe)
-        AWQ_DMA_LAUNCH(kModeQkv, (GemvExtra<kModeQkv>{*fu.qe}));
+        AWQ_DMA_LAUNCH_S(kModeQkv, (GemvExtra<kModeQkv>{*fu.qe}));
     else if (fu.np)
         AWQ_DMA_LAUNCH(kModeNorm, (GemvExtra<kModeNorm>{*fu.np}));
     else if (fu.re)
-        AWQ_DMA_LAUNCH(kModeResid, (GemvExtra<kModeResid>{*fu.re}));
+        AWQ_DMA_LAUNCH_S(kModeResid, (GemvExtra<kModeResid>{*fu.re}));
     else
-        AWQ_DMA_LAUNCH(0, (GemvExtra<0>{}));
+        AWQ_DMA_LAUNCH_S(0, (GemvExtra<0>{}));
 #undef AWQ_DMA_LAUNCH
+#undef AWQ_DMA_LAUNCH_S
+#undef AWQ_DMA_LAUNCH_FORM
     return hipGetLastError();
 }
 
