@@ -236,16 +236,13 @@ struct StepAcc {
     f32x4 d[8];
     f32x4 dones;
 };
-__device__ __forceinline__ void step_acc_clear(StepAcc& a) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) a.d[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    a.dones = f32x4{0.f, 0.f, 0.f, 0.f};
-}
-template <typename T>
+// kFirst: the first step of a chunk; the MFMAs start from a literal zero, so `a` need not be cleared
+template <typename T, bool kFirst = false>
 __device__ __forceinline__ void compute_step(const uint32_t (&w)[8], u32x4 xa, StepAcc& a, const AndOr& emb_lo,
                                              const AndOr& emb_hi) {
     const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
-    a.dones = T::mfma16(xa, ones, a.dones);
+    const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+    a.dones = T::mfma16(xa, ones, kFirst ? zero4 : a.dones);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
         u32x4 flo, fhi;
@@ -256,8 +253,8 @@ __device__ __forceinline__ void compute_step(const uint32_t (&w)[8], u32x4 xa, S
             flo[rp] = emb_lo(Embed<T>::pre_lo(p));
             fhi[rp] = emb_hi(Embed<T>::pre_hi(p));
         }
-        a.d[2 * b] = T::mfma16(xa, flo, a.d[2 * b]);
-        a.d[2 * b + 1] = T::mfma16(xa, fhi, a.d[2 * b + 1]);
+        a.d[2 * b] = T::mfma16(xa, flo, kFirst ? zero4 : a.d[2 * b]);
+        a.d[2 * b + 1] = T::mfma16(xa, fhi, kFirst ? zero4 : a.d[2 * b + 1]);
     }
 }
 // kFirst: acc is known to be zero (nothing was folded into it yet) and need not be live before this call
@@ -772,6 +769,11 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     // decode-size launch, 2.8 x on a kernel that lives on 16-byte LDS reads)
     extern __shared__ __attribute__((aligned(16))) float red[];  // staging while streaming, [WK][32][64] floats afterwards
     __shared__ int s_last;
+    // Every argument the compute path needs, fetched now in one batch of scalar loads: left alone the compiler
+    // fetches them where they are first used, three round trips to the kernel-argument segment one behind the other
+    // in front of the first weight load.
+    asm volatile("" ::"s"(x), "s"(qweight), "s"(scales), "s"(qzeros), "s"(y), "s"(partials), "s"(counters), "s"(M),
+                 "s"(N), "s"(K), "s"(chunks_per_group), "s"(chunks_per_split), "s"(splits), "s"(groups));
     if ((int)blockIdx.x >= groups) {
         if (blockIdx.y != 0 || blockIdx.z != 0) return;   // the extra workgroups exist once per split and row block; one set works
         // Prefetch workgroups (launched beside the compute grid on CUs a small GEMV leaves idle): touch one
@@ -923,7 +925,6 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
         if (c0 < c1) {   // the host launches this form only where a wave has one chunk at most
             const AndOr emb_lo(Embed<T>::kMaskLo, Embed<T>::kMagicLo), emb_hi(Embed<T>::kMaskHi, Embed<T>::kMagicHi);
             StepAcc sa;
-            step_acc_clear(sa);
             uint32_t zw = 0;
             u32x4 sv = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
@@ -948,7 +949,8 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
                     zw = *reinterpret_cast<const uint32_t*>(stage + z_rd_off);
                     sv = *reinterpret_cast<const u32x4*>(stage + s_rd_off);
                 }
-                compute_step<T>(w, xa, sa, emb_lo, emb_hi);
+                if (s == 0) compute_step<T, true>(w, xa, sa, emb_lo, emb_hi);
+                else compute_step<T>(w, xa, sa, emb_lo, emb_hi);
             }
             fold_steps<T, true>(sa, zw, sv, acc[0]);
             c_first = c1;
