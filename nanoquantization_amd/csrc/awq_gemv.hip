@@ -1451,8 +1451,9 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             v = kDma1x8;
         } else if (M <= 4) {
             s = cdiv(3072, tiles * 4);
-            // short K: at most 10 splits (the tail is a larger share of a 6 us launch); long K: up to 32
-            const int64_t cap = chunks < 64 ? (chunks / 2 < 10 ? chunks / 2 : 10) : 32;
+            // short K: one chunk per wave (the step-by-step form), at most 10 splits (the tail is a larger share of
+            // a 6 us launch: 2048 x 1024 at one row 5.55 us in 8 splits, 5.23 in 4); long K: up to 32
+            const int64_t cap = chunks < 64 ? (chunks / 4 < 10 ? chunks / 4 : 10) : 32;
             if (s > cap) s = cap;
             s = balance_splits(chunks, s, 4, cap);
         } else {
