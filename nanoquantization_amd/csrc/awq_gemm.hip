@@ -291,6 +291,19 @@ static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_
         }
         if (best_s > 1 && best_t * 10 <= steps * 9) v = kPipeTailVariant, s = best_s;
     }
+    if (v != kPipe8 && v != kPipeTailVariant) {
+        // Narrow tiles (up to 128 rows): two workgroups of the 128x128 and 32x256 forms share a CU, one of the 64x256
+        // form.  Workgroups run in rounds of that many; a round lasts one split's K steps plus about six steps of
+        // prologue and partial store.  Take the split count with the least rounds x length (5120 x 25600 at 128
+        // rows: 200 tiles unsplit 102 us, two splits 74 us, three -- 600 workgroups, a second, short round -- 93 us).
+        const int64_t slots = v == k64x256 ? kCUs : 2 * kCUs, steps = K / kBK;
+        const int64_t hi = max_s < 16 ? max_s : 16;
+        int64_t best_t = -1;
+        for (int64_t c = 1; c <= hi; ++c) {
+            const int64_t t = cdiv(tiles * c, slots) * (cdiv(steps, c) + 6);
+            if (best_t < 0 || t < best_t) best_t = t, s = c;
+        }
+    }
     if (s > max_s) s = max_s;
     if (s > 16) s = 16;
     if (s < 1) s = 1;
