@@ -187,6 +187,15 @@ def test_dispatch_plans_are_consistent():
     assert rc == 0 and gemv_names[v] == "dma1x4" and s >= 3
     wgs = 34816 // 128 * s
     assert wgs / (256 * -(-wgs // 256)) >= 0.8
+    # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
+    # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
+    rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120)
+    assert rc == 0 and gemm_names[v] == "128x128" and s in (2, 5), s
+    rc, v, s = _plan(L.awq_gemm_plan, 96, 5120, 25600)     # 40 tiles, 400 K steps: about 12 splits, one round
+    assert rc == 0 and gemm_names[v] == "128x128" and 40 * s <= 512 and s >= 8, s
+    # GEMV at up to four rows on a short K: one 128-row chunk per wave of the four-wave workgroups
+    rc, v, s = _plan(L.awq_gemv_plan, 1, 1024, 2048, 128)
+    assert rc == 0 and gemv_names[v] == "dma1x4" and s == 4, (gemv_names[v], s)
     # shapes awq_gemv does not take are refused by the plan as well
     assert _plan(L.awq_gemv_plan, 65, 1024, 1024, 128)[0] != 0
     assert _plan(L.awq_gemv_plan, 4, 1024, 1000, 128)[0] != 0
