@@ -761,7 +761,7 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split,
-    int splits, int act, int groups, PrefetchRegions pf, GemvExtra<MODE> ex) {
+    int splits, int act, int groups, int pair_map, PrefetchRegions pf, GemvExtra<MODE> ex) {
     constexpr bool QKV = (MODE & kModeQkv) != 0, NORM = (MODE & kModeNorm) != 0, RESID = (MODE & kModeResid) != 0;
     constexpr int CH = 4;
     // 16-byte aligned: the dynamic segment starts behind the static one (s_last, 4 bytes), and at the array's
@@ -774,13 +774,27 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     // in front of the first weight load.
     asm volatile("" ::"s"(x), "s"(qweight), "s"(scales), "s"(qzeros), "s"(y), "s"(partials), "s"(counters), "s"(M),
                  "s"(N), "s"(K), "s"(chunks_per_group), "s"(chunks_per_split), "s"(splits), "s"(groups));
-    if ((int)blockIdx.x >= groups) {
+    // Which column tile this workgroup owns.  Workgroups go to the 8 XCDs by linear index mod 8, and two neighbouring
+    // tiles share every 128-byte line of the weights (a tile's row piece is 64 bytes): the two must sit behind the
+    // same L2, or each line is fetched from the fabric twice.  With a multiple of 16 tiles every XCD gets a run of
+    // consecutive tiles.  Otherwise (8 or 24 tiles on the decode shapes) the grid is padded to a multiple of 16 and
+    // dealt in pairs: workgroups x and x + 8 (same XCD) own tiles 2p and 2p + 1 of pair p = 8 * (slot / 2) + x % 8;
+    // the indices past the last tile are the spare workgroups.
+    int tile_of_wg;
+    if (pair_map) {
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        tile_of_wg = 2 * ((slot >> 1) * 8 + xcd) + (slot & 1);
+    } else {
+        tile_of_wg = (int)blockIdx.x < groups ? xcd_aware_group(blockIdx.x, groups) : (int)blockIdx.x;
+    }
+    if (tile_of_wg >= groups) {
         if (blockIdx.y != 0 || blockIdx.z != 0) return;   // the extra workgroups exist once per split and row block; one set works
         // Prefetch workgroups (launched beside the compute grid on CUs a small GEMV leaves idle): touch one
         // dword of every 128-byte line of the hinted regions -- the packed weights, scales and zeros of the
         // NEXT launch -- so that it finds them in the Infinity Cache instead of HBM.
+        if (pf.count == 0) return;
         const long long nthreads = (long long)(gridDim.x - groups) * blockDim.x;
-        const long long tid = (long long)(blockIdx.x - groups) * blockDim.x + threadIdx.x;
+        const long long tid = (long long)(tile_of_wg - groups) * blockDim.x + threadIdx.x;
         uint32_t sink = 0;
         for (int r = 0; r < pf.count; ++r) {
             const long long lines = pf.bytes[r] >> 7;
@@ -821,7 +835,7 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
-    const int tile = xcd_aware_group(blockIdx.x, groups), split = blockIdx.y;   // host guarantees N % 128 == 0
+    const int tile = tile_of_wg, split = blockIdx.y;   // host guarantees N % 128 == 0
 
     const int total_chunks = K / 128;
     const int c_begin = split * chunks_per_split;
@@ -1330,7 +1344,14 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     } else {
         pf.count = 0;
     }
-    const dim3 grid(groups + pf_wgs, splits, row_blocks), block(64 * WK);
+    // tiles in pairs per XCD on the narrow weights of decode-size launches, where the other mapping leaves the two
+    // halves of every line to two XCDs (8 or 24 tiles; fetch from the fabric per launch of the Qwen3-0.6B sweep
+    // 3.1 -> 2.3 MB, 6.0 -> 5.7 us).  Wide weights keep runs of consecutive tiles per XCD: pairs dealt round-robin
+    // measured slower there (40 tiles x 200 chunks at 16 rows 26.5 -> 39.4 us).
+    const int pair_map = (groups % 16 != 0 && groups >= 2 && groups <= 24) ? 1 : 0;
+    int grid_x = groups + pf_wgs;
+    if (pair_map) grid_x = (int)cdiv(grid_x, 16) * 16;
+    const dim3 grid(grid_x, splits, row_blocks), block(64 * WK);
     const bool stream_form = cps <= WK;   // one chunk per wave at most
 #define AWQ_DMA_LAUNCH(MODE, EXTRA)                                                                                \
     AWQ_DMA_LAUNCH_FORM(MODE, false, EXTRA)
@@ -1344,7 +1365,7 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),          \
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),     \
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters, \
-                       M, N, K, g / 128, cps, splits, act, groups, pf, EXTRA)
+                       M, N, K, g / 128, cps, splits, act, groups, pair_map, pf, EXTRA)
     if (fu.qe && fu.np)
         AWQ_DMA_LAUNCH(kModeQkv | kModeNorm, (GemvExtra<kModeQkv | kModeNorm>{*fu.qe, *fu.np}));
     else if (fu.qe)
