@@ -12,7 +12,7 @@ restatement of the reference path on the host cores, bounded sample), and -- as 
 headline -- the same GEMV on the Qwen3-32B MLP shapes where a launch is long enough to be HBM-bound,
 the prefill GEMM TFLOP/s at the Qwen3-8B MLP shapes, the dequantise kernel, and config 1's latency.
 
-python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cfg5] [--no-cpu]
+python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cfg5] [--only-cfg5] [--no-cpu]
 """
 from __future__ import annotations
 
@@ -120,6 +120,8 @@ def main():
     ap.add_argument("--layers", type=int, default=64, help="distinct weight copies of one block per step")
     ap.add_argument("--quick", action="store_true", help="skip the extra (non-headline) measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only-cfg5", action="store_true",
+                    help="with the headline, run only the Qwen3-32B-architecture section of the extra measurements")
     ap.add_argument("--no-cfg5", action="store_true",
                     help="skip the Qwen3-32B-architecture section (about 90 GB of device memory, a minute)")
     args = ap.parse_args()
@@ -213,7 +215,7 @@ def main():
         "per_shape_hot_cache": per_shape,
     }
 
-    if not args.quick:
+    if not args.quick and not args.only_cfg5:
         # ---------------- extra: HBM-bound GEMV at the Qwen3-32B MLP shapes -----------------------------
         large, batched = {}, {}
         for (K, N) in ((5120, 25600), (25600, 5120)):
@@ -276,7 +278,7 @@ def main():
         out["cfg1_single_linear"] = {"shape": "x[16,1024] @ W[1024,3072]", "graph_us": round(time_graph(fn, 5, 1) * 1e3 / 50, 2),
                                      "eager_us": round(time_eager(lambda: nq.awq_gemm(x, *w, 8), 200, 20) * 1e3, 2)}
 
-    if not args.quick:
+    if not args.quick and not args.only_cfg5:
         # ---------------- extra: cfg4, end-to-end Qwen3-0.6B-architecture decode ------------------------
         try:
             from nanoquantization_amd.engine import LLMEngine
