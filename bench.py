@@ -29,10 +29,10 @@ sys.path.insert(0, ROOT)
 
 # HBM bytes per GEMV launch of the headline sweep, from two `rocprofv3 --pmc` runs of this file
 # (FETCH_SIZE, then WRITE_SIZE; profiles/gemv_cfg2_sweep_hbm_traffic.txt).  Each counter is scaled by
-# what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,014 -> 2047 B per count,
+# what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,011.5 -> 2047.3 B per count,
 # WRITE_SIZE 64,000 -> 1024 B per count.
-MEASURED_FETCH_BYTES_PER_LAUNCH = 1511.6 * 2047.2
-MEASURED_WRITE_BYTES_PER_LAUNCH = 108.9 * 1024.0
+MEASURED_FETCH_BYTES_PER_LAUNCH = 1130.85 * 2047.3
+MEASURED_WRITE_BYTES_PER_LAUNCH = 100.68 * 1024.0
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16, published
@@ -168,19 +168,17 @@ def main():
     avg_launch_us = ms_graph * 1e3 / launches_per_step
     avg_bytes = bytes_per_step / launches_per_step
     roofline = {
-        "kernel": "awq::gemv_dma_kernel<F16, WK=4|8>", "bound": "hbm",
+        "kernel": "awq::gemv_dma_kernel<F16, WK=4|8, plain, one chunk per wave>", "bound": "hbm",
         "achieved": avg_bytes / (avg_launch_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "traffic": MEASURED_FETCH_BYTES_PER_LAUNCH + MEASURED_WRITE_BYTES_PER_LAUNCH,
-        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 3.10 MB + write 0.11 MB) from rocprofv3 "
+        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 2.32 MB + write 0.10 MB) from rocprofv3 "
                         "FETCH_SIZE / WRITE_SIZE, copy-calibrated.  The counters sit between the L2s and the fabric "
-                        "and cannot tell Infinity Cache hits from HBM reads: 0.87 MB of the fetch is the prefetch "
+                        "and cannot tell Infinity Cache hits from HBM reads: about 0.87 MB of the fetch is the prefetch "
                         "(spare workgroups read the next launch's weights once to park them in the Infinity Cache, "
-                        "the consumer reads them again from there); without the prefetch the fetch is 2.18 MB "
-                        "against 1.17 MB of packed weights, because a workgroup reads 64-byte row pieces and, with "
-                        "only 8-24 column tiles, the other half of a 128-byte line is often fetched again by another "
-                        "XCD's L2; the writes are split-K partials.  These launches are latency-bound (variants "
-                        "without the re-fetch are 15-25 % slower); at the 68 MB shapes fetch = 1.05 x algorithmic",
+                        "the consumer reads them again from there); the remaining 1.45 MB is 1.24 x the packed "
+                        "weights (x, scales, zeros per workgroup; lines shared across XCDs on the 16-tile shape); "
+                        "the writes are split-K partials.  At the 68 MB shapes fetch = 1.05 x algorithmic",
         "avg_launch_us": avg_launch_us, "algorithmic_bytes_per_launch": avg_bytes,
         "note": "packed-weight bytes (0.5195 B/weight) / HIP-event time per launch over the timed graph replays; "
                 "0.5-1.6 MB per launch: latency-bound, see roofline_large for the HBM-bound regime",
