@@ -76,10 +76,10 @@ size_t awq_gemv_workspace_bytes(int64_t M, int64_t N, int64_t K);
 size_t awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
-/* Decode regime, 1 <= M <= 16 (up to 64 rows where N % 128 == 0 and group_size % 128 == 0: batched
- * decode): y = x @ dequant(W) (+ bias), fp32 accumulation, split-K with a fixed-order (run-to-run
- * bit-stable) reduction, inside the kernel or, for 17..64 rows on the largest weights, as a second
- * kernel on the same stream.
+/* Decode regime, 1 <= M <= 16 (up to 128 rows where N % 128 == 0 and group_size % 128 == 0: batched
+ * decode, as blocks of 16 rows): y = x @ dequant(W) (+ bias), fp32 accumulation, split-K with a
+ * fixed-order (run-to-run bit-stable) reduction, inside the kernel or, for 17..64 rows on the largest
+ * weights, as a second kernel on the same stream.
  * Replaces awq_gemm(x, qweight, qscales, qzeros, split_k_iters) for small M:
  * nanoquantization/layers/gemm.py:329-379 (kernel :183-326, torch.zeros :361,
  * out.sum :378). */
@@ -192,7 +192,8 @@ int awq_gemm(const void* x, const int32_t* qweight, const void* qscales, const i
              int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The whole forward of one AWQ linear: picks the regime from M (awq_gemv for
- * M <= 16, and up to 64 where it takes the shape, awq_gemm above) and applies the bias.
+ * M <= 16, up to 64 where it takes the shape, and up to 128 on weights of at most 20 Mi elements;
+ * awq_gemm above) and applies the bias.
  * A K that is a multiple of 32 but not of 64 (which awq_gemm does not take) is served by
  * awq_gemv in blocks of 16 rows.  Replaces WQLinear_GEMM.forward, nanoquantization/layers/gemm.py:552-567
  * (the reshape of x/y to 2-D stays with the caller). */

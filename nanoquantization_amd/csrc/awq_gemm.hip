@@ -447,9 +447,14 @@ extern "C" int awq_gemm(const void* x, const int32_t* qweight, const void* qscal
                               dtype, workspace, workspace_bytes, stream, v, s);
 }
 
+// 65..128 rows go to the GEMV (blocks of 16 rows) on weights up to this size, see kGemvMaxRows in awq_gemv.hip
+static bool gemv_rows_ok(int64_t M, int64_t N, int64_t K) {
+    return M <= 64 || (M <= 128 && K * N <= (20ll << 20));
+}
+
 extern "C" size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     // the regime depends on the group size, which this query does not get: cover both
-    size_t a = M <= 64 ? awq_gemv_workspace_bytes(M, N, K) : 0;
+    size_t a = gemv_rows_ok(M, N, K) ? awq_gemv_workspace_bytes(M, N, K) : 0;
     const size_t b = M > 16 ? awq_gemm_workspace_bytes(M, N, K) : 0;
     if (M > 16 && K % awq::kBK != 0) {   // served by the GEMV in blocks of 16 rows
         const size_t c = awq_gemv_workspace_bytes(16, N, K);
@@ -485,9 +490,9 @@ extern "C" int awq_linear(const void* x, const int32_t* qweight, const void* qsc
                           const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                           int64_t K, int64_t group_size, int dtype, void* workspace,
                           size_t workspace_bytes, void* stream) {
-    // decode regime: up to 16 rows on any GEMV path, up to 64 on the staged one
+    // decode regime: up to 16 rows on any GEMV path, up to 64 on the staged one (128 on small weights)
     const bool staged = N % 128 == 0 && group_size > 0 && group_size % 128 == 0;
-    if (M >= 1 && ((M <= 16 && group_size % 32 == 0) || (M <= 64 && staged)))
+    if (M >= 1 && ((M <= 16 && group_size % 32 == 0) || (gemv_rows_ok(M, N, K) && staged)))
         return awq_gemv(x, qweight, qscales, qzeros, bias, y, M, N, K, group_size, dtype, workspace,
                         workspace_bytes, stream);
     if (M > 16 && K % awq::kBK != 0 && K % 32 == 0 && group_size > 0 && group_size % 32 == 0 && K % group_size == 0 &&

@@ -1255,6 +1255,11 @@ enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = kDma1x4;
 
+// Rows the staged kernels take as blocks of 16 (grid z).  awq_linear sends 65..128 rows here only on small weights
+// (kGemvWideRowsMaxWeights), where eight blocks re-reading the weights from cache beat the narrow-tile MFMA GEMM by 2 x
+// (1024 x 3072 at 128 rows: 8.2 against 17.5 us; 4096 x 4096: 14.8 against 23.0; equal from about 25 M weights on).
+constexpr int kGemvMaxRows = 128;
+
 // rows per chunk: 128 when the group size allows it, else 32
 static inline int chunk_steps(int64_t g) { return g % 128 == 0 ? 4 : 1; }
 
@@ -1459,7 +1464,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int v = kDma1x4;
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
-        if (allow_shared_chunk && M > 16 && N % 512 == 0 && N >= 5120 &&
+        if (allow_shared_chunk && M > 16 && M <= 64 && N % 512 == 0 && N >= 5120 &&
             K * N >= (M > 48 ? (50ll << 20) : (M > 32 ? 64000000ll : 95000000ll))) {
             // 17..64 rows on the largest weights (from sweeps: the fused gate|up of Qwen3-8B and the MLP of
             // Qwen3-14B/32B and, above 32 rows, the 32B fused q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
@@ -1485,7 +1490,9 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             // (publish, fetch, add) that grows with the rows of a block, hence the penalty: at 5120 x 25600 five
             // splits win at 8 rows (22.9 against 24.4 us) and lose at 16 (27.4 against 24.7).
             const int64_t wgs = tiles * row_blocks;
-            const int64_t cap = chunks / 4 > 1 ? chunks / 4 : 1;
+            // 65..128 rows (five to eight blocks of 16, small weights only): the blocks fill the chip, a split only
+            // adds its tail (2048 x 2048 at 128 rows: 8.6 us unsplit, 9.4 in two)
+            const int64_t cap = M > 64 && wgs >= 64 ? 1 : (chunks / 4 > 1 ? chunks / 4 : 1);
             int64_t s0 = wgs < 200 ? cdiv(200, wgs) : 1;
             if (s0 > cap) s0 = cap;
             const int64_t hi = s0 + 5 < cap ? s0 + 5 : cap;
@@ -1545,8 +1552,8 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                   "staged kernels only (N %% 128 == 0, group_size %% 128 == 0)", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
-    if (M > 64) {
-        set_error("%s: M=%lld is outside the decode regime (1..64); use awq_gemm", fn, (long long)M);
+    if (M > kGemvMaxRows) {
+        set_error("%s: M=%lld is outside the decode regime (1..%d); use awq_gemm", fn, (long long)M, kGemvMaxRows);
         return AWQ_ERR_UNSUPPORTED;
     }
     if (g % 32 != 0 || K % 32 != 0) {
@@ -1636,7 +1643,7 @@ extern "C" const char* awq_gemv_variant_name(int variant) {
 }
 
 extern "C" int awq_gemv_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, int* variant, int* split_k) {
-    if (!variant || !split_k || M < 1 || M > 64 || N < 8 || N % 8 != 0 || K < 32 || group_size < 32 ||
+    if (!variant || !split_k || M < 1 || M > awq::kGemvMaxRows || N < 8 || N % 8 != 0 || K < 32 || group_size < 32 ||
         group_size % 32 != 0 || K % group_size != 0) {
         awq::set_error("awq_gemv_plan: not a shape awq_gemv takes (M=%lld N=%lld K=%lld g=%lld)", (long long)M,
                        (long long)N, (long long)K, (long long)group_size);

@@ -189,7 +189,7 @@ def test_gemv_errors():
     with pytest.raises(_lib.AwqHipError, match="takes at most 16 rows"):
         awq_gemv_variant(x, *dev, 0, 1)
     with pytest.raises(_lib.AwqHipError, match="decode regime"):
-        awq_gemv_variant(torch.zeros(65, 256, dtype=torch.float16, device="cuda"), *dev, 0, 1)
+        awq_gemv_variant(torch.zeros(129, 256, dtype=torch.float16, device="cuda"), *dev, 0, 1)
     with pytest.raises(AssertionError):
         nq.awq_gemm(x[:, :128], *dev, 8)
     with pytest.raises(AssertionError):
@@ -222,3 +222,21 @@ def test_prefetch_hint_never_changes_results():
     assert L.awq_prefetch_hint(buf.data_ptr(), 1024) == 0           # a fifth region is ignored, not an error
     assert L.awq_prefetch_pending() == 4
     assert L.awq_prefetch_hint(None, 0) == 0 and L.awq_prefetch_pending() == 0
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_gemv_row_blocks_up_to_128_rows(dt):
+    """65..128 rows as blocks of 16 rows of the one-tile staged kernels (what awq_linear runs on small weights), with
+    and without a K split and a bias, against the fp32 oracle; a ragged last block included."""
+    tdt = torch.float16 if dt == "f16" else torch.bfloat16
+    for (M, K, N, variant, split) in [(65, 512, 384, 2, 1), (100, 1024, 1024, 3, 1), (128, 2048, 1024, 2, 2),
+                                      (127, 1024, 3072, 3, 1)]:
+        print(f"row blocks {dt} M={M} K={K} N={N} variant={variant} split={split}", flush=True)
+        p = random_packed(K, N, 128, dt, seed=M)
+        xb = make_x(M, K, dt, seed=M + 1)
+        dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dt), to_dev(p["qzeros"])]
+        y = awq_gemv_variant(to_dev(xb, dt), *dev, variant, split)
+        _check(y, xb, p, dt)
+        assert torch.equal(y, awq_gemv_variant(to_dev(xb, dt), *dev, variant, split))
+        yd = nq.awq_gemm(to_dev(xb, dt), *dev, 8)          # the default dispatch takes the same route
+        _check(yd, xb, p, dt)

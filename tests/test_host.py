@@ -197,7 +197,11 @@ def test_dispatch_plans_are_consistent():
     rc, v, s = _plan(L.awq_gemv_plan, 1, 1024, 2048, 128)
     assert rc == 0 and gemv_names[v] == "dma1x4" and s == 4, (gemv_names[v], s)
     # shapes awq_gemv does not take are refused by the plan as well
-    assert _plan(L.awq_gemv_plan, 65, 1024, 1024, 128)[0] != 0
+    assert _plan(L.awq_gemv_plan, 129, 1024, 1024, 128)[0] != 0
+    # 65..128 rows: blocks of 16 rows on the one-tile staged kernels, unsplit once the blocks fill the chip
+    rc, v, s = _plan(L.awq_gemv_plan, 128, 2048, 2048, 128)
+    assert rc == 0 and gemv_names[v] == "dma1x4" and s == 1, (gemv_names[v], s)
+    assert L.awq_gemv_workspace_bytes(128, 2048, 2048) <= L.awq_linear_workspace_bytes(128, 2048, 2048)
     assert _plan(L.awq_gemv_plan, 4, 1024, 1000, 128)[0] != 0
     assert _plan(L.awq_gemm_plan, 64, 1024, 96)[0] != 0
 

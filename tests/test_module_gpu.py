@@ -67,7 +67,8 @@ def test_state_dict_roundtrip_keeps_outputs():
 @pytest.mark.parametrize("bias", [False, True])
 def test_forward_empty_and_boundary_row_counts(bias):
     """No rows at all, and the row counts where the dispatch changes kernel (16/17 one m-tile vs row blocks, 64/65
-    GEMV vs GEMM, 1023/1024 where the reference's own structure changes): shape, dtype and the fp32 oracle at every one of them."""
+    and 128/129 GEMV vs GEMM -- 128 rows on small weights like this one --, 1023/1024 where the reference's own structure
+    changes): shape, dtype and the fp32 oracle at every one of them."""
     K, N, g = 512, 384, 128
     m = _module(K, N, g, torch.bfloat16, bias, seed=3)
     for shape in [(0, K), (2, 0, K)]:
@@ -75,7 +76,7 @@ def test_forward_empty_and_boundary_row_counts(bias):
         assert y.shape == tuple(shape[:-1]) + (N,) and y.dtype == torch.bfloat16 and y.numel() == 0
     qw, qz, qs = m.qweight.cpu().numpy(), m.qzeros.cpu().numpy(), to_bits(m.qscales)
     b = m.bias.float().cpu().numpy() if bias else None
-    for M in (16, 17, 64, 65, 1023, 1024):
+    for M in (16, 17, 64, 65, 128, 129, 1023, 1024):
         print(f"forward boundary M={M} bias={bias}", flush=True)
         torch.manual_seed(M)
         x = torch.randn(M, K).to(torch.bfloat16).cuda()
