@@ -39,6 +39,7 @@ EXTRA = {
     # the SLP vectoriser pairs the two k rows of the unpack into <2 x i32> and/or, which then no
     # longer select as one v_and_or_b32 each
     "awq_gemm_pipe.hip": ["-fno-slp-vectorize"],
+    "awq_gemm_regb.hip": ["-fno-slp-vectorize"],
 }
 
 

@@ -208,9 +208,13 @@ static const GemmVariant kGemmVariants[] = {
     {"32x256", 32, 256, 4},
     {"256x256p", 256, 256, 8},   // the software-pipelined kernel of awq_gemm_pipe.hip, every tile cut split_k ways
     {"256x256pt", 256, 256, 8},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
+    {"256x256r", 256, 256, 4},   // awq_gemm_regb.hip: B operands built in registers, every tile cut split_k ways
+    {"256x256rt", 256, 256, 4},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
 };
 enum { k128x128 = 0, k64x256 = 1, k32x256 = 2 };
-constexpr int kPipeVariant = 3, kPipeTailVariant = 4;
+constexpr int kPipeVariant = 3, kPipeTailVariant = 4, kRegbVariant = 5, kRegbTailVariant = 6;
+static bool is_tile256(int v) { return v >= kPipeVariant && v <= kRegbTailVariant; }
+static bool is_tail_variant(int v) { return v == kPipeTailVariant || v == kRegbTailVariant; }
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 template <typename T, int BM, int BN, int WM, int WN>
@@ -255,8 +259,7 @@ static int gemm_effective_splits(int64_t K, int split_k) {
 }
 
 static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k) {
-    if (variant == kPipeVariant || variant == kPipeTailVariant)
-        return pipe_ws_bytes(make_pipe_plan(M, N, K, split_k, variant == kPipeTailVariant));
+    if (is_tile256(variant)) return pipe_ws_bytes(make_pipe_plan(M, N, K, split_k, is_tail_variant(variant)));
     const int splits = gemm_effective_splits(K, split_k);
     if (splits <= 1) return 0;
     return kCounterBytes + (size_t)splits * M * N * sizeof(float);
@@ -339,7 +342,7 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         set_error("%s: bad variant %d / split_k %d", fn, variant, split_k);
         return AWQ_ERR_INVALID_ARG;
     }
-    if (act && (bias || N % 16 != 0 || (variant != kPipeVariant && variant != kPipeTailVariant))) {
+    if (act && (bias || N % 16 != 0 || !is_tile256(variant))) {
         set_error("%s: the gated epilogue takes no bias, needs N %% 16 == 0 and runs on the pipelined kernel", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
@@ -373,6 +376,15 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         case kPipeTailVariant:
             e = launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
                                  workspace, split_k, variant == kPipeTailVariant, s, act);
+            break;
+        case kRegbVariant:
+        case kRegbTailVariant:
+            if (g % 64 != 0) {
+                set_error("%s: variant %s needs a group size that is a multiple of 64 (g=%lld)", fn, gv.name, (long long)g);
+                return AWQ_ERR_UNSUPPORTED;
+            }
+            e = launch_gemm_regb(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+                                 workspace, split_k, variant == kRegbTailVariant, s, act);
             break;
     }
 #undef AWQ_GEMM_CASE

@@ -63,6 +63,29 @@ struct UnpackRows<BF16> {
 };
 
 
+// Gated epilogue: a lane pair holds a gate word and the up word of the same 8 outputs (already rounded to T); each
+// lane of the pair produces four of them (the even lane outputs 0..3, the odd lane 4..7) and stores 8 bytes:
+// dtype(SiLU(gate)) * up, the rounding points of F.silu(gate_proj(x)) * up_proj(x).  `mine` is this lane's word,
+// `other` its partner's, `odd` says which of the two this lane holds.
+template <typename T>
+__device__ __forceinline__ void swiglu_pair_store(u32x4 mine, u32x4 other, bool odd, uint16_t* __restrict__ dst) {
+    const u32x4 gate = odd ? other : mine, up = odd ? mine : other;
+    uint32_t o[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t gw = odd ? gate[2 + i] : gate[i], uw = odd ? up[2 + i] : up[i];
+        float r[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float g = T::to_f32((uint16_t)(h ? gw >> 16 : gw & 0xFFFFu));
+            const float u = T::to_f32((uint16_t)(h ? uw >> 16 : uw & 0xFFFFu));
+            r[h] = T::to_f32(T::from_f32(g / (1.f + __expf(-g)))) * u;
+        }
+        o[i] = T::pack2(r[0], r[1]);
+    }
+    *reinterpret_cast<u32x2*>(dst + (odd ? 4 : 0)) = u32x2{o[0], o[1]};
+}
+
 // acc[a][b][v] of the 32x32x16 MFMA: row (v/4)*8 + (lane/32)*4 + v%4, column lane%32 of tile
 // (a, b) of the wave's sub-tile at (wm0, wn0).
 template <typename T, int BM, int BN, int TM, int TN, int NT>
@@ -168,6 +191,17 @@ inline size_t pipe_ws_bytes(const PipePlan& p) {
 
 // awq_gemm_pipe.hip: the 256 x 256 software-pipelined kernel (same arguments as the tiled launcher).
 hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
+                            const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
+                            void* workspace, int split_k, bool tail_only, hipStream_t stream, int act = 0);
+
+// awq_gemm_pipe.hip: the second pass over the tail tiles of a PipePlan (fp32 partials [slice][tail tile][256][256]
+// added in slice order, + bias or the gated product), on `stream` after the kernel that wrote them.
+hipError_t launch_pipe_tail_reduce(int dtype, const float* partials, const void* bias, void* y, int M, int N,
+                                   const PipePlan& plan, hipStream_t stream);
+
+// awq_gemm_regb.hip: the 256 x 256 kernel that builds its B operands in registers (same arguments; group sizes that are
+// multiples of 64 only).
+hipError_t launch_gemm_regb(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
                             void* workspace, int split_k, bool tail_only, hipStream_t stream, int act = 0);
 

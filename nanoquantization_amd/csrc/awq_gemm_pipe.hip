@@ -99,29 +99,6 @@ struct Raw {
     u32x4 s;
 };
 
-// Gated epilogue: a lane pair holds a gate word and the up word of the same 8 outputs (already rounded to T); each
-// lane of the pair produces four of them (the even lane outputs 0..3, the odd lane 4..7) and stores 8 bytes:
-// dtype(SiLU(gate)) * up, the rounding points of F.silu(gate_proj(x)) * up_proj(x).  `mine` is this lane's word,
-// `other` its partner's, `odd` says which of the two this lane holds.
-template <typename T>
-__device__ __forceinline__ void swiglu_pair_store(u32x4 mine, u32x4 other, bool odd, uint16_t* __restrict__ dst) {
-    const u32x4 gate = odd ? other : mine, up = odd ? mine : other;
-    uint32_t o[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint32_t gw = odd ? gate[2 + i] : gate[i], uw = odd ? up[2 + i] : up[i];
-        float r[2];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const float g = T::to_f32((uint16_t)(h ? gw >> 16 : gw & 0xFFFFu));
-            const float u = T::to_f32((uint16_t)(h ? uw >> 16 : uw & 0xFFFFu));
-            r[h] = T::to_f32(T::from_f32(g / (1.f + __expf(-g)))) * u;
-        }
-        o[i] = T::pack2(r[0], r[1]);
-    }
-    *reinterpret_cast<u32x2*>(dst + (odd ? 4 : 0)) = u32x2{o[0], o[1]};
-}
-
 template <typename T, int WM, int WN>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
@@ -470,12 +447,22 @@ hipError_t launch_pipe(const void* x, const int32_t* qweight, const void* qscale
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, M, N, K, g, plan);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || plan.tail_tiles == 0) return e;
-    hipLaunchKernelGGL(gemm_tail_reduce_kernel<T>, dim3(plan.tail_tiles * 32), dim3(256), 0, stream, partials,
-                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, plan);
-    return hipGetLastError();
+    return launch_pipe_tail_reduce(T::id, partials, bias, y, M, N, plan, stream);
 }
 
 }  // namespace
+
+hipError_t launch_pipe_tail_reduce(int dtype, const float* partials, const void* bias, void* y, int M, int N,
+                                   const PipePlan& plan, hipStream_t stream) {
+    const dim3 grid(plan.tail_tiles * 32), block(256);
+    if (dtype == AWQ_F16)
+        hipLaunchKernelGGL(gemm_tail_reduce_kernel<F16>, grid, block, 0, stream, partials,
+                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, plan);
+    else
+        hipLaunchKernelGGL(gemm_tail_reduce_kernel<BF16>, grid, block, 0, stream, partials,
+                           reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, plan);
+    return hipGetLastError();
+}
 
 hipError_t launch_gemm_pipe(int dtype, const void* x, const int32_t* qweight, const void* qscales,
                             const int32_t* qzeros, const void* bias, void* y, int M, int N, int K, int g,
