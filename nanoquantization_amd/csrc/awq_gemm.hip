@@ -208,8 +208,10 @@ static const GemmVariant kGemmVariants[] = {
     {"32x256", 32, 256, 4},
     {"256x256p", 256, 256, 8},   // the software-pipelined kernel of awq_gemm_pipe.hip, every tile cut split_k ways
     {"256x256pt", 256, 256, 8},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
-    {"256x256r", 256, 256, 4},   // awq_gemm_regb.hip: B operands built in registers, every tile cut split_k ways
-    {"256x256rt", 256, 256, 4},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
+    // awq_gemm_regb.hip: B operands built in registers, the default above 128 rows; group sizes that are not multiples of
+    // 64 run the pipelined kernel under these names too
+    {"256x256r", 256, 256, 4},   // every tile cut split_k ways
+    {"256x256rt", 256, 256, 4},  // split_k cuts only the tiles beyond the last full round of CUs
 };
 enum { k128x128 = 0, k64x256 = 1, k32x256 = 2 };
 constexpr int kPipeVariant = 3, kPipeTailVariant = 4, kRegbVariant = 5, kRegbTailVariant = 6;
@@ -265,13 +267,15 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
     return kCounterBytes + (size_t)splits * M * N * sizeof(float);
 }
 
-// Tile shape and split for the default entry point.  Large M: the pipelined 256 x 256 kernel with two
-// wavefronts per SIMD, K split so that the tiles cover the CUs once (a split costs one more pass over
-// the fp32 partials, which is cheap next to an idle CU).  Small M: narrower tiles of the plain kernel.
+// Tile shape and split for the default entry point.  Large M: the 256 x 256 kernel that builds its B operands in
+// registers (on one box, M = 8192 x 4096 x 12288: fp16 855-865 us against the pipelined kernel's 935, bf16 804
+// against 801, 12288 x 4096 bf16 774 against 797), K split so that the tiles cover the CUs once (a split costs
+// one more pass over the fp32 partials, which is cheap next to an idle CU).  Small M: narrower tiles of the plain
+// kernel.
 static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     const int kCUs = 256;
     // indices into kGemmVariants
-    constexpr int kPipe8 = kPipeVariant;
+    constexpr int kPipe8 = kRegbVariant;
     int v;
     if (M <= 32) v = k32x256;
     else if (M <= 64) v = k64x256;
@@ -292,9 +296,9 @@ static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_
             const int64_t t = cdiv(R * c, kCUs) * (cdiv(steps, c) + 5);
             if (t < best_t) best_t = t, best_s = c;
         }
-        if (best_s > 1 && best_t * 10 <= steps * 9) v = kPipeTailVariant, s = best_s;
+        if (best_s > 1 && best_t * 10 <= steps * 9) v = kRegbTailVariant, s = best_s;
     }
-    if (v != kPipe8 && v != kPipeTailVariant) {
+    if (!is_tile256(v)) {
         // Narrow tiles (up to 128 rows): two workgroups of the 128x128 and 32x256 forms share a CU, one of the 64x256
         // form.  Workgroups run in rounds of that many; a round lasts one split's K steps plus about six steps of
         // prologue and partial store.  Take the split count with the least rounds x length (5120 x 25600 at 128
@@ -379,12 +383,10 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
             break;
         case kRegbVariant:
         case kRegbTailVariant:
-            if (g % 64 != 0) {
-                set_error("%s: variant %s needs a group size that is a multiple of 64 (g=%lld)", fn, gv.name, (long long)g);
-                return AWQ_ERR_UNSUPPORTED;
-            }
-            e = launch_gemm_regb(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
-                                 workspace, split_k, variant == kRegbTailVariant, s, act);
+            e = g % 64 == 0 ? launch_gemm_regb(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+                                               workspace, split_k, variant == kRegbTailVariant, s, act)
+                            : launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+                                               workspace, split_k, variant == kRegbTailVariant, s, act);
             break;
     }
 #undef AWQ_GEMM_CASE
@@ -492,7 +494,7 @@ extern "C" int awq_linear_swiglu(const void* x, const int32_t* qweight, const vo
     if (M >= 1 && M <= 64 && staged)
         return awq_gemv_swiglu(x, qweight, qscales, qzeros, y, M, N, K, group_size, dtype, workspace,
                                workspace_bytes, stream);
-    int v = awq::kPipeVariant, s = 1;
+    int v = awq::kRegbVariant, s = 1;
     if (K >= awq::kBK && N >= 16 && M >= 1) awq::pick_gemm_pipe(M, N, K, &v, &s);
     return awq::gemm_dispatch("awq_linear_swiglu", x, qweight, qscales, qzeros, nullptr, y, M, N, K, group_size,
                               dtype, workspace, workspace_bytes, stream, v, s, 1);

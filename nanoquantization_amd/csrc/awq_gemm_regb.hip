@@ -1,22 +1,41 @@
 // Kernel (c), large-M form with the B operand built in registers: fused dequant + GEMM on the
-// 16x16x32 MFMA, no dequantised weight ever in LDS.
+// 16x16x32 MFMA; the dequantised weight exists only as MFMA operands.
 //
 // A workgroup of 4 wavefronts (2 x 2, one per SIMD, a 128 x 128 sub-tile and 256 accumulator
-// registers each) owns a 256 x 256 output tile and walks K in steps of 64.
+// registers each) owns a 256 x 256 output tile and walks K in steps of 64, two half steps of 32.
 //
-// Lane roles, as in the decode GEMV: a lane is (j = lane % 16, kq = lane / 16).  Per 32 k rows it
+// Lane roles, as in the decode GEMV: a lane is (j = lane % 16, kq = lane / 16).  Per half step it
 // holds the packed words of rows 8*kq + 0..7 of word column j of the wave's 16 word columns: 8 k x
 // 8 columns, which is what the MFMA wants from this lane as B operand of EIGHT column tiles -- tile
 // t takes nibble position t of every word, so a lane's column in tile t is 8*j + column_of(t) and
-// the 8 k values of its operand are the 8 rows it holds.  v_perm_b32 pairs byte b of two rows, a
-// mask puts the nibbles into a 16-bit float each, and the values are multiplied out to
-// RN_dtype((q - z) * s) in registers.  Each weight is unpacked by the two wavefronts that share its
-// columns (2 x the arithmetic of unpacking once per workgroup) and in exchange the B tile needs no
-// LDS store, no barrier between unpack and use and no LDS operand reads; LDS carries the A tile
-// only (global_load_lds, three buffers), read as 16 operand fragments per wave and step.
+// the 8 k values of its operand are the 8 rows it holds.  v_perm_b32 pairs byte b of two rows (fp16)
+// or a mask puts a nibble into an fp32 mantissa (bf16), and the values are multiplied out to
+// RN_dtype((q - z) * s) in registers.
+//
+// The two wavefronts that share a column range (the upper and the lower 128 rows) split that work:
+// each builds the operands of four of the eight nibble positions, two half steps ahead, and leaves
+// them in LDS in operand layout (16 bytes per lane, lane-linear: no bank conflicts, no transpose);
+// one half step later both read all eight back.  So every weight is unpacked once per workgroup,
+// LDS carries 16 KiB of B operands per half step next to the A tile (global_load_lds, three
+// buffers), and the unpack is a dozen vector-ALU instructions per 8 MFMAs.
 //
 // Epilogue: a lane's eight tiles are the eight columns of its word, so a row of its accumulators
 // leaves as one 16-byte store (fp32 partials of a K slice: two), without staging.
+//
+// What the instructions cost (measured on one wave per SIMD, MFMAs back to back with one other
+// instruction mixed in per 8): a 16x16x32 MFMA occupies the matrix core for 18.5 cycles and the
+// SIMD's issue port for 12 of them, any other instruction for 4; LDS reads and global loads to
+// registers are such 4-cycle instructions, but an LDS write of 1 KiB holds the port 32 cycles, a
+// load-to-LDS of 1 KiB 44 and a barrier 12, and with one wave per SIMD nobody issues meanwhile.
+// Per step that adds up to more than the matrix core's 128 x 18.5 cycles, so every instruction
+// saved shows: the shared unpack (half the vector-ALU work, 8 more LDS writes per wave and step)
+// is worth 3 % in bf16 and nothing in fp16 against unpacking everything in both waves of a pair.
+// Forms of this kernel on the 32x32x16 MFMA (a quarter of the issue cost per flop; a 64 x 256
+// sub-tile per wave with a four-way split of the unpack, or 128 x 128 with the lanes of a 32-wide
+// column tile taking the low and the high nibble of 16 words) gave bit-identical results 10-15 %
+// slower, and so did loading the A operands straight from global memory (no LDS at all).
+#include <type_traits>
+
 #include "awq_common.hpp"
 #include "awq_gemm_parts.hpp"
 
@@ -37,17 +56,19 @@ __host__ __device__ constexpr int column_of(int t) { return t < 4 ? 2 * t : 2 * 
 __host__ __device__ constexpr int position_of(int c) { return 4 * (c & 1) + (c >> 1); }
 
 // ---- 8 MFMAs and the unpack that hides behind them, as one assembly statement ---------------------------------
-// A row tile's 8 MFMAs (one A fragment against the 8 B operands of the running half step) are issued with a piece of
-// the NEXT half step's unpack behind each: at most three vector-ALU instructions between two MFMAs, none of them
-// reading the result of the instruction right before it.  Written as assembly because the order is the point: left to
-// the compiler, ordinary expressions are placed freely by instruction selection (they clump), accumulators wander
-// between the two register files, and every value that one assembly statement hands to the next costs a wait state
-// (the hazard pass assumes the worst of a statement it cannot read) -- so a statement is a whole row tile, whose
-// results are first read a row tile later.
+// A row tile's 8 MFMAs (one A fragment against the 8 B operands of the running half step) are issued with one eighth
+// of the wave's unpack work behind them: one or two vector-ALU instructions between two MFMAs, none of them reading the
+// result of the instruction right before it.  (Measured on one wave per SIMD: a 16x16x32 MFMA takes 12 of its 18.5
+// cycles to issue, every other instruction 4, so more than one and a half of them per MFMA and the matrix core
+// waits.)  Written as assembly because the order is the point: left to the compiler, ordinary expressions are placed
+// freely by instruction selection (they clump), accumulators wander between the two register files, and every value
+// that one assembly statement hands to the next costs a wait state (the hazard pass assumes the worst of a statement it
+// cannot read) -- so a statement is a whole row tile, whose results are first read a row tile later.
 // The accumulators are pinned to the AGPR file by the operand constraint: all 256 of a wave's are accumulators, the
 // 256 VGPRs stay free for operands and the unpack.  An MFMA's result is next read 64 MFMAs later, or after the wait in
-// front of the epilogue.
-template <typename T>
+// front of the epilogue.  The "memory" clobber keeps the loads and LDS traffic that the loop places between two
+// statements where they are.
+template <typename T, int ROLE>
 struct FragUnpack;
 
 #define AWQ_RB_ACC_OPERANDS                                                                                          \
@@ -60,18 +81,21 @@ struct FragUnpack;
 
 // fp16: byte b of rows k, k+1 -> 0x00HL00HL (v_perm_b32); the low nibbles under 0x6400 are 1024 + q, the high nibbles
 // under 0x5400 are 64 + q (no shift); minus the zero point embedded the same way (exact), times the scale (one
-// rounding: the reference's RN_f16((q - z) * s)).  Row tile mg of a half step does bytes 2*(mg%2), +1 of row pair mg/2.
-template <>
-struct FragUnpack<F16> {
-    uint32_t ezlo[4], ezhi[4], slo[4], shi[4];
-    uint32_t sel[4];             // v_perm selectors, in VGPRs
+// rounding: the reference's RN_f16((q - z) * s)).  Wave ROLE of a pair owns bytes 2*ROLE, 2*ROLE + 1 of every word,
+// i.e. nibble positions 4*ROLE .. 4*ROLE + 3; row tile m of a half step does byte 2*ROLE + m%2 of row pair m/2.
+template <int ROLE>
+struct FragUnpack<F16, ROLE> {
+    static __device__ __forceinline__ constexpr int own(int i) { return 4 * ROLE + i; }   // nibble position of own[i]
+    uint32_t ezlo[2], ezhi[2], slo[2], shi[2];   // of the two own bytes
+    uint32_t sel[2];             // v_perm selectors, in VGPRs
     uint32_t mask_lo, mask_hi;   // SGPRs
     uint32_t magic_lo, magic_hi; // VGPRs (v_and_or_b32 takes one scalar operand)
     __device__ __forceinline__ void init() {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            sel[b] = 0x0C040C00u | (uint32_t)b | ((uint32_t)b << 16);
-            asm volatile("" : "+v"(sel[b]));
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t b = 2 * ROLE + i;
+            sel[i] = 0x0C040C00u | b | (b << 16);
+            asm volatile("" : "+v"(sel[i]));
         }
         mask_lo = 0x000F000Fu; mask_hi = 0x00F000F0u; magic_lo = 0x64006400u; magic_hi = 0x54005400u;
         asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));
@@ -79,75 +103,59 @@ struct FragUnpack<F16> {
     }
     __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const uint32_t zb = __builtin_amdgcn_perm(zw, zw, 0x0C000C00u | (uint32_t)b | ((uint32_t)b << 16));
-            ezlo[b] = (zb & mask_lo) | magic_lo;
-            ezhi[b] = (zb & mask_hi) | magic_hi;
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t b = 2 * ROLE + i;
+            const uint32_t zb = __builtin_amdgcn_perm(zw, zw, 0x0C000C00u | b | (b << 16));
+            ezlo[i] = (zb & mask_lo) | magic_lo;
+            ezhi[i] = (zb & mask_hi) | magic_hi;
             constexpr uint32_t dup_lo = 0x01000100u, dup_hi = 0x03020302u;
             const int cl = column_of(2 * b), ch = column_of(2 * b + 1);
-            slo[b] = __builtin_amdgcn_perm(sv[cl >> 1], sv[cl >> 1], (cl & 1) ? dup_hi : dup_lo);
-            shi[b] = __builtin_amdgcn_perm(sv[ch >> 1], sv[ch >> 1], (ch & 1) ? dup_hi : dup_lo);
+            slo[i] = __builtin_amdgcn_perm(sv[cl >> 1], sv[cl >> 1], (cl & 1) ? dup_hi : dup_lo);
+            shi[i] = __builtin_amdgcn_perm(sv[ch >> 1], sv[ch >> 1], (ch & 1) ? dup_hi : dup_lo);
         }
     }
-    // acc[t] += af x bfc[t] for the 8 column tiles; meanwhile bfn[t][r] = (W[k + 2r, col t], W[k + 2r + 1, col t]) of
-    // the 8 rows w[0..7] of the next half step, for r = mg/2 and the four positions t of bytes 2*(mg%2), +1
-    __device__ __forceinline__ void row_tile(int mg, f32x4 (&acc)[8], const u32x4& af, const u32x4 (&bfc)[8],
-                                             const uint32_t (&w)[8], u32x4 (&bfn)[8]) {
-        const int r = mg >> 1, b0 = 2 * (mg & 1), b1 = b0 + 1;
-        uint32_t o0, o1, o2, o3, t0, t1, t2;
+    // acc[t] += af x bfc[t] for the 8 column tiles; meanwhile out[i][r] = (W[k + 2r, own(i)], W[k + 2r + 1, own(i)])
+    // of the 8 rows w[0..7] of a later half step, for r = m/2 and i = 2*(m%2), +1
+    __device__ __forceinline__ void row_tile(int m, f32x4 (&acc)[8], const u32x4& af, const u32x4 (&bfc)[8],
+                                             const uint32_t (&w)[8], u32x4 (&out)[4]) {
+        const int r = m >> 1, i = m & 1;
+        uint32_t o0, o1, t0, t1, t2;
         asm volatile(
             AWQ_RB_MFMA("f16", 0) "v_perm_b32 %[t0], %[w1], %[w0], %[s0]\n\t"
             AWQ_RB_MFMA("f16", 1) "v_and_or_b32 %[t1], %[mlo], %[t0], %[glo]\n\t"
-                                  "v_and_or_b32 %[t2], %[mhi], %[t0], %[ghi]\n\t"
-            AWQ_RB_MFMA("f16", 2) "v_pk_add_f16 %[t1], %[t1], %[z0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
-                                  "v_pk_add_f16 %[t2], %[t2], %[z1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
-            AWQ_RB_MFMA("f16", 3) "v_pk_mul_f16 %[o0], %[t1], %[q0]\n\t"
-                                  "v_pk_mul_f16 %[o1], %[t2], %[q1]\n\t"
-            AWQ_RB_MFMA("f16", 4) "v_perm_b32 %[t0], %[w1], %[w0], %[s1]\n\t"
-            AWQ_RB_MFMA("f16", 5) "v_and_or_b32 %[t1], %[mlo], %[t0], %[glo]\n\t"
-                                  "v_and_or_b32 %[t2], %[mhi], %[t0], %[ghi]\n\t"
-            AWQ_RB_MFMA("f16", 6) "v_pk_add_f16 %[t1], %[t1], %[z2] neg_lo:[0,1] neg_hi:[0,1]\n\t"
-                                  "v_pk_add_f16 %[t2], %[t2], %[z3] neg_lo:[0,1] neg_hi:[0,1]\n\t"
-            AWQ_RB_MFMA("f16", 7) "v_pk_mul_f16 %[o2], %[t1], %[q2]\n\t"
-                                  "v_pk_mul_f16 %[o3], %[t2], %[q3]\n\t"
-            : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [o2] "=&v"(o2), [o3] "=&v"(o3), [t0] "=&v"(t0),
-              [t1] "=&v"(t1), [t2] "=&v"(t2)
-            : AWQ_RB_AB_OPERANDS, [w0] "v"(w[2 * r]), [w1] "v"(w[2 * r + 1]), [s0] "v"(sel[b0]), [s1] "v"(sel[b1]),
-              [mlo] "s"(mask_lo), [mhi] "s"(mask_hi), [glo] "v"(magic_lo), [ghi] "v"(magic_hi), [z0] "v"(ezlo[b0]),
-              [z1] "v"(ezhi[b0]), [z2] "v"(ezlo[b1]), [z3] "v"(ezhi[b1]), [q0] "v"(slo[b0]), [q1] "v"(shi[b0]),
-              [q2] "v"(slo[b1]), [q3] "v"(shi[b1])
+            AWQ_RB_MFMA("f16", 2) "v_and_or_b32 %[t2], %[mhi], %[t0], %[ghi]\n\t"
+            AWQ_RB_MFMA("f16", 3) "v_pk_add_f16 %[t1], %[t1], %[z0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            AWQ_RB_MFMA("f16", 4) "v_pk_add_f16 %[t2], %[t2], %[z1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            AWQ_RB_MFMA("f16", 5) "v_pk_mul_f16 %[o0], %[t1], %[q0]\n\t"
+            AWQ_RB_MFMA("f16", 6) "v_pk_mul_f16 %[o1], %[t2], %[q1]\n\t"
+            AWQ_RB_MFMA("f16", 7)
+            : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2)
+            : AWQ_RB_AB_OPERANDS, [w0] "v"(w[2 * r]), [w1] "v"(w[2 * r + 1]), [s0] "v"(sel[i]), [mlo] "s"(mask_lo),
+              [mhi] "s"(mask_hi), [glo] "v"(magic_lo), [ghi] "v"(magic_hi), [z0] "v"(ezlo[i]), [z1] "v"(ezhi[i]),
+              [q0] "v"(slo[i]), [q1] "v"(shi[i])
             : "memory");
-        bfn[2 * b0][r] = o0;
-        bfn[2 * b0 + 1][r] = o1;
-        bfn[2 * b1][r] = o2;
-        bfn[2 * b1 + 1][r] = o3;
-    }
-    // the same unpack without MFMAs (the first half step of a workgroup)
-    __device__ __forceinline__ void unpack_only(const uint32_t (&w)[8], u32x4 (&bfn)[8]) const {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const uint32_t p = __builtin_amdgcn_perm(w[2 * r + 1], w[2 * r], 0x0C040C00u | (uint32_t)b | ((uint32_t)b << 16));
-                const uint32_t lo = (p & mask_lo) | magic_lo, hi = (p & mask_hi) | magic_hi;
-                bfn[2 * b][r] = as_u32((as_f16x2(lo) - as_f16x2(ezlo[b])) * as_f16x2(slo[b]));
-                bfn[2 * b + 1][r] = as_u32((as_f16x2(hi) - as_f16x2(ezhi[b])) * as_f16x2(shi[b]));
-            }
+        out[2 * i][r] = o0;
+        out[2 * i + 1][r] = o1;
     }
 };
 
 // bf16: a nibble is masked in place at mantissa bit 8, 12 or 16 of the fp32 pattern 0x4B000000 (value 2^23 + q * 2^e),
 // so fma(f, s * 2^-e, -(2^(23-e) + z) * s) = (q - z) * s exactly (product and constant have at most 24 significant
 // bits, the sum at most 13); positions 0-1 and 5-7 are brought there by one shift of the word each (w << 8, w >> 12).
-// Two rows are packed with one round-to-nearest-even conversion.  Row tile mg of a half step does row pair mg/2:
-// positions 2, 3, 4, 0 (even mg; it also makes the two left shifts) or 1, 5, 6, 7 (odd mg; the right shifts).
-template <>
-struct FragUnpack<BF16> {
-    float sc[8], off[8];   // per nibble position
-    uint32_t mask8, mask12, mask16, magic;
-    uint32_t l0, l1;
-    static __device__ __forceinline__ constexpr int src_of(int t) { return t < 2 ? 0 : (t < 5 ? 1 : 2); }   // w<<8, w, w>>12
+// Two rows are packed with one round-to-nearest-even conversion.  Wave 0 of a pair owns positions 2, 3, 4, 0 (the
+// word itself and its left-shifted copy), wave 1 positions 1, 5, 6, 7 (the left- and the right-shifted copy); row
+// tiles 2r and 2r + 1 of a half step do two of them each for row pair r.
+#define AWQ_RB_E(D, SRC, MSK) "v_and_or_b32 %[" D "], %[" MSK "], %[" SRC "], %[g]\n\t"
+#define AWQ_RB_F(D, E, P) "v_fma_f32 %[" D "], %[" E "], %[s" P "], %[k" P "]\n\t"
+#define AWQ_RB_C(O) "v_cvt_pk_bf16_f32 %[" O "], %[f0], %[f1]\n\t"
+template <int ROLE>
+struct FragUnpack<BF16, ROLE> {
+    static __device__ __forceinline__ constexpr int own(int i) { return ROLE == 0 ? (i < 3 ? i + 2 : 0) : (i == 0 ? 1 : i + 4); }
     static __device__ __forceinline__ constexpr int bit_of(int t) { return t < 2 ? 4 * t + 8 : (t < 5 ? 4 * t : 4 * t - 12); }
+    static __device__ __forceinline__ constexpr int src_of(int t) { return t < 2 ? 0 : (t < 5 ? 1 : 2); }   // w<<8, w, w>>12
+    float sc[4], off[4];   // of the four own positions
+    uint32_t mask8, mask12, mask16, magic;
+    uint32_t x0, x1, x2, x3;   // shifted copies handed from the even to the odd row tile of a row pair
     __device__ __forceinline__ void init() {
         mask8 = 0xF00u; mask12 = 0xF000u; mask16 = 0xF0000u; magic = 0x4B000000u;
         asm volatile("" : "+s"(mask8), "+s"(mask12), "+s"(mask16));
@@ -159,86 +167,109 @@ struct FragUnpack<BF16> {
     __device__ __forceinline__ void set_group(uint32_t zw, u32x4 sv) {
         const uint32_t zl = zw << 8, zh = zw >> 12;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const int c = column_of(t);
+        for (int i = 0; i < 4; ++i) {
+            const int t = own(i), c = column_of(t);
             const uint32_t pr = sv[c >> 1];
             const float s = __builtin_bit_cast(float, (c & 1) ? (pr & 0xFFFF0000u) : (pr << 16));
             const float down = bit_of(t) == 8 ? 0x1p-8f : (bit_of(t) == 12 ? 0x1p-12f : 0x1p-16f);
             const uint32_t src = src_of(t) == 0 ? zl : (src_of(t) == 1 ? zw : zh);
-            sc[t] = s * down;                                                                  // exact: a power of two
-            off[t] = -(__builtin_bit_cast(float, (src & mask_of(t)) | magic) * sc[t]);   // (2^(23-e) + z) * s: <= 24 bits
+            sc[i] = s * down;                                                                  // exact: a power of two
+            off[i] = -(__builtin_bit_cast(float, (src & mask_of(t)) | magic) * sc[i]);   // (2^(23-e) + z) * s: <= 24 bits
         }
     }
-#define AWQ_RB_BF16_POS(P, SRC0, SRC1)                                     \
-    "v_and_or_b32 %[e0], %[m" #P "], %[" SRC0 "], %[g]\n\t"                \
-    "v_and_or_b32 %[e1], %[m" #P "], %[" SRC1 "], %[g]\n\t"
-#define AWQ_RB_BF16_FMA(P)                                                 \
-    "v_fma_f32 %[f0], %[e0], %[s" #P "], %[k" #P "]\n\t"                   \
-    "v_fma_f32 %[f1], %[e1], %[s" #P "], %[k" #P "]\n\t"
-    __device__ __forceinline__ void row_tile(int mg, f32x4 (&acc)[8], const u32x4& af, const u32x4 (&bfc)[8],
-                                             const uint32_t (&w)[8], u32x4 (&bfn)[8]) {
-        const int r = mg >> 1;
-        uint32_t o0, o1, o2, o3, e0, e1, x0, x1;
+    __device__ __forceinline__ void row_tile(int m, f32x4 (&acc)[8], const u32x4& af, const u32x4 (&bfc)[8],
+                                             const uint32_t (&w)[8], u32x4 (&out)[4]) {
+        const int r = m >> 1;
+        uint32_t o0, o1, e0, e1, e2, e3;
         float f0, f1;
-        if ((mg & 1) == 0) {
-            // positions 2, 3, 4 from the word itself, 0 from the left-shifted copy made on the way
+        if (ROLE == 0 && (m & 1) == 0) {
+            // positions 2, 3 from the word itself; the left-shifted copies for the odd row tile
             asm volatile(
-                AWQ_RB_MFMA("bf16", 0) AWQ_RB_BF16_POS(A, "w0", "w1") "v_lshlrev_b32 %[x0], 8, %[w0]\n\t"
-                AWQ_RB_MFMA("bf16", 1) AWQ_RB_BF16_FMA(A) "v_lshlrev_b32 %[x1], 8, %[w1]\n\t"
-                AWQ_RB_MFMA("bf16", 2) "v_cvt_pk_bf16_f32 %[o0], %[f0], %[f1]\n\t" AWQ_RB_BF16_POS(B, "w0", "w1")
-                AWQ_RB_MFMA("bf16", 3) AWQ_RB_BF16_FMA(B)
-                AWQ_RB_MFMA("bf16", 4) "v_cvt_pk_bf16_f32 %[o1], %[f0], %[f1]\n\t" AWQ_RB_BF16_POS(C, "w0", "w1")
-                AWQ_RB_MFMA("bf16", 5) AWQ_RB_BF16_FMA(C)
-                AWQ_RB_MFMA("bf16", 6) "v_cvt_pk_bf16_f32 %[o2], %[f0], %[f1]\n\t" AWQ_RB_BF16_POS(D, "x0", "x1")
-                AWQ_RB_MFMA("bf16", 7) AWQ_RB_BF16_FMA(D)
-                "s_nop 0\n\t"
-                "v_cvt_pk_bf16_f32 %[o3], %[f0], %[f1]\n\t"
-                : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [o2] "=&v"(o2), [o3] "=&v"(o3), [e0] "=&v"(e0),
-                  [e1] "=&v"(e1), [f0] "=&v"(f0), [f1] "=&v"(f1), [x0] "=&v"(x0), [x1] "=&v"(x1)
+                AWQ_RB_MFMA("bf16", 0) AWQ_RB_E("e0", "w0", "mA") AWQ_RB_E("e1", "w1", "mA")
+                AWQ_RB_MFMA("bf16", 1) AWQ_RB_F("f0", "e0", "A") AWQ_RB_F("f1", "e1", "A")
+                AWQ_RB_MFMA("bf16", 2) AWQ_RB_E("e2", "w0", "mB") AWQ_RB_E("e3", "w1", "mB")
+                AWQ_RB_MFMA("bf16", 3) AWQ_RB_C("o0") "v_lshlrev_b32 %[x0], 8, %[w0]\n\t"
+                AWQ_RB_MFMA("bf16", 4) AWQ_RB_F("f0", "e2", "B") AWQ_RB_F("f1", "e3", "B")
+                AWQ_RB_MFMA("bf16", 5) "v_lshlrev_b32 %[x1], 8, %[w1]\n\t"
+                AWQ_RB_MFMA("bf16", 6) AWQ_RB_C("o1")
+                AWQ_RB_MFMA("bf16", 7)
+                : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [e0] "=&v"(e0), [e1] "=&v"(e1), [e2] "=&v"(e2),
+                  [e3] "=&v"(e3), [f0] "=&v"(f0), [f1] "=&v"(f1), [x0] "=&v"(x0), [x1] "=&v"(x1)
                 : AWQ_RB_AB_OPERANDS, [w0] "v"(w[2 * r]), [w1] "v"(w[2 * r + 1]), [g] "v"(magic), [mA] "s"(mask_of(2)),
-                  [mB] "s"(mask_of(3)), [mC] "s"(mask_of(4)), [mD] "s"(mask_of(0)), [sA] "v"(sc[2]), [sB] "v"(sc[3]),
-                  [sC] "v"(sc[4]), [sD] "v"(sc[0]), [kA] "v"(off[2]), [kB] "v"(off[3]), [kC] "v"(off[4]),
-                  [kD] "v"(off[0])
+                  [mB] "s"(mask_of(3)), [sA] "v"(sc[0]), [sB] "v"(sc[1]), [kA] "v"(off[0]), [kB] "v"(off[1])
                 : "memory");
-            l0 = x0, l1 = x1;
-            bfn[2][r] = o0, bfn[3][r] = o1, bfn[4][r] = o2, bfn[0][r] = o3;
-        } else {
-            // position 1 from the left-shifted copies of the even row tile, 5, 6, 7 from right-shifted ones
+            out[0][r] = o0, out[1][r] = o1;
+        } else if (ROLE == 0) {
+            // position 4 from the word itself, position 0 from the left-shifted copies
             asm volatile(
-                AWQ_RB_MFMA("bf16", 0) AWQ_RB_BF16_POS(A, "l0", "l1") "v_lshrrev_b32 %[x0], 12, %[w0]\n\t"
-                AWQ_RB_MFMA("bf16", 1) AWQ_RB_BF16_FMA(A) "v_lshrrev_b32 %[x1], 12, %[w1]\n\t"
-                AWQ_RB_MFMA("bf16", 2) "v_cvt_pk_bf16_f32 %[o0], %[f0], %[f1]\n\t" AWQ_RB_BF16_POS(B, "x0", "x1")
-                AWQ_RB_MFMA("bf16", 3) AWQ_RB_BF16_FMA(B)
-                AWQ_RB_MFMA("bf16", 4) "v_cvt_pk_bf16_f32 %[o1], %[f0], %[f1]\n\t" AWQ_RB_BF16_POS(C, "x0", "x1")
-                AWQ_RB_MFMA("bf16", 5) AWQ_RB_BF16_FMA(C)
-                AWQ_RB_MFMA("bf16", 6) "v_cvt_pk_bf16_f32 %[o2], %[f0], %[f1]\n\t" AWQ_RB_BF16_POS(D, "x0", "x1")
-                AWQ_RB_MFMA("bf16", 7) AWQ_RB_BF16_FMA(D)
-                "s_nop 0\n\t"
-                "v_cvt_pk_bf16_f32 %[o3], %[f0], %[f1]\n\t"
-                : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [o2] "=&v"(o2), [o3] "=&v"(o3), [e0] "=&v"(e0),
-                  [e1] "=&v"(e1), [f0] "=&v"(f0), [f1] "=&v"(f1), [x0] "=&v"(x0), [x1] "=&v"(x1)
-                : AWQ_RB_AB_OPERANDS, [w0] "v"(w[2 * r]), [w1] "v"(w[2 * r + 1]), [l0] "v"(l0), [l1] "v"(l1),
-                  [g] "v"(magic), [mA] "s"(mask_of(1)), [mB] "s"(mask_of(5)), [mC] "s"(mask_of(6)), [mD] "s"(mask_of(7)),
-                  [sA] "v"(sc[1]), [sB] "v"(sc[5]), [sC] "v"(sc[6]), [sD] "v"(sc[7]), [kA] "v"(off[1]),
-                  [kB] "v"(off[5]), [kC] "v"(off[6]), [kD] "v"(off[7])
+                AWQ_RB_MFMA("bf16", 0) AWQ_RB_E("e0", "w0", "mA") AWQ_RB_E("e1", "w1", "mA")
+                AWQ_RB_MFMA("bf16", 1) AWQ_RB_F("f0", "e0", "A") AWQ_RB_F("f1", "e1", "A")
+                AWQ_RB_MFMA("bf16", 2) AWQ_RB_E("e2", "x0", "mB") AWQ_RB_E("e3", "x1", "mB")
+                AWQ_RB_MFMA("bf16", 3) AWQ_RB_C("o0")
+                AWQ_RB_MFMA("bf16", 4) AWQ_RB_F("f0", "e2", "B") AWQ_RB_F("f1", "e3", "B")
+                AWQ_RB_MFMA("bf16", 5)
+                AWQ_RB_MFMA("bf16", 6) AWQ_RB_C("o1")
+                AWQ_RB_MFMA("bf16", 7)
+                : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [e0] "=&v"(e0), [e1] "=&v"(e1), [e2] "=&v"(e2),
+                  [e3] "=&v"(e3), [f0] "=&v"(f0), [f1] "=&v"(f1)
+                : AWQ_RB_AB_OPERANDS, [w0] "v"(w[2 * r]), [w1] "v"(w[2 * r + 1]), [x0] "v"(x0), [x1] "v"(x1),
+                  [g] "v"(magic), [mA] "s"(mask_of(4)), [mB] "s"(mask_of(0)), [sA] "v"(sc[2]), [sB] "v"(sc[3]),
+                  [kA] "v"(off[2]), [kB] "v"(off[3])
                 : "memory");
-            bfn[1][r] = o0, bfn[5][r] = o1, bfn[6][r] = o2, bfn[7][r] = o3;
-        }
-    }
-    __device__ __forceinline__ void unpack_only(const uint32_t (&w)[8], u32x4 (&bfn)[8]) const {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t w0 = w[2 * r], w1 = w[2 * r + 1];
-            const uint32_t s0[3] = {w0 << 8, w0, w0 >> 12}, s1[3] = {w1 << 8, w1, w1 >> 12};
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                const float e0 = __builtin_bit_cast(float, (s0[src_of(t)] & mask_of(t)) | magic);
-                const float e1 = __builtin_bit_cast(float, (s1[src_of(t)] & mask_of(t)) | magic);
-                bfn[t][r] = BF16::pack2(__builtin_fmaf(e0, sc[t], off[t]), __builtin_fmaf(e1, sc[t], off[t]));
-            }
+            out[2][r] = o0, out[3][r] = o1;
+        } else if ((m & 1) == 0) {
+            // position 1 from left-shifted copies, position 5 from right-shifted ones (kept for the odd row tile)
+            asm volatile(
+                AWQ_RB_MFMA("bf16", 0) "v_lshlrev_b32 %[x0], 8, %[w0]\n\t" "v_lshlrev_b32 %[x1], 8, %[w1]\n\t"
+                AWQ_RB_MFMA("bf16", 1) "v_lshrrev_b32 %[x2], 12, %[w0]\n\t" AWQ_RB_E("e0", "x0", "mA")
+                AWQ_RB_MFMA("bf16", 2) AWQ_RB_E("e1", "x1", "mA") "v_lshrrev_b32 %[x3], 12, %[w1]\n\t"
+                AWQ_RB_MFMA("bf16", 3) AWQ_RB_F("f0", "e0", "A") AWQ_RB_F("f1", "e1", "A")
+                AWQ_RB_MFMA("bf16", 4) AWQ_RB_E("e2", "x2", "mB") AWQ_RB_E("e3", "x3", "mB")
+                AWQ_RB_MFMA("bf16", 5) AWQ_RB_C("o0")
+                AWQ_RB_MFMA("bf16", 6) AWQ_RB_F("f0", "e2", "B") AWQ_RB_F("f1", "e3", "B")
+                AWQ_RB_MFMA("bf16", 7) AWQ_RB_C("o1")
+                : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [e0] "=&v"(e0), [e1] "=&v"(e1), [e2] "=&v"(e2),
+                  [e3] "=&v"(e3), [f0] "=&v"(f0), [f1] "=&v"(f1), [x0] "=&v"(x0), [x1] "=&v"(x1), [x2] "=&v"(x2),
+                  [x3] "=&v"(x3)
+                : AWQ_RB_AB_OPERANDS, [w0] "v"(w[2 * r]), [w1] "v"(w[2 * r + 1]), [g] "v"(magic), [mA] "s"(mask_of(1)),
+                  [mB] "s"(mask_of(5)), [sA] "v"(sc[0]), [sB] "v"(sc[1]), [kA] "v"(off[0]), [kB] "v"(off[1])
+                : "memory");
+            out[0][r] = o0, out[1][r] = o1;
+        } else {
+            // positions 6, 7 from the right-shifted copies
+            asm volatile(
+                AWQ_RB_MFMA("bf16", 0) AWQ_RB_E("e0", "x2", "mA") AWQ_RB_E("e1", "x3", "mA")
+                AWQ_RB_MFMA("bf16", 1) AWQ_RB_F("f0", "e0", "A") AWQ_RB_F("f1", "e1", "A")
+                AWQ_RB_MFMA("bf16", 2) AWQ_RB_E("e2", "x2", "mB") AWQ_RB_E("e3", "x3", "mB")
+                AWQ_RB_MFMA("bf16", 3) AWQ_RB_C("o0")
+                AWQ_RB_MFMA("bf16", 4) AWQ_RB_F("f0", "e2", "B") AWQ_RB_F("f1", "e3", "B")
+                AWQ_RB_MFMA("bf16", 5)
+                AWQ_RB_MFMA("bf16", 6) AWQ_RB_C("o1")
+                AWQ_RB_MFMA("bf16", 7)
+                : AWQ_RB_ACC_OPERANDS, [o0] "=&v"(o0), [o1] "=&v"(o1), [e0] "=&v"(e0), [e1] "=&v"(e1), [e2] "=&v"(e2),
+                  [e3] "=&v"(e3), [f0] "=&v"(f0), [f1] "=&v"(f1)
+                : AWQ_RB_AB_OPERANDS, [x2] "v"(x2), [x3] "v"(x3), [g] "v"(magic), [mA] "s"(mask_of(6)),
+                  [mB] "s"(mask_of(7)), [sA] "v"(sc[2]), [sB] "v"(sc[3]), [kA] "v"(off[2]), [kB] "v"(off[3])
+                : "memory");
+            out[2][r] = o0, out[3][r] = o1;
         }
     }
 };
+
+// The whole unpack of 8 rows of a word column in plain code: the B operands of all eight positions, for the first two
+// half steps of a workgroup (nothing to hide behind yet).
+template <typename T>
+__device__ __forceinline__ void unpack_all(const uint32_t (&w)[8], uint32_t zw, u32x4 sv, u32x4 (&bf)[8]) {
+    UnpackRows<T> u;
+    u.set_group(zw, sv);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        uint32_t o[8];   // by column
+        u.pair(w[2 * r], w[2 * r + 1], o);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) bf[position_of(c)][r] = o[c];
+    }
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_regb_kernel(
@@ -248,8 +279,10 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
     constexpr int BM = 256, BN = 256;
     constexpr int NDMA = 8;              // direct-to-LDS loads per wave and step (4 waves x 8 x 1 KiB = the A tile)
     constexpr int A_SLOTS = 8 * BM;      // 16-byte slots per A buffer
-    constexpr int NBUF = 4;
-    extern __shared__ __attribute__((aligned(16))) u32x4 lds[];   // [NBUF][A_SLOTS]
+    constexpr int NBUF = 3;
+    constexpr int X_SLOTS = 4 * 4 * 64;  // 16-byte slots per B operand buffer: [wave][own position][lane]
+    extern __shared__ __attribute__((aligned(16))) u32x4 lds[];   // [NBUF][A_SLOTS] A tiles, [2][X_SLOTS] B operands
+    u32x4* const xlds = lds + NBUF * A_SLOTS;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -292,11 +325,9 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
         const int kc = (lane & 7) ^ rb_row_swz(row);
         a_off[i] = (min(row, M - 1 - m0) * K + kc * 8) * 2;
     }
-    auto dma_a = [&](int it, int buf) {
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, AWQ_RB_LPTR(lds + buf * A_SLOTS + (wave * NDMA + i) * 64), 16,
-                                                     a_off[i], it * (kRBK * 2), 0, 0);
+    auto dma_a_part = [&](int it, int buf, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, AWQ_RB_LPTR(lds + buf * A_SLOTS + (wave * NDMA + i) * 64), 16,
+                                                 a_off[i], it * (kRBK * 2), 0, 0);
     };
 
     // ---- B: word column j of the wave's 16, rows 8*kq + i of each 32-row half step ---------------------------
@@ -304,10 +335,8 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
     int w_off[8];   // byte offsets of the lane's 8 rows inside a half step
 #pragma unroll
     for (int i = 0; i < 8; ++i) w_off[i] = ((kq * 8 + i) * words + gwc) * 4;
-    auto load_half = [&](int it, int ks, uint32_t (&w)[8]) {
-        const int so = (it * kRBK + ks * 32) * words * 4;   // uniform
-#pragma unroll
-        for (int i = 0; i < 8; ++i) w[i] = __builtin_amdgcn_raw_buffer_load_b32(rs_w, w_off[i], so, 0);
+    auto load_word = [&](int half_step, int i) {   // half step = 2 * step + half
+        return __builtin_amdgcn_raw_buffer_load_b32(rs_w, w_off[i], half_step * 32 * words * 4, 0);
     };
     const int steps_per_group = g / kRBK;   // g % 64 == 0
     auto load_group = [&](int grp, uint32_t& z, u32x4& sv) {
@@ -326,37 +355,52 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    FragUnpack<T> up;
-    up.init();
-
-    // One K step per pass, two half steps of 64 MFMAs each (row-tile-major: an A fragment serves 8 MFMAs in a row and
-    // is read from LDS two fragments ahead, into a ring of four).  While half step h runs, the B operands of half step
-    // h+1 are built behind its MFMAs.  Global loads are dealt out over the row tiles, one or two after each (a wave
-    // that issues its 26 loads of a step back to back stalls on the memory pipeline's queue with its MFMAs waiting
-    // behind): the two words a row tile has just consumed are re-loaded for the same half of the next step (a full
-    // step ahead), and one eighth of this wave's share of the A tile of step it+2 goes out.  Four LDS buffers: the
-    // barrier sits in the middle of a step, so a wave can be filling step i+2's buffer while another still reads step
-    // i-1's -- never step i-2's, which is the same buffer.  Loads past the end of K are not guarded: the buffer
+    // Half step h = 2 * step + half runs 8 row tiles of 8 MFMAs on the B operands bf[h % 2] (row-tile-major: an A
+    // fragment serves 8 MFMAs in a row and is read from LDS two fragments ahead, into a ring of four).  Behind its
+    // MFMAs the wave builds its four positions' operands for half step h + 2 from the words ws[h % 2], stores them to
+    // the B operand buffer xlds[h % 2] after the last row tile, and -- once every wave has done so: the barrier after
+    // row tile 0 of half step h + 1 -- both waves of a pair read all eight back into bf[h % 2], which half step h has
+    // just released.
+    // Global loads are dealt out over the row tiles, one to three after each (a wave that issues its 26 loads of a
+    // step back to back stalls on the memory pipeline's queue with its MFMAs waiting behind): the two words a row
+    // tile has just consumed are re-loaded for half step h + 4 (a full step until they are used), and one eighth of
+    // this wave's share of the A tile of step + 2 goes out behind row tiles 1..7 of the first half and row tile 1
+    // of the second -- after the step's first barrier, which every wave reaches only when it is done with step - 1,
+    // whose LDS buffer (three in rotation) this fills.  The A tile of step + 1 is complete at the second barrier of a
+    // step: 23 loads have been issued since its last part (25 if the compiler puts that part in front of the two words
+    // that go out behind the same row tile).  Loads past the end of K are not guarded: the buffer
     // descriptors return zero (or another row's x, in bounds) and nothing uses them.
-    if (it_begin < it_end) {
-        uint32_t hi[8], lo_n[8], z_n;   // second-half words of this step, first-half words and group of the next
+    auto main_loop = [&](auto role) {
+        constexpr int ROLE = decltype(role)::value;
+        FragUnpack<T, ROLE> up;
+        FragUnpack<T, 1 - ROLE> other;   // for the partner's position list only
+        (void)other;
+        up.init();
+        uint32_t ws[2][8], z_n;   // words of half steps h + 2 (parity h % 2), group of the next step
         u32x4 s_n;
-        u32x4 bf[2][8], af[4];
-        dma_a(it_begin, 0);
-        dma_a(it_begin + 1, 1);
+        u32x4 bf[2][8], af[4], own[4];
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma_a_part(it_begin, 0, i);
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma_a_part(it_begin + 1, 1, i);
         {
-            uint32_t lo[8], z;
+            uint32_t w0[8], w1[8], z;
             u32x4 sv;
-            load_half(it_begin, 0, lo);
-            load_half(it_begin, 1, hi);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w0[i] = load_word(2 * it_begin, i), w1[i] = load_word(2 * it_begin + 1, i);
             load_group(it_begin / steps_per_group, z, sv);
-            load_half(it_begin + 1, 0, lo_n);
-            up.set_group(z, sv);
-            up.unpack_only(lo, bf[0]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ws[0][i] = load_word(2 * it_begin + 2, i), ws[1][i] = load_word(2 * it_begin + 3, i);
+            load_group((it_begin + 1) / steps_per_group, z_n, s_n);
+            unpack_all<T>(w0, z, sv, bf[0]);
+            unpack_all<T>(w1, z, sv, bf[1]);
         }
-        // group of step it+2 (loaded in the middle of step it), without a division per step
+        // group of step + 2 (loaded at the start of a step), without a division per step
         int grp_nn = (it_begin + 2) / steps_per_group, cnt_nn = (it_begin + 2) % steps_per_group;
-        load_group((it_begin + 1) / steps_per_group, z_n, s_n);
+        const int x_own = wave * 256 + lane, x_partner = (wave ^ 2) * 256 + lane;
+        // the first half step reads the operands of the second back like any other: leave this wave's four there
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xlds[X_SLOTS + x_own + i * 64] = bf[1][FragUnpack<T, ROLE>::own(i)];
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0F70);
         asm volatile("" ::: "memory");
@@ -365,26 +409,17 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
         af[0] = lds[a_rd[0]];
         af[1] = lds[a_rd[0] + 128];
         for (int it = it_begin; it < it_end; ++it) {
-            const int nb = (buf + 1) & 3;
+            const int nb = buf == NBUF - 1 ? 0 : buf + 1, nnb = nb == NBUF - 1 ? 0 : nb + 1;
             const u32x4* abase = lds + buf * A_SLOTS;
             const u32x4* anext = lds + nb * A_SLOTS;
-            const int so_hi = ((it + 1) * kRBK + 32) * words * 4, so_lo = (it + 2) * kRBK * words * 4;   // uniform
-            const int so_a = (it + 2) * (kRBK * 2);
-            u32x4* a_dst = lds + ((buf + 2) & 3) * A_SLOTS + wave * NDMA * 64;
+            // the operands built during this step belong to step + 1
+            up.set_group(z_n, s_n);
+            load_group(grp_nn, z_n, s_n);
+            if (++cnt_nn == steps_per_group) cnt_nn = 0, ++grp_nn;
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                if (ks == 1) {
-                    // The A tile of step it+1 has landed in every wave: its last part went out behind the last row
-                    // tile of the first half of step it-1, and 2 + 8 + 8 + NDMA loads have been issued since.
-                    // (A bare barrier: __syncthreads() would also wait for those.)
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(18 + NDMA) : "memory");
-                    __builtin_amdgcn_s_barrier();
-                    asm volatile("" : "+v"(z_n), "+v"(s_n));   // not before the barrier
-                    up.set_group(z_n, s_n);
-                    load_group(grp_nn, z_n, s_n);
-                    if (++cnt_nn == steps_per_group) cnt_nn = 0, ++grp_nn;
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                u32x4* xbuf = xlds + ks * X_SLOTS;
 #pragma unroll
                 for (int m = 0; m < 8; ++m) {
                     const int f = ks * 8 + m;
@@ -393,23 +428,41 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
                         af[(f + 2) & 3] = abase[a_rd[(f + 2) >> 3] + ((f + 2) & 7) * 128];
                     else
                         af[(f + 2) & 3] = anext[a_rd[0] + (f + 2 - 16) * 128];
-                    if (ks == 0) up.row_tile(m, acc[m], af[f & 3], bf[0], hi, bf[1]);
-                    else up.row_tile(m, acc[m], af[f & 3], bf[1], lo_n, bf[0]);
-                    if (m & 1) {
-                        uint32_t(&w)[8] = ks == 0 ? hi : lo_n;
-                        w[m - 1] = __builtin_amdgcn_raw_buffer_load_b32(rs_w, w_off[m - 1], ks == 0 ? so_hi : so_lo, 0);
-                        w[m] = __builtin_amdgcn_raw_buffer_load_b32(rs_w, w_off[m], ks == 0 ? so_hi : so_lo, 0);
+                    up.row_tile(m, acc[m], af[f & 3], bf[ks], ws[ks], own);
+                    if (m == 0) {
+                        // Every wave has stored its operands of half step h + 1 (at the end of half step h - 1; the
+                        // stores completed behind row tile 0) -- and, in the second half, its part of the A tile of
+                        // step + 1.  A bare barrier: __syncthreads() would also wait for this step's own loads.
+                        if (ks == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        else asm volatile("s_waitcnt vmcnt(23) lgkmcnt(0)" ::: "memory");
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
+                    } else if (m <= 4) {
+                        // operands of half step h + 1, written at the end of half step h - 1 into the other buffer
+                        const u32x4* xprev = xlds + (1 - ks) * X_SLOTS;
+                        const int i = m - 1;
+                        bf[1 - ks][FragUnpack<T, ROLE>::own(i)] = xprev[x_own + i * 64];
+                        bf[1 - ks][FragUnpack<T, 1 - ROLE>::own(i)] = xprev[x_partner + i * 64];
                     }
-                    if (ks == 0)
-                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, AWQ_RB_LPTR(a_dst + m * 64), 16, a_off[m], so_a, 0, 0);
+                    if (m & 1) {
+                        ws[ks][m - 1] = load_word(2 * it + ks + 4, m - 1);
+                        ws[ks][m] = load_word(2 * it + ks + 4, m);
+                    }
+                    if (m >= 1 && (ks == 0 || m == 1)) dma_a_part(it + 2, nnb, ks == 0 ? m - 1 : 7);
                     __builtin_amdgcn_sched_barrier(0);
                 }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) xbuf[x_own + i * 64] = own[i];
             }
             buf = nb;
         }
         // the last MFMAs' results: 4 passes to write, read by the epilogue below
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
+    };
+    if (it_begin < it_end) {
+        if ((wave >> 1) == 0) main_loop(std::integral_constant<int, 0>{});
+        else main_loop(std::integral_constant<int, 1>{});
     }
 
     // acc[m][t][i]: row wm0 + 16*m + 4*kq + i, column wn0 + 8*j + column_of(t)
@@ -473,7 +526,7 @@ hipError_t launch_regb(const void* x, const int32_t* qweight, const void* qscale
     plan.act = act;
     float* partials =
         workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes) : nullptr;
-    const size_t lds = (size_t)4 * 8 * 256 * 16;  // 128 KiB
+    const size_t lds = (size_t)(3 * 8 * 256 + 2 * 4 * 4 * 64) * 16;  // 96 KiB of A tiles + 32 KiB of B operands
     auto kern = gemm_regb_kernel<T>;
     static bool raised = false;  // once per process and instantiation
     if (!raised) {

@@ -91,14 +91,15 @@ def test_gemm_bias_and_determinism(dtype):
     assert torch.count_nonzero(awq_gemm_variant(torch.zeros_like(xd), *dev, v, 4)) == 0
 
 
+@pytest.mark.parametrize("form", ["p", "r"])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_gemm_tail_tiles_split(dtype):
+def test_gemm_tail_tiles_split(dtype, form):
     # 9 x 30 = 270 tiles of 256 x 256 (ragged in M and N): 256 whole tiles and a tail of 14 whose K range is cut;
     # the mixed launch must agree with the oracle, with the uncut launch bit for bit where no cut applies,
-    # and be bit-stable
+    # and be bit-stable -- for the pipelined kernel (p) and the one that builds its B operands in registers (r)
     L = _lib.lib()
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
-    tail, whole = names.index("256x256pt"), names.index("256x256p")
+    tail, whole = names.index(f"256x256{form}t"), names.index(f"256x256{form}")
     M, K, N = 2300, 256, 7672
     p = random_packed(K, N, 128, dtype, seed=95)
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
@@ -109,7 +110,7 @@ def test_gemm_tail_tiles_split(dtype):
     y1 = awq_gemm_variant(xd, *dev, whole, 1, bias=bd)
     _check(y1, xb, p, dtype, o.to_dtype_f32(bias, dtype))
     for split in (2, 4):
-        print(f"gemm tail split={split} {dtype}", flush=True)
+        print(f"gemm tail {form} split={split} {dtype}", flush=True)
         y = awq_gemm_variant(xd, *dev, tail, split, bias=bd)
         torch.cuda.synchronize()
         _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
@@ -153,10 +154,38 @@ def test_linear_large_m_equals_dequantise_then_matmul(dtype, M, K, N, g):
     L = _lib.lib()
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
     fused = awq_gemm_variant(xd, *dev, names.index("256x256p"), 1)
+    fused_r = awq_gemm_variant(xd, *dev, names.index("256x256r"), 1)
     two_step = torch.matmul(xd, nq.awq_dequantize_transposed(*dev).t())
-    for other in (fused, two_step):
+    for other in (fused, fused_r, two_step):
         err = (y.float() - other.float()).abs().max().item() / other.float().abs().max().item()
         assert err <= (2e-3 if dtype == "f16" else 1.6e-2), err     # both round an fp32 sum of the same products once
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,K,N,g,split", [(300, 1024, 520, 128, 1), (777, 2048, 1032, 64, 3), (256, 64, 256, 64, 1),
+                                            (1000, 768, 2048, 768, 2), (513, 512, 264, 32, 1)])
+def test_gemm_register_b_kernel_equals_pipelined(dtype, M, K, N, g, split):
+    # the two 256 x 256 kernels multiply the same rounded weights (on MFMAs of different depth, so the fp32 sums may
+    # differ in their last bits): ragged M and N, K of one step, odd K slices, every group size (g = 32 runs the
+    # pipelined kernel under the r names, bit for bit), with bias
+    print(f"gemm r vs p {dtype} M={M} K={K} N={N} g={g} split={split}", flush=True)
+    L = _lib.lib()
+    names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
+    p = random_packed(K, N, g, dtype, seed=K + N + g)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    xb = make_x(M, K, dtype, seed=M)
+    xd = to_dev(xb, dtype)
+    bias = np.linspace(-1, 1, N).astype(np.float32)
+    bd = to_dev(o.to_bits16(bias, dtype), dtype)
+    for form in ("", "t"):
+        yp = awq_gemm_variant(xd, *dev, names.index("256x256p" + form), split, bias=bd)
+        yr = awq_gemm_variant(xd, *dev, names.index("256x256r" + form), split, bias=bd)
+        torch.cuda.synchronize()
+        if g % 64 != 0:
+            assert torch.equal(yp, yr), form
+        diff = (yp.float() - yr.float()).abs().max().item() / yp.float().abs().max().item()
+        assert diff <= (1e-3 if dtype == "f16" else 8e-3), (form, diff)
+        _check(yr, xb, p, dtype, o.to_dtype_f32(bias, dtype))
 
 
 def test_gemm_prefill_full_size_bf16():
@@ -174,8 +203,9 @@ def test_gemm_prefill_full_size_bf16():
 def test_gemm_largest_shapes_properties(M, K, N):
     """The prefill shapes at their real sizes (Qwen3-8B MLP at M = 512 / 2048 / 8192, Qwen3-32B o_proj at a 4096-token
     prefill and gate/up at a ragged M), too big for the CPU oracle: checked through size-independent properties, on
-    the default dispatch and on the pipelined fused kernel forced in both of its forms (every tile whole; the tiles
-    of the last round cut along K with the plan's split).  (1) rows sampled across every workgroup tile equal the
+    the default dispatch and on both 256 x 256 fused kernels (the pipelined one, p, and the one that builds its B
+    operands in registers, r) forced in both of their forms (every tile whole; the tiles of the last round cut along K
+    with the plan's split).  (1) rows sampled across every workgroup tile equal the
     fp32 matmul of those rows with the dequantised weight (itself bit-exact against the oracle); (2) the same rows
     pushed through alone (another tile shape) agree too; (3) run-to-run bit-stable; (4) a zero row gives exact zeros."""
     print(f"gemm properties M={M} K={K} N={N} bf16", flush=True)
@@ -196,7 +226,10 @@ def test_gemm_largest_shapes_properties(M, K, N):
     runs = [("default " + names[v.value] + f" split {sp.value}", lambda: nq.awq_gemm(x, qw, sc, qz, 8)),
             ("256x256p split 1", lambda: awq_gemm_variant(x, qw, sc, qz, names.index("256x256p"), 1)),
             (f"256x256pt split {max(sp.value, 2)}",
-             lambda: awq_gemm_variant(x, qw, sc, qz, names.index("256x256pt"), max(sp.value, 2)))]
+             lambda: awq_gemm_variant(x, qw, sc, qz, names.index("256x256pt"), max(sp.value, 2))),
+            ("256x256r split 1", lambda: awq_gemm_variant(x, qw, sc, qz, names.index("256x256r"), 1)),
+            (f"256x256rt split {max(sp.value, 2)}",
+             lambda: awq_gemm_variant(x, qw, sc, qz, names.index("256x256rt"), max(sp.value, 2)))]
     for what, run in runs:
         print(f"  {what}", flush=True)
         y = run()
