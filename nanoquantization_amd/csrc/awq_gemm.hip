@@ -208,8 +208,9 @@ static const GemmVariant kGemmVariants[] = {
     {"32x256", 32, 256, 4},
     {"256x256p", 256, 256, 8},   // the software-pipelined kernel of awq_gemm_pipe.hip, every tile cut split_k ways
     {"256x256pt", 256, 256, 8},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
-    // awq_gemm_regb.hip: B operands built in registers, the default above 128 rows; group sizes that are not multiples of
-    // 64 run the pipelined kernel under these names too
+    // awq_gemm_regb.hip: B operands built in registers; the default entry points take it in place of the pipelined
+    // kernel for fp16 on 256 tiles or more (see gemm_dispatch); group sizes that are not multiples of 64 run the
+    // pipelined kernel under these names too
     {"256x256r", 256, 256, 4},   // every tile cut split_k ways
     {"256x256rt", 256, 256, 4},  // split_k cuts only the tiles beyond the last full round of CUs
 };
@@ -267,15 +268,13 @@ static size_t gemm_ws_bytes(int64_t M, int64_t N, int64_t K, int variant, int sp
     return kCounterBytes + (size_t)splits * M * N * sizeof(float);
 }
 
-// Tile shape and split for the default entry point.  Large M: the 256 x 256 kernel that builds its B operands in
-// registers (on one box, M = 8192 x 4096 x 12288: fp16 855-865 us against the pipelined kernel's 935, bf16 804
-// against 801, 12288 x 4096 bf16 774 against 797), K split so that the tiles cover the CUs once (a split costs
-// one more pass over the fp32 partials, which is cheap next to an idle CU).  Small M: narrower tiles of the plain
-// kernel.
+// Tile shape and split for the default entry point.  Large M: the pipelined 256 x 256 kernel with two
+// wavefronts per SIMD, K split so that the tiles cover the CUs once (a split costs one more pass over
+// the fp32 partials, which is cheap next to an idle CU).  Small M: narrower tiles of the plain kernel.
 static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
     const int kCUs = 256;
     // indices into kGemmVariants
-    constexpr int kPipe8 = kRegbVariant;
+    constexpr int kPipe8 = kPipeVariant;
     int v;
     if (M <= 32) v = k32x256;
     else if (M <= 64) v = k64x256;
@@ -296,7 +295,7 @@ static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_
             const int64_t t = cdiv(R * c, kCUs) * (cdiv(steps, c) + 5);
             if (t < best_t) best_t = t, best_s = c;
         }
-        if (best_s > 1 && best_t * 10 <= steps * 9) v = kRegbTailVariant, s = best_s;
+        if (best_s > 1 && best_t * 10 <= steps * 9) v = kPipeTailVariant, s = best_s;
     }
     if (!is_tile256(v)) {
         // Narrow tiles (up to 128 rows): two workgroups of the 128x128 and 32x256 forms share a CU, one of the 64x256
@@ -326,7 +325,7 @@ static void pick_gemm_pipe(int64_t M, int64_t N, int64_t K, int* variant, int* s
 static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, const void* qscales,
                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
-                         void* stream, int variant, int split_k, int act = 0) {
+                         void* stream, int variant, int split_k, int act = 0, bool planned = false) {
     // prefetch hints pending on this thread were meant for this call; the GEMM fills the chip, so they are dropped
     // (before any check: an error return must not leave them for an unrelated later launch)
     PrefetchRegions dropped;
@@ -349,6 +348,13 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     if (act && (bias || N % 16 != 0 || !is_tile256(variant))) {
         set_error("%s: the gated epilogue takes no bias, needs N %% 16 == 0 and runs on the pipelined kernel", fn);
         return AWQ_ERR_UNSUPPORTED;
+    }
+    // A planned (not forced) launch of the pipelined kernel in fp16 on at least one full round of tiles runs the
+    // register-operand kernel instead: M = 8192 x 4096 x 12288 on one box 855 against 935 us (bf16: 804 against 801,
+    // and 6-15 % slower on the short K slices of 96 or 384 tiles -- its prologue unpacks two half steps unaided).
+    if (planned && dtype == AWQ_F16 && g % 64 == 0 && cdiv(M, 256) * cdiv(N, 256) >= 256) {
+        if (variant == kPipeVariant) variant = kRegbVariant;
+        else if (variant == kPipeTailVariant) variant = kRegbTailVariant;
     }
     const GemmVariant& gv = kGemmVariants[variant];
     if (cdiv(M, gv.BM) > 65535) {
@@ -458,7 +464,7 @@ extern "C" int awq_gemm(const void* x, const int32_t* qweight, const void* qscal
     int v = 0, s = 1;
     if (K >= awq::kBK && N >= 8 && M >= 1) awq::pick_gemm(M, N, K, &v, &s);
     return awq::gemm_dispatch("awq_gemm", x, qweight, qscales, qzeros, bias, y, M, N, K, group_size,
-                              dtype, workspace, workspace_bytes, stream, v, s);
+                              dtype, workspace, workspace_bytes, stream, v, s, 0, true);
 }
 
 // 65..128 rows go to the GEMV (blocks of 16 rows) on weights up to this size, see kGemvMaxRows in awq_gemv.hip
@@ -494,10 +500,10 @@ extern "C" int awq_linear_swiglu(const void* x, const int32_t* qweight, const vo
     if (M >= 1 && M <= 64 && staged)
         return awq_gemv_swiglu(x, qweight, qscales, qzeros, y, M, N, K, group_size, dtype, workspace,
                                workspace_bytes, stream);
-    int v = awq::kRegbVariant, s = 1;
+    int v = awq::kPipeVariant, s = 1;
     if (K >= awq::kBK && N >= 16 && M >= 1) awq::pick_gemm_pipe(M, N, K, &v, &s);
     return awq::gemm_dispatch("awq_linear_swiglu", x, qweight, qscales, qzeros, nullptr, y, M, N, K, group_size,
-                              dtype, workspace, workspace_bytes, stream, v, s, 1);
+                              dtype, workspace, workspace_bytes, stream, v, s, 1, true);
 }
 
 extern "C" int awq_linear(const void* x, const int32_t* qweight, const void* qscales,

@@ -188,6 +188,29 @@ def test_gemm_register_b_kernel_equals_pipelined(dtype, M, K, N, g, split):
         _check(yr, xb, p, dtype, o.to_dtype_f32(bias, dtype))
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_default_kernel_on_full_rounds(dtype):
+    # 16 x 17 = 272 tiles: the default entry point runs the register-operand kernel in fp16 and the pipelined one in
+    # bf16, both with the planned tail split -- bit for bit what the forced variants give
+    import ctypes
+    L = _lib.lib()
+    names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
+    M, K, N = 4096, 512, 4352
+    v, sp = ctypes.c_int(), ctypes.c_int()
+    assert L.awq_gemm_plan(M, N, K, ctypes.byref(v), ctypes.byref(sp)) == 0
+    assert names[v.value] in ("256x256p", "256x256pt")
+    print(f"gemm default on full rounds {dtype}: plan {names[v.value]} split {sp.value}", flush=True)
+    p = random_packed(K, N, 128, dtype, seed=123)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    xd = to_dev(make_x(M, K, dtype, seed=124), dtype)
+    y = nq.awq_gemm(xd, *dev, 8)
+    forced = names[v.value].replace("p", "r") if dtype == "f16" else names[v.value]
+    assert torch.equal(y, awq_gemm_variant(xd, *dev, names.index(forced), sp.value)), forced
+    rows = torch.arange(0, M, 97, device="cuda")
+    ref = xd[rows].float() @ nq.awq_dequantize(*dev).float()
+    assert ((y[rows].float() - ref).abs().max() / ref.abs().max()).item() <= TIGHT[dtype]
+
+
 def test_gemm_prefill_full_size_bf16():
     # Qwen3-8B MLP gate/up at M=512, its real size (oracle: numpy float64 matmul, a few seconds)
     print("gemm full size M=512 4096x12288 bf16", flush=True)
