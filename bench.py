@@ -259,6 +259,28 @@ def main():
             "workload": "cfg3: Qwen3-8B MLP shapes, bf16, M in {512,2048,8192}; the fused dequant + MFMA kernel "
                         "(default dispatch at every M)",
             "cases": fused}
+        # the same shapes in fp16 at the row counts that fill whole rounds of tiles: the default dispatch runs the
+        # kernel that builds its B operands in registers there (awq::gemm_regb_kernel)
+        hdt = torch.float16
+        fused16 = {}
+        for (K, N) in ((4096, 12288), (12288, 4096)):
+            w = rand_packed(K, N, hdt, dev)
+            for M in (2048, 8192):
+                x = torch.randn(M, K, device=dev).to(hdt)
+                fn = lambda: [nq.awq_gemm(x, *w, 8) for _ in range(4)]
+                us = time_graph(fn, 5, 1) * 1e3 / 4
+                tf = 2.0 * M * N * K / us / 1e6
+                fused16[f"M{M}_{K}x{N}"] = {"us": round(us, 1), "TFLOPs": round(tf, 1),
+                                            "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4)}
+            del w
+        best16 = max(v["TFLOPs"] for v in fused16.values())
+        out["roofline_prefill_f16"] = {
+            "kernel": "awq::gemm_regb_kernel<F16> (launches of 256 output tiles or more: all but M = 2048 on 12288x4096, which "
+                      "runs awq::gemm_pipe_kernel<F16,2,4>)",
+            "bound": "mfma", "achieved": best16, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": best16 / MFMA_PEAK_TFLOPS,
+            "workload": "cfg3's shapes with fp16 activations and scales, M in {2048, 8192}, default dispatch",
+            "cases": fused16}
 
         # ---------------- extra: dequantise kernel ------------------------------------------------------
         K, N = 4096, 12288
