@@ -349,12 +349,16 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         set_error("%s: the gated epilogue takes no bias, needs N %% 16 == 0 and runs on the pipelined kernel", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
-    // A planned (not forced) launch of the pipelined kernel in fp16 on at least one full round of tiles runs the
-    // register-operand kernel instead: M = 8192 x 4096 x 12288 on one box 855 against 935 us (bf16: 804 against 801,
-    // and 6-15 % slower on the short K slices of 96 or 384 tiles -- its prologue unpacks two half steps unaided).
-    if (planned && dtype == AWQ_F16 && g % 64 == 0 && cdiv(M, 256) * cdiv(N, 256) >= 256) {
-        if (variant == kPipeVariant) variant = kRegbVariant;
-        else if (variant == kPipeTailVariant) variant = kRegbTailVariant;
+    // A planned (not forced) launch of the pipelined kernel whose work items -- whole tiles plus K slices of the tail
+    // tiles -- outnumber the CUs runs the register-operand kernel instead: it walks a workgroup's items as one run of
+    // K steps (no prologue, no dispatch between tiles).  M = 8192 x 4096 x 12288: 729 against 822 us in fp16, 774
+    // against 800 in bf16; 16384 x 1024 x 6144: 227 / 234 against 256 / 261.  With one item per workgroup its heavier
+    // start costs 3-11 % in bf16 (fp16: level from 256 items on, its unpack being the cheaper one).
+    if (planned && g % 64 == 0 && N % 128 == 0 && (variant == kPipeVariant || variant == kPipeTailVariant)) {
+        const PipePlan pp = make_pipe_plan(M, N, K, split_k, variant == kPipeTailVariant);
+        const int64_t items = (int64_t)pp.full_tiles + (int64_t)pp.tail_tiles * pp.splits;
+        if (items > 256 || (dtype == AWQ_F16 && items == 256))
+            variant = variant == kPipeVariant ? kRegbVariant : kRegbTailVariant;
     }
     const GemmVariant& gv = kGemmVariants[variant];
     if (cdiv(M, gv.BM) > 65535) {
@@ -389,7 +393,8 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
             break;
         case kRegbVariant:
         case kRegbTailVariant:
-            e = g % 64 == 0 ? launch_gemm_regb(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+            // (group sizes below 64 and widths that cut a wave's 16 word columns run the pipelined kernel)
+            e = g % 64 == 0 && N % 128 == 0 ? launch_gemm_regb(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
                                                workspace, split_k, variant == kRegbTailVariant, s, act)
                             : launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
                                                workspace, split_k, variant == kRegbTailVariant, s, act);

@@ -19,6 +19,8 @@
 // 0x4B000000 (value 2^23 + q * 2^e), so  fma(f, s * 2^-e, -(2^(23-e) + z) * s) = (q - z) * s
 // exactly: the product and the constant have at most 24 significant bits each, and the sum has at
 // most 13.  Nibbles 0-1 and 5-7 are brought to those positions by one shift of the word each.
+#include <type_traits>
+
 #include "awq_common.hpp"
 #include "awq_gemm_parts.hpp"
 
@@ -294,32 +296,40 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
             const int n = n0 + wn0 + b * 32 + li;
             bv[b] = (bias && n < N) ? T::to_f32(bias[n]) : 0.f;
         }
+        // one code path per epilogue, chosen once (merged, every value would pay for the bias rounding and the gate
+        // product whether wanted or not; conversions run at a quarter of the ALU rate)
+        auto rows = [&](auto mode) {
+            constexpr int MODE = decltype(mode)::value;   // 0: plain, 1: + bias, 2: gated
 #pragma unroll
-        for (int a = 0; a < TM; ++a) {
+            for (int a = 0; a < TM; ++a) {
 #pragma unroll
-            for (int b = 0; b < TN; ++b)
+                for (int b = 0; b < TN; ++b)
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    stage[((v >> 2) * 8 + kb2 * 4 + (v & 3)) * PITCH + b * 32 + li] =
-                        T::from_f32(bias ? add_bias<T>(acc[a][b][v], bv[b]) : acc[a][b][v]);
+                    for (int v = 0; v < 16; ++v)
+                        stage[((v >> 2) * 8 + kb2 * 4 + (v & 3)) * PITCH + b * 32 + li] =
+                            T::from_f32(MODE == 1 ? add_bias<T>(acc[a][b][v], bv[b]) : acc[a][b][v]);
 #pragma unroll
-            for (int j = 0; j < 32 / RPP; ++j) {
-                const int row = RPP * j + lane / LPR, chunk = lane % LPR;
-                const u32x4 val = *reinterpret_cast<const u32x4*>(stage + row * PITCH + chunk * 8);
-                const int m = m0 + wm0 + a * 32 + row, n = n0 + wn0 + chunk * 8;
-                if (plan.act) {
-                    // a lane holds one word of 8 columns; even words are gate columns, the next word the up
-                    // columns of the same outputs (N % 16 == 0, so a pair is in range or out of range together)
-                    u32x4 other;
+                for (int j = 0; j < 32 / RPP; ++j) {
+                    const int row = RPP * j + lane / LPR, chunk = lane % LPR;
+                    const u32x4 val = *reinterpret_cast<const u32x4*>(stage + row * PITCH + chunk * 8);
+                    const int m = m0 + wm0 + a * 32 + row, n = n0 + wn0 + chunk * 8;
+                    if constexpr (MODE == 2) {
+                        // a lane holds one word of 8 columns; even words are gate columns, the next word the up
+                        // columns of the same outputs (N % 16 == 0, so a pair is in range or out of range together)
+                        u32x4 other;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(val[i], 1);
-                    if (m < M && n < N)
-                        swiglu_pair_store<T>(val, other, chunk & 1, y + (size_t)m * (N >> 1) + ((n & ~15) >> 1));
-                } else if (m < M && n < N) {
-                    *reinterpret_cast<u32x4*>(y + (size_t)m * N + n) = val;
+                        for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(val[i], 1);
+                        if (m < M && n < N)
+                            swiglu_pair_store<T>(val, other, chunk & 1, y + (size_t)m * (N >> 1) + ((n & ~15) >> 1));
+                    } else if (m < M && n < N) {
+                        *reinterpret_cast<u32x4*>(y + (size_t)m * N + n) = val;
+                    }
                 }
             }
-        }
+        };
+        if (plan.act) rows(std::integral_constant<int, 2>{});
+        else if (bias) rows(std::integral_constant<int, 1>{});
+        else rows(std::integral_constant<int, 0>{});
     } else {
         // fp32 partial of this K slice, tile-compact: [slice][tail tile][256][256].  Rows and columns past
         // M and N are stored too (they stay inside the tile's slot); the reduction pass masks them.

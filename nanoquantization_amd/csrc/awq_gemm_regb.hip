@@ -43,6 +43,7 @@ namespace awq {
 namespace {
 
 constexpr int kRBK = 64;
+constexpr int kResidentWgs = 256;   // one workgroup per CU (128 KiB of LDS each)
 
 #define AWQ_RB_GPTR(p) ((__attribute__((address_space(1))) const void*)(p))
 #define AWQ_RB_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -288,60 +289,94 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
     const int j = lane & 15, kq = lane >> 4;
-    // Workgroups [0, full_tiles) own a whole output tile each; the rest share the tail tiles, `splits`
-    // K slices per tile, slice-major.
-    int tile = blockIdx.x, split = 0;
-    const bool whole = (int)blockIdx.x < plan.full_tiles;
-    if (!whole) {
-        const int r = blockIdx.x - plan.full_tiles;
-        split = r / plan.tail_tiles;
-        tile = plan.full_tiles + (r - split * plan.tail_tiles);
-    }
-    const int m0 = (tile / plan.tiles_n) * BM, n0 = (tile % plan.tiles_n) * BN;
     const int words = N >> 3;
     const int total_iters = K / kRBK;
-    const int it_begin = whole ? 0 : split * plan.iters_per_split;
-    const int it_end = whole ? total_iters : min(it_begin + plan.iters_per_split, total_iters);
+    const int groups = K / g;
+    const int steps_per_group = g / kRBK;   // g % 64 == 0
 
-    // Global reads go through buffer descriptors: a 32-bit per-lane offset (loop-invariant) plus a scalar offset per
-    // step, no 64-bit address arithmetic in the loop, and reads past the end of a tensor return zero.
+    // Work items [0, full_tiles) are whole output tiles; the rest are the tail tiles, `splits` K slices per tile,
+    // slice-major.  A workgroup stays resident (one per CU) and takes items blockIdx.x, blockIdx.x + gridDim.x, ...
+    // as ONE run of K steps: the loads of a step are always those of the step two ahead, which near the end of an
+    // item is a step of the next one, so an item starts with its operands in place -- no prologue, no load latency,
+    // no dispatch between tiles; only the accumulators are stored and cleared in between.
+    const int items = plan.full_tiles + plan.tail_tiles * plan.splits;
+    struct Item {
+        int tile, split, m0, n0, it_begin, it_end;
+        bool whole;
+    };
+    auto decode = [&](int item) {
+        Item d;
+        d.tile = item, d.split = 0;
+        d.whole = item < plan.full_tiles;
+        if (!d.whole) {
+            const int r = item - plan.full_tiles;
+            d.split = r / plan.tail_tiles;
+            d.tile = plan.full_tiles + (r - d.split * plan.tail_tiles);
+        }
+        d.m0 = (d.tile / plan.tiles_n) * BM, d.n0 = (d.tile % plan.tiles_n) * BN;
+        d.it_begin = d.whole ? 0 : d.split * plan.iters_per_split;
+        d.it_end = d.whole ? total_iters : min(d.it_begin + plan.iters_per_split, total_iters);
+        return d;
+    };
+
+    // Global reads go through buffer descriptors: a 32-bit per-lane offset (the same for every item) plus a scalar
+    // offset per step, no 64-bit address arithmetic in the loop.  What depends on the item -- the tile's first row of
+    // x, the wave's first word column -- is in the descriptor's base, and its size ends the tensor: rows past M read
+    // zero.  (N % 128 == 0, so a wave's 16 word columns are inside the row or all outside; a window outside is moved
+    // onto the row's last 16 words, whose results nobody stores.)
     auto rsrc = [](const void* base, size_t bytes) {
         return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0,
                                                  (int)(bytes < 0x7fffffffu ? bytes : 0x7fffffffu), 0x00020000);
     };
-    const int groups = K / g;
-    const __amdgpu_buffer_rsrc_t rs_a = rsrc(x + (size_t)m0 * K, (size_t)(M - m0) * K * 2);
-    const __amdgpu_buffer_rsrc_t rs_w = rsrc(qweight, (size_t)K * words * 4);
-    const __amdgpu_buffer_rsrc_t rs_z = rsrc(qzeros, (size_t)groups * words * 4);
-    const __amdgpu_buffer_rsrc_t rs_s = rsrc(scales, (size_t)groups * words * 16);
+    // the cursor: the step whose operands are being loaded (two ahead of the one that computes)
+    __amdgpu_buffer_rsrc_t pf_a = rsrc(x, 0), pf_w = pf_a, pf_z = pf_a, pf_s = pf_a;
+    int pf_item = 0, pf_it = 0, pf_end = 0, pf_grp = 0, pf_cnt = 0;
+    auto open_cursor = [&](int item) {
+        pf_item = item;
+        if (item >= items) {   // past the workgroup's last item: nothing is fetched, the load counts stay the same
+            pf_a = pf_w = pf_z = pf_s = rsrc(x, 0);
+            pf_it = 0, pf_end = 0x7fffffff, pf_grp = 0, pf_cnt = 0;
+            return;
+        }
+        const Item d = decode(item);
+        const int wc0 = min((d.n0 + wn0) >> 3, words - 16);
+        pf_a = rsrc(x + (size_t)d.m0 * K, (size_t)(M - d.m0) * K * 2);
+        pf_w = rsrc(qweight + wc0, ((size_t)K * words - wc0) * 4);
+        pf_z = rsrc(qzeros + wc0, ((size_t)groups * words - wc0) * 4);
+        pf_s = rsrc(scales + (size_t)wc0 * 8, ((size_t)groups * words - wc0) * 16);
+        pf_it = d.it_begin, pf_end = d.it_end;
+        pf_grp = d.it_begin / steps_per_group, pf_cnt = d.it_begin % steps_per_group;
+    };
+    auto advance = [&]() {
+        ++pf_it;
+        if (++pf_cnt == steps_per_group) pf_cnt = 0, ++pf_grp;
+        if (pf_it == pf_end) open_cursor(pf_item + (int)gridDim.x);
+    };
 
-    // ---- A: load i of wave w fills slots (NDMA*w + i)*64 + lane, i.e. rows 8*(NDMA*w + i) + lane/8, whose chunk
-    //      at position lane%8 is kc = lane%8 ^ swz(row).  Rows past M read the last row; their results are never
-    //      stored.
+    // ---- A: load i of wave w fills slots (NDMA*w + i)*64 + lane, i.e. rows 8*(NDMA*w + i) + lane/8 of the tile, whose
+    //      chunk at position lane%8 is kc = lane%8 ^ swz(row).
     int a_off[NDMA];
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) {
         const int row = (wave * NDMA + i) * 8 + (lane >> 3);
         const int kc = (lane & 7) ^ rb_row_swz(row);
-        a_off[i] = (min(row, M - 1 - m0) * K + kc * 8) * 2;
+        a_off[i] = (row * K + kc * 8) * 2;
     }
-    auto dma_a_part = [&](int it, int buf, int i) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, AWQ_RB_LPTR(lds + buf * A_SLOTS + (wave * NDMA + i) * 64), 16,
-                                                 a_off[i], it * (kRBK * 2), 0, 0);
+    auto dma_a_part = [&](int step, int buf, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(pf_a, AWQ_RB_LPTR(lds + buf * A_SLOTS + (wave * NDMA + i) * 64), 16,
+                                                 a_off[i], step * (kRBK * 2), 0, 0);
     };
 
     // ---- B: word column j of the wave's 16, rows 8*kq + i of each 32-row half step ---------------------------
-    const int gwc = min(((n0 + wn0) >> 3) + j, words - 1);
     int w_off[8];   // byte offsets of the lane's 8 rows inside a half step
 #pragma unroll
-    for (int i = 0; i < 8; ++i) w_off[i] = ((kq * 8 + i) * words + gwc) * 4;
+    for (int i = 0; i < 8; ++i) w_off[i] = ((kq * 8 + i) * words + j) * 4;
     auto load_word = [&](int half_step, int i) {   // half step = 2 * step + half
-        return __builtin_amdgcn_raw_buffer_load_b32(rs_w, w_off[i], half_step * 32 * words * 4, 0);
+        return __builtin_amdgcn_raw_buffer_load_b32(pf_w, w_off[i], half_step * 32 * words * 4, 0);
     };
-    const int steps_per_group = g / kRBK;   // g % 64 == 0
     auto load_group = [&](int grp, uint32_t& z, u32x4& sv) {
-        z = __builtin_amdgcn_raw_buffer_load_b32(rs_z, gwc * 4, grp * words * 4, 0);
-        sv = __builtin_amdgcn_raw_buffer_load_b128(rs_s, gwc * 16, grp * words * 16, 0);
+        z = __builtin_amdgcn_raw_buffer_load_b32(pf_z, j * 4, grp * words * 4, 0);
+        sv = __builtin_amdgcn_raw_buffer_load_b128(pf_s, j * 16, grp * words * 16, 0);
     };
 
     // ---- A operand reads: fragment f = 8*ks + m of a step is row wm0 + 16*m + j, chunk 4*ks + kq ----------------
@@ -354,6 +389,82 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
     for (int m = 0; m < 8; ++m)
 #pragma unroll
         for (int t = 0; t < 8; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // The accumulators stay in the AGPR file until the store reads them, a row tile at a time (copied out all at once
+    // they would push the next item's operands, which are live across the store, into scratch).
+    auto pin_acc = [](f32x4 (&a)[8]) {
+        asm volatile("" : "+a"(a[0]), "+a"(a[1]), "+a"(a[2]), "+a"(a[3]), "+a"(a[4]), "+a"(a[5]), "+a"(a[6]), "+a"(a[7]));
+    };
+    // An item's result: acc[m][t][i] is row m0 + wm0 + 16*m + 4*kq + i, column n0 + wn0 + 8*j + column_of(t).
+    auto store_item = [&](const Item& d) {
+        const int n = d.n0 + wn0 + 8 * j;
+        if (d.whole) {
+            // one code path per epilogue (chosen once per item: merged, every value would pay for the bias rounding
+            // and the gate product whether it is wanted or not -- conversions run at a quarter of the ALU rate)
+            auto rows = [&](auto mode) {
+                constexpr int MODE = decltype(mode)::value;   // 0: plain, 1: + bias, 2: gated
+                float bv[8];
+                if constexpr (MODE == 1) {
+                    if (n < N) {
+                        const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + n);
+#pragma unroll
+                        for (int c = 0; c < 8; ++c)
+                            bv[c] = T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < 8; ++m) {
+                    pin_acc(acc[m]);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = d.m0 + wm0 + m * 16 + 4 * kq + i;
+                        u32x4 val;
+#pragma unroll
+                        for (int h = 0; h < 4; ++h) {
+                            float lo = acc[m][position_of(2 * h)][i], hi = acc[m][position_of(2 * h + 1)][i];
+                            if constexpr (MODE == 1) lo = add_bias<T>(lo, bv[2 * h]), hi = add_bias<T>(hi, bv[2 * h + 1]);
+                            val[h] = T::pack2(lo, hi);
+                        }
+                        if constexpr (MODE == 2) {
+                            // a lane holds one word of 8 columns; even words are gate columns, the next word the up
+                            // columns of the same outputs (N % 16 == 0, so a pair is in range or out of range together)
+                            u32x4 other;
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) other[q] = __shfl_xor(val[q], 1);
+                            if (row < M && n < N)
+                                swiglu_pair_store<T>(val, other, j & 1, y + (size_t)row * (N >> 1) + ((n & ~15) >> 1));
+                        } else if (row < M && n < N) {
+                            *reinterpret_cast<u32x4*>(y + (size_t)row * N + n) = val;
+                        }
+                        // one row at a time: the operands of the next item stay in their registers meanwhile
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            };
+            if (plan.act) rows(std::integral_constant<int, 2>{});
+            else if (bias) rows(std::integral_constant<int, 1>{});
+            else rows(std::integral_constant<int, 0>{});
+        } else {
+            // fp32 partial of this K slice, tile-compact: [slice][tail tile][256][256].  Rows and columns past
+            // M and N are stored too (they stay inside the tile's slot); the reduction pass masks them.
+            float* slot = partials + ((size_t)(d.split * plan.tail_tiles + (d.tile - plan.full_tiles)) << 16);
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                pin_acc(acc[m]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float* dst = slot + (wm0 + m * 16 + 4 * kq + i) * BN + wn0 + 8 * j;
+                    *reinterpret_cast<f32x4*>(dst) =
+                        f32x4{acc[m][position_of(0)][i], acc[m][position_of(1)][i], acc[m][position_of(2)][i],
+                              acc[m][position_of(3)][i]};
+                    *reinterpret_cast<f32x4*>(dst + 4) =
+                        f32x4{acc[m][position_of(4)][i], acc[m][position_of(5)][i], acc[m][position_of(6)][i],
+                              acc[m][position_of(7)][i]};
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    };
 
     // Half step h = 2 * step + half runs 8 row tiles of 8 MFMAs on the B operands bf[h % 2] (row-tile-major: an A
     // fragment serves 8 MFMAs in a row and is read from LDS two fragments ahead, into a ring of four).  Behind its
@@ -368,8 +479,7 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
     // of the second -- after the step's first barrier, which every wave reaches only when it is done with step - 1,
     // whose LDS buffer (three in rotation) this fills.  The A tile of step + 1 is complete at the second barrier of a
     // step: 23 loads have been issued since its last part (25 if the compiler puts that part in front of the two words
-    // that go out behind the same row tile).  Loads past the end of K are not guarded: the buffer
-    // descriptors return zero (or another row's x, in bounds) and nothing uses them.
+    // that go out behind the same row tile).  "Step + 2" is the cursor `pf`: it walks the workgroup's items end to end.
     auto main_loop = [&](auto role) {
         constexpr int ROLE = decltype(role)::value;
         FragUnpack<T, ROLE> up;
@@ -379,24 +489,28 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
         uint32_t ws[2][8], z_n;   // words of half steps h + 2 (parity h % 2), group of the next step
         u32x4 s_n;
         u32x4 bf[2][8], af[4], own[4];
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_a_part(it_begin, 0, i);
-#pragma unroll
-        for (int i = 0; i < NDMA; ++i) dma_a_part(it_begin + 1, 1, i);
+        int item = blockIdx.x;
+        Item cur = decode(item);
+        open_cursor(item);
+        // ---- the first two steps of the run, unaided (the second may already belong to the next item) ----
         {
             uint32_t w0[8], w1[8], z;
             u32x4 sv;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) w0[i] = load_word(2 * it_begin, i), w1[i] = load_word(2 * it_begin + 1, i);
-            load_group(it_begin / steps_per_group, z, sv);
+            for (int i = 0; i < NDMA; ++i) dma_a_part(pf_it, 0, i);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ws[0][i] = load_word(2 * it_begin + 2, i), ws[1][i] = load_word(2 * it_begin + 3, i);
-            load_group((it_begin + 1) / steps_per_group, z_n, s_n);
+            for (int i = 0; i < 8; ++i) w0[i] = load_word(2 * pf_it, i), w1[i] = load_word(2 * pf_it + 1, i);
+            load_group(pf_grp, z, sv);
+            advance();
+#pragma unroll
+            for (int i = 0; i < NDMA; ++i) dma_a_part(pf_it, 1, i);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ws[0][i] = load_word(2 * pf_it, i), ws[1][i] = load_word(2 * pf_it + 1, i);
+            load_group(pf_grp, z_n, s_n);
+            advance();
             unpack_all<T>(w0, z, sv, bf[0]);
             unpack_all<T>(w1, z, sv, bf[1]);
         }
-        // group of step + 2 (loaded at the start of a step), without a division per step
-        int grp_nn = (it_begin + 2) / steps_per_group, cnt_nn = (it_begin + 2) % steps_per_group;
         const int x_own = wave * 256 + lane, x_partner = (wave ^ 2) * 256 + lane;
         // the first half step reads the operands of the second back like any other: leave this wave's four there
 #pragma unroll
@@ -408,114 +522,71 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
         int buf = 0;
         af[0] = lds[a_rd[0]];
         af[1] = lds[a_rd[0] + 128];
-        for (int it = it_begin; it < it_end; ++it) {
-            const int nb = buf == NBUF - 1 ? 0 : buf + 1, nnb = nb == NBUF - 1 ? 0 : nb + 1;
-            const u32x4* abase = lds + buf * A_SLOTS;
-            const u32x4* anext = lds + nb * A_SLOTS;
-            // the operands built during this step belong to step + 1
-            up.set_group(z_n, s_n);
-            load_group(grp_nn, z_n, s_n);
-            if (++cnt_nn == steps_per_group) cnt_nn = 0, ++grp_nn;
+        for (;;) {
+            for (int it = cur.it_begin; it < cur.it_end; ++it) {
+                const int nb = buf == NBUF - 1 ? 0 : buf + 1, nnb = nb == NBUF - 1 ? 0 : nb + 1;
+                const u32x4* abase = lds + buf * A_SLOTS;
+                const u32x4* anext = lds + nb * A_SLOTS;
+                // the operands built during this step belong to step + 1
+                up.set_group(z_n, s_n);
+                load_group(pf_grp, z_n, s_n);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    u32x4* xbuf = xlds + ks * X_SLOTS;
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) {
+                        const int f = ks * 8 + m;
+                        // fragment f + 2, of the next step's buffer from f = 14 on
+                        if (f + 2 < 16)
+                            af[(f + 2) & 3] = abase[a_rd[(f + 2) >> 3] + ((f + 2) & 7) * 128];
+                        else
+                            af[(f + 2) & 3] = anext[a_rd[0] + (f + 2 - 16) * 128];
+                        up.row_tile(m, acc[m], af[f & 3], bf[ks], ws[ks], own);
+                        if (m == 0) {
+                            // Every wave has stored its operands of half step h + 1 (at the end of half step h - 1; the
+                            // stores completed behind row tile 0) -- and, in the second half, its part of the A tile of
+                            // step + 1.  A bare barrier: __syncthreads() would also wait for this step's own loads.
+                            if (ks == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                            else asm volatile("s_waitcnt vmcnt(23) lgkmcnt(0)" ::: "memory");
+                            __builtin_amdgcn_s_barrier();
+                            asm volatile("" ::: "memory");
+                        } else if (m <= 4) {
+                            // operands of half step h + 1, written at the end of half step h - 1 into the other buffer
+                            const u32x4* xprev = xlds + (1 - ks) * X_SLOTS;
+                            const int i = m - 1;
+                            bf[1 - ks][FragUnpack<T, ROLE>::own(i)] = xprev[x_own + i * 64];
+                            bf[1 - ks][FragUnpack<T, 1 - ROLE>::own(i)] = xprev[x_partner + i * 64];
+                        }
+                        if (m & 1) {
+                            ws[ks][m - 1] = load_word(2 * pf_it + ks, m - 1);
+                            ws[ks][m] = load_word(2 * pf_it + ks, m);
+                        }
+                        if (m >= 1 && (ks == 0 || m == 1)) dma_a_part(pf_it, nnb, ks == 0 ? m - 1 : 7);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) xbuf[x_own + i * 64] = own[i];
+                }
+                buf = nb;
+                advance();
+            }
+            // the last MFMAs' results: 4 passes to write
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
+            store_item(cur);
+            item += gridDim.x;
+            if (item >= items) break;
+            cur = decode(item);
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                u32x4* xbuf = xlds + ks * X_SLOTS;
+            for (int m = 0; m < 8; ++m)
 #pragma unroll
-                for (int m = 0; m < 8; ++m) {
-                    const int f = ks * 8 + m;
-                    // fragment f + 2, of the next step's buffer from f = 14 on
-                    if (f + 2 < 16)
-                        af[(f + 2) & 3] = abase[a_rd[(f + 2) >> 3] + ((f + 2) & 7) * 128];
-                    else
-                        af[(f + 2) & 3] = anext[a_rd[0] + (f + 2 - 16) * 128];
-                    up.row_tile(m, acc[m], af[f & 3], bf[ks], ws[ks], own);
-                    if (m == 0) {
-                        // Every wave has stored its operands of half step h + 1 (at the end of half step h - 1; the
-                        // stores completed behind row tile 0) -- and, in the second half, its part of the A tile of
-                        // step + 1.  A bare barrier: __syncthreads() would also wait for this step's own loads.
-                        if (ks == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                        else asm volatile("s_waitcnt vmcnt(23) lgkmcnt(0)" ::: "memory");
-                        __builtin_amdgcn_s_barrier();
-                        asm volatile("" ::: "memory");
-                    } else if (m <= 4) {
-                        // operands of half step h + 1, written at the end of half step h - 1 into the other buffer
-                        const u32x4* xprev = xlds + (1 - ks) * X_SLOTS;
-                        const int i = m - 1;
-                        bf[1 - ks][FragUnpack<T, ROLE>::own(i)] = xprev[x_own + i * 64];
-                        bf[1 - ks][FragUnpack<T, 1 - ROLE>::own(i)] = xprev[x_partner + i * 64];
-                    }
-                    if (m & 1) {
-                        ws[ks][m - 1] = load_word(2 * it + ks + 4, m - 1);
-                        ws[ks][m] = load_word(2 * it + ks + 4, m);
-                    }
-                    if (m >= 1 && (ks == 0 || m == 1)) dma_a_part(it + 2, nnb, ks == 0 ? m - 1 : 7);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) xbuf[x_own + i * 64] = own[i];
-            }
-            buf = nb;
+                for (int t = 0; t < 8; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            __builtin_amdgcn_sched_barrier(0);
         }
-        // the last MFMAs' results: 4 passes to write, read by the epilogue below
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
     };
-    if (it_begin < it_end) {
-        if ((wave >> 1) == 0) main_loop(std::integral_constant<int, 0>{});
-        else main_loop(std::integral_constant<int, 1>{});
-    }
-
-    // acc[m][t][i]: row wm0 + 16*m + 4*kq + i, column wn0 + 8*j + column_of(t)
-    const int n = n0 + wn0 + 8 * j;
-    if (whole) {
-        float bv[8];
-        if (bias && n < N) {
-            const u32x4 bvv = *reinterpret_cast<const u32x4*>(bias + n);
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-                bv[c] = T::to_f32((uint16_t)((c & 1) ? (bvv[c >> 1] >> 16) : (bvv[c >> 1] & 0xFFFFu)));
-        }
-#pragma unroll
-        for (int m = 0; m < 8; ++m)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = m0 + wm0 + m * 16 + 4 * kq + i;
-                u32x4 val;
-#pragma unroll
-                for (int h = 0; h < 4; ++h) {
-                    float lo = acc[m][position_of(2 * h)][i], hi = acc[m][position_of(2 * h + 1)][i];
-                    if (bias) lo = add_bias<T>(lo, bv[2 * h]), hi = add_bias<T>(hi, bv[2 * h + 1]);
-                    val[h] = T::pack2(lo, hi);
-                }
-                if (plan.act) {
-                    // a lane holds one word of 8 columns; even words are gate columns, the next word the up
-                    // columns of the same outputs (N % 16 == 0, so a pair is in range or out of range together)
-                    u32x4 other;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) other[q] = __shfl_xor(val[q], 1);
-                    if (row < M && n < N)
-                        swiglu_pair_store<T>(val, other, j & 1, y + (size_t)row * (N >> 1) + ((n & ~15) >> 1));
-                } else if (row < M && n < N) {
-                    *reinterpret_cast<u32x4*>(y + (size_t)row * N + n) = val;
-                }
-            }
-    } else {
-        // fp32 partial of this K slice, tile-compact: [slice][tail tile][256][256].  Rows and columns past
-        // M and N are stored too (they stay inside the tile's slot); the reduction pass masks them.
-        float* slot = partials + ((size_t)(split * plan.tail_tiles + (tile - plan.full_tiles)) << 16);
-#pragma unroll
-        for (int m = 0; m < 8; ++m)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float* dst = slot + (wm0 + m * 16 + 4 * kq + i) * BN + wn0 + 8 * j;
-                *reinterpret_cast<f32x4*>(dst) =
-                    f32x4{acc[m][position_of(0)][i], acc[m][position_of(1)][i], acc[m][position_of(2)][i],
-                          acc[m][position_of(3)][i]};
-                *reinterpret_cast<f32x4*>(dst + 4) =
-                    f32x4{acc[m][position_of(4)][i], acc[m][position_of(5)][i], acc[m][position_of(6)][i],
-                          acc[m][position_of(7)][i]};
-            }
-    }
+    if ((wave >> 1) == 0) main_loop(std::integral_constant<int, 0>{});
+    else main_loop(std::integral_constant<int, 1>{});
 }
 
 template <typename T>
@@ -536,7 +607,8 @@ hipError_t launch_regb(const void* x, const int32_t* qweight, const void* qscale
         raised = true;
     }
     (void)hipGetLastError();
-    hipLaunchKernelGGL(kern, dim3(plan.full_tiles + plan.tail_tiles * plan.splits), dim3(256), lds, stream,
+    const int items = plan.full_tiles + plan.tail_tiles * plan.splits;
+    hipLaunchKernelGGL(kern, dim3(items < kResidentWgs ? items : kResidentWgs), dim3(256), lds, stream,
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, M, N, K, g, plan);

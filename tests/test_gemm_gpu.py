@@ -100,7 +100,9 @@ def test_gemm_tail_tiles_split(dtype, form):
     L = _lib.lib()
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
     tail, whole = names.index(f"256x256{form}t"), names.index(f"256x256{form}")
-    M, K, N = 2300, 256, 7672
+    # (the register-operand kernel takes widths that are multiples of 128; other widths run the pipelined one under
+    # its name: its case has the last tile half empty instead of ragged)
+    M, K, N = 2300, 256, (7672 if form == "p" else 7552)
     p = random_packed(K, N, 128, dtype, seed=95)
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
     xb = make_x(M, K, dtype, seed=96)
@@ -189,22 +191,27 @@ def test_gemm_register_b_kernel_equals_pipelined(dtype, M, K, N, g, split):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_gemm_default_kernel_on_full_rounds(dtype):
-    # 16 x 17 = 272 tiles: the default entry point runs the register-operand kernel in fp16 and the pipelined one in
-    # bf16, both with the planned tail split -- bit for bit what the forced variants give
+@pytest.mark.parametrize("M,K,N", [(4096, 512, 4352), (4096, 1024, 4096), (2048, 1024, 4096)])
+def test_gemm_default_kernel_by_work_items(dtype, M, K, N):
+    # The default entry point runs the register-operand kernel (r) where the plan's work items -- whole tiles plus the
+    # K slices of the tail tiles -- outnumber the 256 CUs (16 x 17 = 272 tiles), in fp16 also at exactly 256 (16 x 16),
+    # and the pipelined kernel (p) below that (8 x 16 tiles cut in two): bit for bit what the forced variants give.
     import ctypes
     L = _lib.lib()
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
-    M, K, N = 4096, 512, 4352
     v, sp = ctypes.c_int(), ctypes.c_int()
     assert L.awq_gemm_plan(M, N, K, ctypes.byref(v), ctypes.byref(sp)) == 0
     assert names[v.value] in ("256x256p", "256x256pt")
-    print(f"gemm default on full rounds {dtype}: plan {names[v.value]} split {sp.value}", flush=True)
+    tiles = (M // 256) * (N // 256)
+    tail = tiles % 256 if names[v.value] == "256x256pt" else (tiles if sp.value > 1 else 0)
+    items = tiles - tail + tail * sp.value
+    print(f"gemm default {dtype} M={M} K={K} N={N}: plan {names[v.value]} split {sp.value}, {items} items", flush=True)
     p = random_packed(K, N, 128, dtype, seed=123)
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
     xd = to_dev(make_x(M, K, dtype, seed=124), dtype)
     y = nq.awq_gemm(xd, *dev, 8)
-    forced = names[v.value].replace("p", "r") if dtype == "f16" else names[v.value]
+    use_r = items > 256 or (dtype == "f16" and items == 256)
+    forced = names[v.value].replace("p", "r") if use_r else names[v.value]
     assert torch.equal(y, awq_gemm_variant(xd, *dev, names.index(forced), sp.value)), forced
     rows = torch.arange(0, M, 97, device="cuda")
     ref = xd[rows].float() @ nq.awq_dequantize(*dev).float()
