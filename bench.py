@@ -254,13 +254,14 @@ def main():
             del w
         bestf = max(v["TFLOPs"] for v in fused.values())
         out["roofline_prefill"] = {
-            "kernel": "awq::gemm_pipe_kernel<BF16,2,4>", "bound": "mfma", "achieved": bestf,
+            "kernel": "awq::gemm_regb_kernel<BF16> (M = 2048 on 4096x12288 and M = 8192: more work items than CUs) / "
+                      "awq::gemm_pipe_kernel<BF16,2,4> (the others)", "bound": "mfma", "achieved": bestf,
             "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": bestf / MFMA_PEAK_TFLOPS,
             "workload": "cfg3: Qwen3-8B MLP shapes, bf16, M in {512,2048,8192}; the fused dequant + MFMA kernel "
                         "(default dispatch at every M)",
             "cases": fused}
-        # the same shapes in fp16 at the row counts that fill whole rounds of tiles: the default dispatch runs the
-        # kernel that builds its B operands in registers there (awq::gemm_regb_kernel)
+        # the same shapes in fp16 at the row counts whose work items fill the CUs: the default dispatch runs the
+        # kernel with resident workgroups that builds its B operands in registers there (awq::gemm_regb_kernel)
         hdt = torch.float16
         fused16 = {}
         for (K, N) in ((4096, 12288), (12288, 4096)):
@@ -275,8 +276,7 @@ def main():
             del w
         best16 = max(v["TFLOPs"] for v in fused16.values())
         out["roofline_prefill_f16"] = {
-            "kernel": "awq::gemm_regb_kernel<F16> (launches of 256 output tiles or more: all but M = 2048 on 12288x4096, which "
-                      "runs awq::gemm_pipe_kernel<F16,2,4>)",
+            "kernel": "awq::gemm_regb_kernel<F16> (256 work items or more: all four cases)",
             "bound": "mfma", "achieved": best16, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": best16 / MFMA_PEAK_TFLOPS,
             "workload": "cfg3's shapes with fp16 activations and scales, M in {2048, 8192}, default dispatch",
