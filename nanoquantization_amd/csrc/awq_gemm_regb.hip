@@ -22,6 +22,11 @@
 // Epilogue: a lane's eight tiles are the eight columns of its word, so a row of its accumulators
 // leaves as one 16-byte store (fp32 partials of a K slice: two), without staging.
 //
+// The workgroups are resident: the grid is at most one workgroup per CU, and a workgroup walks its
+// work items (whole tiles, K slices of tail tiles) as one run of K steps -- the loads of a step are
+// those of the step two ahead, across item boundaries, so only the first item of a workgroup pays
+// for an unaided start, and between two items only the accumulators are stored and cleared.
+//
 // What the instructions cost (measured on one wave per SIMD, MFMAs back to back with one other
 // instruction mixed in per 8): a 16x16x32 MFMA occupies the matrix core for 18.5 cycles and the
 // SIMD's issue port for 12 of them, any other instruction for 4; LDS reads and global loads to
