@@ -296,8 +296,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_pipe_kernel(
             const int n = n0 + wn0 + b * 32 + li;
             bv[b] = (bias && n < N) ? T::to_f32(bias[n]) : 0.f;
         }
-        // one code path per epilogue, chosen once (merged, every value would pay for the bias rounding and the gate
-        // product whether wanted or not; conversions run at a quarter of the ALU rate)
+        // one code path per epilogue, chosen once (merged by selects, every value pays for the bias rounding and the
+        // gate product whether wanted or not: three times the instructions)
         auto rows = [&](auto mode) {
             constexpr int MODE = decltype(mode)::value;   // 0: plain, 1: + bias, 2: gated
 #pragma unroll
