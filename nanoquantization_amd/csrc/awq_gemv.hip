@@ -798,14 +798,18 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
         uint32_t sink = 0;
         for (int r = 0; r < pf.count; ++r) {
             const long long lines = pf.bytes[r] >> 7;
-            // four independent loads in flight per thread and round
+            // four independent loads in flight per thread and round: issued as assembly and waited for once (as
+            // volatile accesses the compiler waits after each of them: four memory round trips in a row, which made
+            // the prefetch workgroups the last to finish)
             for (long long l = tid; l < lines; l += 4 * nthreads) {
                 uint32_t v[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const long long lu = l + u * nthreads;
-                    v[u] = *reinterpret_cast<const volatile uint32_t*>(pf.ptr[r] + ((lu < lines ? lu : l) << 7));
+                    const char* addr = pf.ptr[r] + ((lu < lines ? lu : l) << 7);
+                    asm volatile("global_load_dword %0, %1, off" : "=v"(v[u]) : "v"(addr) : "memory");
                 }
+                asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
                 sink ^= v[0] ^ v[1] ^ v[2] ^ v[3];
             }
         }
