@@ -48,7 +48,6 @@ namespace awq {
 namespace {
 
 constexpr int kRBK = 64;
-constexpr int kResidentWgs = 256;   // one workgroup per CU (128 KiB of LDS each)
 
 #define AWQ_RB_GPTR(p) ((__attribute__((address_space(1))) const void*)(p))
 #define AWQ_RB_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -612,8 +611,17 @@ hipError_t launch_regb(const void* x, const int32_t* qweight, const void* qscale
         raised = true;
     }
     (void)hipGetLastError();
+    // one resident workgroup per CU (128 KiB of LDS each); the CU count is asked for once
+    static int resident = 0;
+    if (resident <= 0) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        resident = cus;
+    }
     const int items = plan.full_tiles + plan.tail_tiles * plan.splits;
-    hipLaunchKernelGGL(kern, dim3(items < kResidentWgs ? items : kResidentWgs), dim3(256), lds, stream,
+    hipLaunchKernelGGL(kern, dim3(items < resident ? items : resident), dim3(256), lds, stream,
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, M, N, K, g, plan);
