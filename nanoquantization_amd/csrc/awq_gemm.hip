@@ -353,11 +353,14 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     // tiles -- outnumber the CUs runs the register-operand kernel instead: it walks a workgroup's items as one run of
     // K steps (no prologue, no dispatch between tiles).  M = 8192 x 4096 x 12288: 729 against 822 us in fp16, 774
     // against 800 in bf16; 16384 x 1024 x 6144: 227 / 234 against 256 / 261.  With one item per workgroup its heavier
-    // start costs 3-11 % in bf16 (fp16: level from 256 items on, its unpack being the cheaper one).
+    // start costs 3-11 % in bf16 on short items (fp16: level from 256 items on, its unpack being the cheaper one).
     if (planned && g % 64 == 0 && N % 128 == 0 && (variant == kPipeVariant || variant == kPipeTailVariant)) {
         const PipePlan pp = make_pipe_plan(M, N, K, split_k, variant == kPipeTailVariant);
         const int64_t items = (int64_t)pp.full_tiles + (int64_t)pp.tail_tiles * pp.splits;
-        if (items > 256 || (dtype == AWQ_F16 && items == 256))
+        // exactly one item per CU: fp16 always; bf16 from 64 K steps per item on (2048 x 12288 x 4096 cut in two,
+        // 96 steps: 216 against 220 us; 16384 x 2048 x 1024, 32 steps: 79 against 74)
+        const int64_t steps = pp.tail_tiles > 0 && pp.full_tiles == 0 ? pp.iters_per_split : K / 64;
+        if (items > 256 || (items == 256 && (dtype == AWQ_F16 || steps >= 64)))
             variant = variant == kPipeVariant ? kRegbVariant : kRegbTailVariant;
     }
     const GemmVariant& gv = kGemmVariants[variant];

@@ -191,11 +191,13 @@ def test_gemm_register_b_kernel_equals_pipelined(dtype, M, K, N, g, split):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("M,K,N", [(4096, 512, 4352), (4096, 1024, 4096), (2048, 1024, 4096)])
+@pytest.mark.parametrize("M,K,N", [(4096, 512, 4352), (4096, 1024, 4096), (2048, 1024, 4096), (4096, 4096, 4096),
+                                   (1024, 1024, 4096)])
 def test_gemm_default_kernel_by_work_items(dtype, M, K, N):
     # The default entry point runs the register-operand kernel (r) where the plan's work items -- whole tiles plus the
-    # K slices of the tail tiles -- outnumber the 256 CUs (16 x 17 = 272 tiles), in fp16 also at exactly 256 (16 x 16),
-    # and the pipelined kernel (p) below that (8 x 16 tiles cut in two): bit for bit what the forced variants give.
+    # K slices of the tail tiles -- outnumber the 256 CUs (16 x 17 = 272 tiles); at exactly 256 items (16 x 16 tiles, or
+    # 8 x 16 cut in two) in fp16, and in bf16 if an item has 64 K steps at least; the pipelined kernel (p) otherwise
+    # (4 x 16 tiles cut in two): bit for bit what the forced variants give.
     import ctypes
     L = _lib.lib()
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
@@ -210,7 +212,8 @@ def test_gemm_default_kernel_by_work_items(dtype, M, K, N):
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
     xd = to_dev(make_x(M, K, dtype, seed=124), dtype)
     y = nq.awq_gemm(xd, *dev, 8)
-    use_r = items > 256 or (dtype == "f16" and items == 256)
+    steps = K // 64 // (sp.value if tail == tiles else 1)
+    use_r = items > 256 or (items == 256 and (dtype == "f16" or steps >= 64))
     forced = names[v.value].replace("p", "r") if use_r else names[v.value]
     assert torch.equal(y, awq_gemm_variant(xd, *dev, names.index(forced), sp.value)), forced
     rows = torch.arange(0, M, 97, device="cuda")
