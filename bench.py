@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 # (FETCH_SIZE, then WRITE_SIZE; profiles/gemv_cfg2_sweep_hbm_traffic.txt).  Each counter is scaled by
 # what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,011.5 -> 2047.3 B per count,
 # WRITE_SIZE 64,000 -> 1024 B per count.
-MEASURED_FETCH_BYTES_PER_LAUNCH = 1130.85 * 2047.3
+MEASURED_FETCH_BYTES_PER_LAUNCH = 1123.98 * 2047.3
 MEASURED_WRITE_BYTES_PER_LAUNCH = 100.68 * 1024.0
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
@@ -172,7 +172,7 @@ def main():
         "achieved": avg_bytes / (avg_launch_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "traffic": MEASURED_FETCH_BYTES_PER_LAUNCH + MEASURED_WRITE_BYTES_PER_LAUNCH,
-        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 2.32 MB + write 0.10 MB) from rocprofv3 "
+        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 2.30 MB + write 0.10 MB) from rocprofv3 "
                         "FETCH_SIZE / WRITE_SIZE, copy-calibrated.  The counters sit between the L2s and the fabric "
                         "and cannot tell Infinity Cache hits from HBM reads: about 0.87 MB of the fetch is the prefetch "
                         "(spare workgroups read the next launch's weights once to park them in the Infinity Cache, "
