@@ -13,6 +13,11 @@ headline -- the same GEMV on the Qwen3-32B MLP shapes where a launch is long eno
 the prefill GEMM TFLOP/s at the Qwen3-8B MLP shapes, the dequantise kernel, and config 1's latency.
 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cfg5] [--only-cfg5] [--no-cpu]
+
+For a profiler or a counter collection to look at one kernel (no timing, no JSON line):
+python bench.py --one linear|dequant|copy K N M [--one-dtype bf16|f16] [--one-iters 6]
+launches that one problem a few times on the same seeded buffers (`copy`: a device copy of the packed weight,
+the known-size kernel the traffic counters are calibrated with).
 """
 from __future__ import annotations
 
@@ -112,8 +117,47 @@ def time_eager(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
+def run_one(kind, K, N, M, dtype, iters, g=G):
+    """One problem, `iters` launches, nothing timed: the subject of a rocprofv3 run."""
+    import nanoquantization_amd as nq
+    dev = torch.device("cuda:0")
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float16
+    gen = torch.Generator(device=dev).manual_seed(K + N)
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device=dev, generator=gen)
+    qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, device=dev, generator=gen)
+    qs = (torch.rand(K // g, N, device=dev, generator=gen) * 0.02 + 0.001).to(tdt)
+    x = torch.randn(max(M, 1), K, device=dev, generator=gen).to(tdt)
+    fn = {"linear": lambda: nq.awq_gemm(x, qw, qs, qz, 8),
+          "dequant": lambda: nq.awq_dequantize(qw, qs, qz), "copy": lambda: qw.clone()}[kind]
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    print(f"{kind} K={K} N={N} M={M} {dtype}: {iters} launches")
+
+
+def gemm_kernel_name(M, N, K, dtype_name, g=G):
+    """The kernel awq_gemm runs for a prefill problem, from the library's own plan."""
+    import ctypes
+    from nanoquantization_amd import _lib
+    L = _lib.lib()
+    v, sp = ctypes.c_int(), ctypes.c_int()
+    did = _lib.AWQ_F16 if dtype_name == "f16" else _lib.AWQ_BF16
+    if L.awq_gemm_plan(M, N, K, g, did, ctypes.byref(v), ctypes.byref(sp)) != 0:
+        return "?"
+    name = L.awq_gemm_variant_name(v.value).decode()
+    T = "F16" if dtype_name == "f16" else "BF16"
+    kern = {"256x256p": f"awq::gemm_pipe_kernel<{T},2,4>", "256x256pt": f"awq::gemm_pipe_kernel<{T},2,4>",
+            "256x256r": f"awq::gemm_regb_kernel<{T}>", "256x256rt": f"awq::gemm_regb_kernel<{T}>"}.get(
+                name, f"awq::gemm_kernel<{T},{name}>")
+    return f"{kern} (plan {name}, split {sp.value})"
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--one", nargs=4, metavar=("KIND", "K", "N", "M"),
+                    help="launch one problem a few times for a profiler: linear|dequant|copy K N M")
+    ap.add_argument("--one-dtype", choices=["bf16", "f16"], default="bf16")
+    ap.add_argument("--one-iters", type=int, default=6)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -142,6 +186,12 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.one:
+        kind, K1, N1, M1 = args.one[0], int(args.one[1]), int(args.one[2]), int(args.one[3])
+        if kind not in ("linear", "dequant", "copy"):
+            ap.error("--one KIND must be linear, dequant or copy")
+        run_one(kind, K1, N1, M1, args.one_dtype, args.one_iters)
+        return
     tdt = torch.float16
     torch.manual_seed(0)
 
@@ -250,12 +300,14 @@ def main():
                 us = time_graph(fn, 5, 1) * 1e3 / 4
                 tf = 2.0 * M * N * K / us / 1e6
                 fused[f"M{M}_{K}x{N}"] = {"us": round(us, 1), "TFLOPs": round(tf, 1),
-                                          "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4)}
+                                          "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4),
+                                          "kernel": gemm_kernel_name(M, N, K, "bf16")}
             del w
         bestf = max(v["TFLOPs"] for v in fused.values())
+        best_case = max(fused, key=lambda k: fused[k]["TFLOPs"])
         out["roofline_prefill"] = {
-            "kernel": "awq::gemm_regb_kernel<BF16> (M = 2048 on 4096x12288 and M = 8192: more work items than CUs) / "
-                      "awq::gemm_pipe_kernel<BF16,2,4> (the others)", "bound": "mfma", "achieved": bestf,
+            "kernel": fused[best_case]["kernel"] + f" at {best_case} (each case names its own)", "bound": "mfma",
+            "achieved": bestf,
             "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": bestf / MFMA_PEAK_TFLOPS,
             "workload": "cfg3: Qwen3-8B MLP shapes, bf16, M in {512,2048,8192}; the fused dequant + MFMA kernel "
                         "(default dispatch at every M)",
@@ -272,11 +324,13 @@ def main():
                 us = time_graph(fn, 5, 1) * 1e3 / 4
                 tf = 2.0 * M * N * K / us / 1e6
                 fused16[f"M{M}_{K}x{N}"] = {"us": round(us, 1), "TFLOPs": round(tf, 1),
-                                            "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4)}
+                                            "frac_of_2.5PF": round(tf / MFMA_PEAK_TFLOPS, 4),
+                                            "kernel": gemm_kernel_name(M, N, K, "f16")}
             del w
         best16 = max(v["TFLOPs"] for v in fused16.values())
+        best_case16 = max(fused16, key=lambda k: fused16[k]["TFLOPs"])
         out["roofline_prefill_f16"] = {
-            "kernel": "awq::gemm_regb_kernel<F16> (256 work items or more: all four cases)",
+            "kernel": fused16[best_case16]["kernel"] + f" at {best_case16} (each case names its own)",
             "bound": "mfma", "achieved": best16, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": best16 / MFMA_PEAK_TFLOPS,
             "workload": "cfg3's shapes with fp16 activations and scales, M in {2048, 8192}, default dispatch",

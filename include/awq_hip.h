@@ -211,10 +211,14 @@ int awq_gemv_variant_count(void);
 int awq_gemm_variant_count(void);
 const char* awq_gemv_variant_name(int variant);
 const char* awq_gemm_variant_name(int variant);
-/* The variant and K-split that awq_gemv / awq_gemm pick by themselves for a shape (host-only: no device call), so
- * that a caller can see, log or pin what will run. */
+/* The variant and K-split that awq_gemv / awq_gemm pick by themselves for a problem (host-only: no device call), so
+ * that a caller can see, log or pin what will run: awq_gemv_ex / awq_gemm_ex with the returned pair launch exactly
+ * what awq_gemv / awq_gemm launch for the same arguments.  The GEMM's choice depends on the tensor type and the
+ * group size as well as on the shape (which of the two 256 x 256 kernels runs), the workspace size does not.  The
+ * rules are tuned for the 256 compute units of a whole MI355X; on a partition with fewer the results are the same
+ * and only the balance of the launch is not the best one. */
 int awq_gemv_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, int* variant, int* split_k);
-int awq_gemm_plan(int64_t M, int64_t N, int64_t K, int* variant, int* split_k);
+int awq_gemm_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, int dtype, int* variant, int* split_k);
 size_t awq_gemv_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k);
 size_t awq_gemm_ex_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant, int split_k);
 int awq_gemv_ex(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,

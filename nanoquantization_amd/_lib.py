@@ -51,7 +51,7 @@ SYMBOLS = {
     "awq_gemm": (_int, _LINEAR_ARGS),
     "awq_linear": (_int, _LINEAR_ARGS),
     "awq_gemv_plan": (_int, [_i64, _i64, _i64, _i64, ctypes.POINTER(_int), ctypes.POINTER(_int)]),
-    "awq_gemm_plan": (_int, [_i64, _i64, _i64, ctypes.POINTER(_int), ctypes.POINTER(_int)]),
+    "awq_gemm_plan": (_int, [_i64, _i64, _i64, _i64, _int, ctypes.POINTER(_int), ctypes.POINTER(_int)]),
     "awq_gemv_variant_count": (_int, []),
     "awq_gemm_variant_count": (_int, []),
     "awq_gemv_variant_name": (ctypes.c_char_p, [_int]),

@@ -209,7 +209,7 @@ static const GemmVariant kGemmVariants[] = {
     {"256x256p", 256, 256, 8},   // the software-pipelined kernel of awq_gemm_pipe.hip, every tile cut split_k ways
     {"256x256pt", 256, 256, 8},  // the same kernel; split_k cuts only the tiles beyond the last full round of CUs
     // awq_gemm_regb.hip: B operands built in registers; the default entry points take it in place of the pipelined
-    // kernel for fp16 on 256 tiles or more (see gemm_dispatch); group sizes that are not multiples of 64 run the
+    // kernel where the work items outnumber the CUs (see substitute_regb); group sizes that are not multiples of 64 run the
     // pipelined kernel under these names too
     {"256x256r", 256, 256, 4},   // every tile cut split_k ways
     {"256x256rt", 256, 256, 4},  // split_k cuts only the tiles beyond the last full round of CUs
@@ -317,15 +317,43 @@ static void pick_gemm(int64_t M, int64_t N, int64_t K, int* variant, int* split_
     *split_k = (int)s;
 }
 
-// The same for the pipelined kernel at any M (the gated epilogue exists there only).
-static void pick_gemm_pipe(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
+// The register-operand kernel addresses a launch through 32-bit buffer offsets: the packed weight and the 256 rows of
+// x a tile reads must each stay below 2 GiB.
+static bool regb_takes(int64_t N, int64_t K, int64_t g) {
+    return g % 64 == 0 && N % 128 == 0 && K * (N / 8) * 4 < (1ll << 31) && 256 * K * 2 < (1ll << 31);
+}
+
+// What the default entry points run: pick_gemm's choice, with the pipelined 256 x 256 kernel replaced by the
+// register-operand one where the work items -- whole tiles plus K slices of the tail tiles -- outnumber the CUs (that
+// kernel walks a workgroup's items as one run of K steps: no prologue, no dispatch between tiles).  M = 8192 x 4096 x
+// 12288: 729 against 822 us in fp16, 774 against 800 in bf16; 16384 x 1024 x 6144: 227 / 234 against 256 / 261.  With
+// one item per workgroup its heavier start costs 3-11 % in bf16 on short items (fp16: level from 256 items on, its
+// unpack being the cheaper one), so at exactly one item per CU: fp16 always; bf16 from 64 K steps per item on
+// (2048 x 12288 x 4096 cut in two, 96 steps: 216 against 220 us; 16384 x 2048 x 1024, 32 steps: 79 against 74).
+static void substitute_regb(int64_t M, int64_t N, int64_t K, int64_t g, int dtype, int* variant, int split_k) {
+    if ((*variant != kPipeVariant && *variant != kPipeTailVariant) || !regb_takes(N, K, g)) return;
+    const PipePlan pp = make_pipe_plan(M, N, K, split_k, *variant == kPipeTailVariant);
+    const int64_t items = (int64_t)pp.full_tiles + (int64_t)pp.tail_tiles * pp.splits;
+    const int64_t steps = pp.tail_tiles > 0 && pp.full_tiles == 0 ? pp.iters_per_split : K / 64;
+    if (items > 256 || (items == 256 && (dtype == AWQ_F16 || steps >= 64)))
+        *variant = *variant == kPipeVariant ? kRegbVariant : kRegbTailVariant;
+}
+
+static void plan_gemm(int64_t M, int64_t N, int64_t K, int64_t g, int dtype, int* variant, int* split_k) {
+    pick_gemm(M, N, K, variant, split_k);
+    substitute_regb(M, N, K, g, dtype, variant, *split_k);
+}
+
+// The same on the 256 x 256 kernels at any M (the gated epilogue exists there only).
+static void plan_gemm_tile256(int64_t M, int64_t N, int64_t K, int64_t g, int dtype, int* variant, int* split_k) {
     pick_gemm(M > 128 ? M : 129, N, K, variant, split_k);   // tile counts depend on ceil(M / 256) only
+    substitute_regb(M, N, K, g, dtype, variant, *split_k);
 }
 
 static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, const void* qscales,
                          const int32_t* qzeros, const void* bias, void* y, int64_t M, int64_t N,
                          int64_t K, int64_t g, int dtype, void* workspace, size_t workspace_bytes,
-                         void* stream, int variant, int split_k, int act = 0, bool planned = false) {
+                         void* stream, int variant, int split_k, int act = 0) {
     // prefetch hints pending on this thread were meant for this call; the GEMM fills the chip, so they are dropped
     // (before any check: an error return must not leave them for an unrelated later launch)
     PrefetchRegions dropped;
@@ -348,20 +376,6 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     if (act && (bias || N % 16 != 0 || !is_tile256(variant))) {
         set_error("%s: the gated epilogue takes no bias, needs N %% 16 == 0 and runs on the pipelined kernel", fn);
         return AWQ_ERR_UNSUPPORTED;
-    }
-    // A planned (not forced) launch of the pipelined kernel whose work items -- whole tiles plus K slices of the tail
-    // tiles -- outnumber the CUs runs the register-operand kernel instead: it walks a workgroup's items as one run of
-    // K steps (no prologue, no dispatch between tiles).  M = 8192 x 4096 x 12288: 729 against 822 us in fp16, 774
-    // against 800 in bf16; 16384 x 1024 x 6144: 227 / 234 against 256 / 261.  With one item per workgroup its heavier
-    // start costs 3-11 % in bf16 on short items (fp16: level from 256 items on, its unpack being the cheaper one).
-    if (planned && g % 64 == 0 && N % 128 == 0 && (variant == kPipeVariant || variant == kPipeTailVariant)) {
-        const PipePlan pp = make_pipe_plan(M, N, K, split_k, variant == kPipeTailVariant);
-        const int64_t items = (int64_t)pp.full_tiles + (int64_t)pp.tail_tiles * pp.splits;
-        // exactly one item per CU: fp16 always; bf16 from 64 K steps per item on (2048 x 12288 x 4096 cut in two,
-        // 96 steps: 216 against 220 us; 16384 x 2048 x 1024, 32 steps: 79 against 74)
-        const int64_t steps = pp.tail_tiles > 0 && pp.full_tiles == 0 ? pp.iters_per_split : K / 64;
-        if (items > 256 || (items == 256 && (dtype == AWQ_F16 || steps >= 64)))
-            variant = variant == kPipeVariant ? kRegbVariant : kRegbTailVariant;
     }
     const GemmVariant& gv = kGemmVariants[variant];
     if (cdiv(M, gv.BM) > 65535) {
@@ -396,8 +410,9 @@ static int gemm_dispatch(const char* fn, const void* x, const int32_t* qweight, 
             break;
         case kRegbVariant:
         case kRegbTailVariant:
-            // (group sizes below 64 and widths that cut a wave's 16 word columns run the pipelined kernel)
-            e = g % 64 == 0 && N % 128 == 0 ? launch_gemm_regb(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
+            // (group sizes below 64, widths that cut a wave's 16 word columns and tensors of 2 GiB or more run the
+            // pipelined kernel)
+            e = regb_takes(N, K, g) ? launch_gemm_regb(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
                                                workspace, split_k, variant == kRegbTailVariant, s, act)
                             : launch_gemm_pipe(dtype, x, qweight, qscales, qzeros, bias, y, (int)M, (int)N, (int)K, (int)g,
                                                workspace, split_k, variant == kRegbTailVariant, s, act);
@@ -432,13 +447,15 @@ extern "C" const char* awq_gemm_variant_name(int variant) {
     return (variant >= 0 && variant < awq::kNumGemmVariants) ? awq::kGemmVariants[variant].name : "";
 }
 
-extern "C" int awq_gemm_plan(int64_t M, int64_t N, int64_t K, int* variant, int* split_k) {
-    if (!variant || !split_k || M < 1 || N < 8 || N % 8 != 0 || K < awq::kBK || K % awq::kBK != 0) {
-        awq::set_error("awq_gemm_plan: not a shape awq_gemm takes (M=%lld N=%lld K=%lld)", (long long)M, (long long)N,
-                       (long long)K);
+extern "C" int awq_gemm_plan(int64_t M, int64_t N, int64_t K, int64_t group_size, int dtype, int* variant,
+                             int* split_k) {
+    if (!variant || !split_k || M < 1 || N < 8 || N % 8 != 0 || K < awq::kBK || K % awq::kBK != 0 || group_size < 1 ||
+        K % group_size != 0 || (dtype != AWQ_F16 && dtype != AWQ_BF16)) {
+        awq::set_error("awq_gemm_plan: not a problem awq_gemm takes (M=%lld N=%lld K=%lld g=%lld dtype=%d)", (long long)M,
+                       (long long)N, (long long)K, (long long)group_size, dtype);
         return AWQ_ERR_UNSUPPORTED;
     }
-    awq::pick_gemm(M, N, K, variant, split_k);
+    awq::plan_gemm(M, N, K, group_size, dtype, variant, split_k);
     return AWQ_OK;
 }
 
@@ -470,9 +487,9 @@ extern "C" int awq_gemm(const void* x, const int32_t* qweight, const void* qscal
                         int64_t K, int64_t group_size, int dtype, void* workspace,
                         size_t workspace_bytes, void* stream) {
     int v = 0, s = 1;
-    if (K >= awq::kBK && N >= 8 && M >= 1) awq::pick_gemm(M, N, K, &v, &s);
+    if (K >= awq::kBK && N >= 8 && M >= 1 && group_size > 0) awq::plan_gemm(M, N, K, group_size, dtype, &v, &s);
     return awq::gemm_dispatch("awq_gemm", x, qweight, qscales, qzeros, bias, y, M, N, K, group_size,
-                              dtype, workspace, workspace_bytes, stream, v, s, 0, true);
+                              dtype, workspace, workspace_bytes, stream, v, s);
 }
 
 // 65..128 rows go to the GEMV (blocks of 16 rows) on weights up to this size, see kGemvMaxRows in awq_gemv.hip
@@ -495,7 +512,7 @@ extern "C" size_t awq_linear_swiglu_workspace_bytes(int64_t M, int64_t N, int64_
     if (K < awq::kBK || N < 16 || M < 1) return 0;
     const size_t a = M <= 64 ? awq_gemv_workspace_bytes(M, N, K) : 0;
     int v, s;
-    awq::pick_gemm_pipe(M, N, K, &v, &s);
+    awq::plan_gemm_tile256(M, N, K, 128, AWQ_F16, &v, &s);   // the workspace is the same for both 256 x 256 kernels
     const size_t b = awq::gemm_ws_bytes(M, N, K, v, s);
     return a > b ? a : b;
 }
@@ -509,9 +526,10 @@ extern "C" int awq_linear_swiglu(const void* x, const int32_t* qweight, const vo
         return awq_gemv_swiglu(x, qweight, qscales, qzeros, y, M, N, K, group_size, dtype, workspace,
                                workspace_bytes, stream);
     int v = awq::kPipeVariant, s = 1;
-    if (K >= awq::kBK && N >= 16 && M >= 1) awq::pick_gemm_pipe(M, N, K, &v, &s);
+    if (K >= awq::kBK && N >= 16 && M >= 1 && group_size > 0)
+        awq::plan_gemm_tile256(M, N, K, group_size, dtype, &v, &s);
     return awq::gemm_dispatch("awq_linear_swiglu", x, qweight, qscales, qzeros, nullptr, y, M, N, K, group_size,
-                              dtype, workspace, workspace_bytes, stream, v, s, 1, true);
+                              dtype, workspace, workspace_bytes, stream, v, s, 1);
 }
 
 extern "C" int awq_linear(const void* x, const int32_t* qweight, const void* qscales,

@@ -276,6 +276,27 @@ __device__ __forceinline__ void unpack_all(const uint32_t (&w)[8], uint32_t zw, 
     }
 }
 
+// Which row tiles of a half step (ks = 0, 1; m = 0..7) have global loads issued behind them, and how many loads a wave
+// has issued between the last part of an A tile and the barrier that needs the tile complete.
+constexpr int kRegbGroupLoads = 2;   // load_group at the top of a step: the zero word and the scales
+constexpr bool regb_issues_words(int m) { return (m & 1) != 0; }                      // two packed words
+constexpr bool regb_issues_a_part(int ks, int m) { return m >= 1 && (ks == 0 || m == 1); }   // one part of the A tile
+constexpr int regb_a_parts_per_step() {
+    int n = 0;
+    for (int ks = 0; ks < 2; ++ks)
+        for (int m = 0; m < 8; ++m) n += regb_issues_a_part(ks, m) ? 1 : 0;
+    return n;
+}
+// The last part goes out behind row tile 1 of the second half, after that row tile's words; the barrier that needs
+// the tile sits in row tile 0 of the next step's second half, before that row tile issues anything.
+constexpr int regb_loads_after_last_a_part() {
+    int n = 0;
+    for (int m = 2; m < 8; ++m) n += (regb_issues_words(m) ? 2 : 0) + (regb_issues_a_part(1, m) ? 1 : 0);
+    n += kRegbGroupLoads;
+    for (int m = 0; m < 8; ++m) n += (regb_issues_words(m) ? 2 : 0) + (regb_issues_a_part(0, m) ? 1 : 0);
+    return n;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_regb_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
@@ -484,6 +505,11 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
     // whose LDS buffer (three in rotation) this fills.  The A tile of step + 1 is complete at the second barrier of a
     // step: 23 loads have been issued since its last part (25 if the compiler puts that part in front of the two words
     // that go out behind the same row tile).  "Step + 2" is the cursor `pf`: it walks the workgroup's items end to end.
+    // The wait in front of a step's second barrier is counted by hand; the count comes from the same predicates the
+    // issue sites below use, so an edit that adds, drops or moves a load changes the wait with it.
+    constexpr int kWaitATile = regb_loads_after_last_a_part();
+    static_assert(kWaitATile == 23, "loads in flight allowed at the second barrier of a step");
+    static_assert(regb_a_parts_per_step() == NDMA, "every part of the A tile is issued once per step");
     auto main_loop = [&](auto role) {
         constexpr int ROLE = decltype(role)::value;
         FragUnpack<T, ROLE> up;
@@ -552,7 +578,7 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
                             // stores completed behind row tile 0) -- and, in the second half, its part of the A tile of
                             // step + 1.  A bare barrier: __syncthreads() would also wait for this step's own loads.
                             if (ks == 0) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                            else asm volatile("s_waitcnt vmcnt(23) lgkmcnt(0)" ::: "memory");
+                            else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kWaitATile) : "memory");
                             __builtin_amdgcn_s_barrier();
                             asm volatile("" ::: "memory");
                         } else if (m <= 4) {
@@ -562,11 +588,11 @@ __global__ __launch_bounds__(256) void gemm_regb_kernel(
                             bf[1 - ks][FragUnpack<T, ROLE>::own(i)] = xprev[x_own + i * 64];
                             bf[1 - ks][FragUnpack<T, 1 - ROLE>::own(i)] = xprev[x_partner + i * 64];
                         }
-                        if (m & 1) {
+                        if (regb_issues_words(m)) {
                             ws[ks][m - 1] = load_word(2 * pf_it + ks, m - 1);
                             ws[ks][m] = load_word(2 * pf_it + ks, m);
                         }
-                        if (m >= 1 && (ks == 0 || m == 1)) dma_a_part(pf_it, nnb, ks == 0 ? m - 1 : 7);
+                        if (regb_issues_a_part(ks, m)) dma_a_part(pf_it, nnb, ks == 0 ? m - 1 : 7);
                         __builtin_amdgcn_sched_barrier(0);
                     }
 #pragma unroll
@@ -611,7 +637,9 @@ hipError_t launch_regb(const void* x, const int32_t* qweight, const void* qscale
         raised = true;
     }
     (void)hipGetLastError();
-    // one resident workgroup per CU (128 KiB of LDS each); the CU count is asked for once
+    // one resident workgroup per CU (128 KiB of LDS each); the CU count is asked for once per process, of the device
+    // that is current at the first launch (a larger grid on another device is still correct: the kernel strides by
+    // its grid size, and workgroups beyond a device's CUs wait their turn)
     static int resident = 0;
     if (resident <= 0) {
         int dev = 0, cus = 0;

@@ -947,15 +947,20 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
             u32x4 sv = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
             for (int s = 0; s < CH; ++s) {
-                // loads still allowed in flight: the later steps' (2 each, 3 with an x load per step) and zeros/scales
+                // Loads still allowed in flight while step s is read: those issue_dma issues behind it -- the later
+                // steps' (kWLoads weight loads each, one more where x travels per step) and the zero words and scales.
+                // The counts come from the constants issue_dma's order is written with.
+                constexpr int kWLoads = 2, kZsLoads = 2;
+                static_assert(3 * (kWLoads + 1) + kZsLoads <= 15, "the wait count is four bits wide here");
+                static_assert(CH == 4, "one wait per step below");
                 if (x_few) {
-                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
-                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
-                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * kWLoads + kZsLoads));
+                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kWLoads + kZsLoads));
+                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (1 * kWLoads + kZsLoads));
                 } else {
-                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | 11);
-                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
-                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | 5);
+                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * (kWLoads + 1) + kZsLoads));
+                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (kWLoads + 1) + kZsLoads));
+                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (1 * (kWLoads + 1) + kZsLoads));
                 }
                 if (s == 3) __builtin_amdgcn_s_waitcnt(0x0F70);
                 asm volatile("" ::: "memory");

@@ -197,25 +197,26 @@ def test_gemm_default_kernel_by_work_items(dtype, M, K, N):
     # The default entry point runs the register-operand kernel (r) where the plan's work items -- whole tiles plus the
     # K slices of the tail tiles -- outnumber the 256 CUs (16 x 17 = 272 tiles); at exactly 256 items (16 x 16 tiles, or
     # 8 x 16 cut in two) in fp16, and in bf16 if an item has 64 K steps at least; the pipelined kernel (p) otherwise
-    # (4 x 16 tiles cut in two): bit for bit what the forced variants give.
+    # (4 x 16 tiles cut in two).  awq_gemm_plan names that kernel, and forcing the planned pair gives the same bits.
     import ctypes
     L = _lib.lib()
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
     v, sp = ctypes.c_int(), ctypes.c_int()
-    assert L.awq_gemm_plan(M, N, K, ctypes.byref(v), ctypes.byref(sp)) == 0
-    assert names[v.value] in ("256x256p", "256x256pt")
+    dt = _lib.AWQ_F16 if dtype == "f16" else _lib.AWQ_BF16
+    assert L.awq_gemm_plan(M, N, K, 128, dt, ctypes.byref(v), ctypes.byref(sp)) == 0
+    name = names[v.value]
     tiles = (M // 256) * (N // 256)
-    tail = tiles % 256 if names[v.value] == "256x256pt" else (tiles if sp.value > 1 else 0)
+    tail = tiles % 256 if name.endswith("t") else (tiles if sp.value > 1 else 0)
     items = tiles - tail + tail * sp.value
-    print(f"gemm default {dtype} M={M} K={K} N={N}: plan {names[v.value]} split {sp.value}, {items} items", flush=True)
+    print(f"gemm default {dtype} M={M} K={K} N={N}: plan {name} split {sp.value}, {items} items", flush=True)
+    steps = K // 64 // (sp.value if tail == tiles else 1)
+    use_r = items > 256 or (items == 256 and (dtype == "f16" or steps >= 64))
+    assert name in (("256x256r", "256x256rt") if use_r else ("256x256p", "256x256pt")), (name, items, steps)
     p = random_packed(K, N, 128, dtype, seed=123)
     dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
     xd = to_dev(make_x(M, K, dtype, seed=124), dtype)
     y = nq.awq_gemm(xd, *dev, 8)
-    steps = K // 64 // (sp.value if tail == tiles else 1)
-    use_r = items > 256 or (items == 256 and (dtype == "f16" or steps >= 64))
-    forced = names[v.value].replace("p", "r") if use_r else names[v.value]
-    assert torch.equal(y, awq_gemm_variant(xd, *dev, names.index(forced), sp.value)), forced
+    assert torch.equal(y, awq_gemm_variant(xd, *dev, v.value, sp.value)), name
     rows = torch.arange(0, M, 97, device="cuda")
     ref = xd[rows].float() @ nq.awq_dequantize(*dev).float()
     assert ((y[rows].float() - ref).abs().max() / ref.abs().max()).item() <= TIGHT[dtype]
@@ -246,7 +247,7 @@ def test_gemm_largest_shapes_properties(M, K, N):
     names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
     import ctypes
     v, sp = ctypes.c_int(), ctypes.c_int()
-    assert L.awq_gemm_plan(M, N, K, ctypes.byref(v), ctypes.byref(sp)) == 0
+    assert L.awq_gemm_plan(M, N, K, 128, _lib.AWQ_BF16, ctypes.byref(v), ctypes.byref(sp)) == 0
     g = torch.Generator(device="cuda").manual_seed(M + K)
     qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=g)
     qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, N // 8), dtype=torch.int32, device="cuda", generator=g)

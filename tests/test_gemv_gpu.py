@@ -240,3 +240,47 @@ def test_gemv_row_blocks_up_to_128_rows(dt):
         assert torch.equal(y, awq_gemv_variant(to_dev(xb, dt), *dev, variant, split))
         yd = nq.awq_gemm(to_dev(xb, dt), *dev, 8)          # the default dispatch takes the same route
         _check(yd, xb, p, dt)
+
+
+def test_gemv_splitk_exchange_endurance():
+    """About 500 launches cycling three split-K problems (1, 16 and 32 rows) back to back on one stream, sharing one
+    workspace: the cross-workgroup exchange of partials (write-through stores, arrival counter, last arriver adds in
+    split order, counter left at zero) must give the bits of the first launch every time.  Stops at the first
+    mismatch."""
+    import ctypes
+    L = _lib.lib()
+    names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
+    cases = []
+    for (M, K, N, dtype) in ((1, 2048, 1024, "f16"), (16, 5120, 25600, "bf16"), (32, 3072, 1024, "f16")):
+        v, sp = ctypes.c_int(), ctypes.c_int()
+        assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
+        assert sp.value > 1 and not names[v.value].startswith("wide"), (M, K, N, names[v.value], sp.value)
+        gen = torch.Generator(device="cuda").manual_seed(M + K)
+        tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+        qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+        qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 128, N // 8), dtype=torch.int32, device="cuda", generator=gen)
+        qs = (torch.rand(K // 128, N, device="cuda", generator=gen) * 0.02 + 0.001).to(tdt)
+        x = torch.randn(M, K, device="cuda", generator=gen).to(tdt)
+        cases.append((M, K, N, _lib.dtype_id(tdt), x, qw, qs, qz, torch.empty(M, N, dtype=tdt, device="cuda")))
+    nbytes = max(L.awq_gemv_workspace_bytes(M, N, K) for (M, K, N, *_rest) in cases)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    stream = _lib.current_stream_ptr(ws.device)
+
+    def launch(c):
+        M, K, N, did, x, qw, qs, qz, y = c
+        _lib.check(L.awq_gemv(x.data_ptr(), qw.data_ptr(), qs.data_ptr(), qz.data_ptr(), None, y.data_ptr(), M, N, K, 128,
+                              did, ws.data_ptr(), ws.numel(), stream))
+    first = []
+    for c in cases:
+        launch(c)
+        first.append(c[-1].clone())
+    print("gemv split-K endurance: 168 rounds of 3 launches", flush=True)
+    for rnd in range(168):
+        for c in cases:
+            c[-1].fill_(float("nan"))
+        for c in cases:      # three launches back to back: the second starts while the first's tail may still run
+            launch(c)
+        for i, c in enumerate(cases):
+            assert torch.equal(c[-1], first[i]), f"round {rnd}: launch {i} (M={c[0]} K={c[1]} N={c[2]}) changed bits"
+    # every arrival counter is back at zero (the first 16 KiB of the workspace)
+    assert torch.count_nonzero(ws[:16384]) == 0

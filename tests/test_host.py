@@ -176,10 +176,21 @@ def test_dispatch_plans_are_consistent():
         for M in (17, 64, 65, 128, 129, 512, 1000, 2048, 8192):
             if K % 64:
                 continue
-            rc, v, s = _plan(L.awq_gemm_plan, M, N, K)
+            rc, v, s = _plan(L.awq_gemm_plan, M, N, K, 128, _lib.AWQ_BF16)
             assert rc == 0 and 0 <= v < len(gemm_names) and 1 <= s <= 16, (M, N, K, rc, v, s)
             assert s <= max(K // 64 // 8, 1)                         # at least 8 K steps per split
             assert (gemm_names[v].startswith("256x256")) == (M > 128)
+            # the plan names the kernel that runs: the register-operand one (r) only where the work items reach the
+            # 256 CUs, the group size is a multiple of 64 and N of 128; never for a group size it does not take
+            tiles = -(-M // 256) * -(-N // 256)
+            tail = tiles % 256 if gemm_names[v].endswith("t") else (tiles if s > 1 else 0)
+            items = tiles - tail + tail * s
+            if gemm_names[v] in ("256x256r", "256x256rt"):
+                assert items >= 256 and N % 128 == 0, (M, N, K, gemm_names[v], s)
+            elif gemm_names[v] in ("256x256p", "256x256pt") and N % 128 == 0:
+                assert items <= 256, (M, N, K, gemm_names[v], s)
+            rc32, v32, s32 = _plan(L.awq_gemm_plan, M, N, K, 32, _lib.AWQ_BF16)
+            assert rc32 == 0 and s32 == s and gemm_names[v32] == gemm_names[v].replace("r", "p"), (M, N, K)
             assert L.awq_gemm_ex_workspace_bytes(M, N, K, v, s) == L.awq_gemm_workspace_bytes(M, N, K)
             assert L.awq_gemm_workspace_bytes(M, N, K) <= L.awq_linear_workspace_bytes(M, N, K)
     # the whole-rounds rule for 5..64 rows: 272 column tiles are cut so that the workgroups fill the 256 CUs evenly
@@ -189,9 +200,9 @@ def test_dispatch_plans_are_consistent():
     assert wgs / (256 * -(-wgs // 256)) >= 0.8
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
     # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
-    rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120)
+    rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120, 128, _lib.AWQ_BF16)
     assert rc == 0 and gemm_names[v] == "128x128" and s in (2, 5), s
-    rc, v, s = _plan(L.awq_gemm_plan, 96, 5120, 25600)     # 40 tiles, 400 K steps: about 12 splits, one round
+    rc, v, s = _plan(L.awq_gemm_plan, 96, 5120, 25600, 128, _lib.AWQ_BF16)     # 40 tiles, 400 K steps: about 12 splits, one round
     assert rc == 0 and gemm_names[v] == "128x128" and 40 * s <= 512 and s >= 8, s
     # GEMV at up to four rows on a short K: one 128-row chunk per wave of the four-wave workgroups
     rc, v, s = _plan(L.awq_gemv_plan, 1, 1024, 2048, 128)
@@ -203,7 +214,19 @@ def test_dispatch_plans_are_consistent():
     assert rc == 0 and gemv_names[v] == "dma1x4" and s == 1, (gemv_names[v], s)
     assert L.awq_gemv_workspace_bytes(128, 2048, 2048) <= L.awq_linear_workspace_bytes(128, 2048, 2048)
     assert _plan(L.awq_gemv_plan, 4, 1024, 1000, 128)[0] != 0
-    assert _plan(L.awq_gemm_plan, 64, 1024, 96)[0] != 0
+    assert _plan(L.awq_gemm_plan, 64, 1024, 96, 32, _lib.AWQ_BF16)[0] != 0
+    # which 256 x 256 kernel: more items than CUs -> r in both types; exactly 256 items -> fp16 r, bf16 r only with 64
+    # K steps per item or more; fewer -> p
+    for (M, N, K, f16_name, bf16_name) in ((8192, 12288, 4096, "256x256r", "256x256r"),
+                                           (4096, 4096, 1024, "256x256r", "256x256p"),
+                                           (4096, 4096, 4096, "256x256r", "256x256r"),
+                                           (1024, 4096, 1024, "256x256p", "256x256p")):
+        assert gemm_names[_plan(L.awq_gemm_plan, M, N, K, 128, _lib.AWQ_F16)[1]] == f16_name, (M, N, K)
+        assert gemm_names[_plan(L.awq_gemm_plan, M, N, K, 128, _lib.AWQ_BF16)[1]] == bf16_name, (M, N, K)
+    # the register-operand kernel addresses a launch with 32-bit offsets: a packed weight of 2 GiB or a K whose 256
+    # rows of x reach 2 GiB stay on the pipelined kernel
+    assert gemm_names[_plan(L.awq_gemm_plan, 8192, 65536, 32768, 128, _lib.AWQ_F16)[1]].startswith("256x256r")
+    assert gemm_names[_plan(L.awq_gemm_plan, 8192, 65536, 65536, 128, _lib.AWQ_F16)[1]].startswith("256x256p")
 
 
 def test_every_entry_point_validates_before_touching_a_device():

@@ -318,6 +318,34 @@ def test_engine_qwen3_32b_widths_batch_64_context_2048():
 
 
 @pytest.mark.gpu
+def test_engine_mixed_decode_and_long_prefill_qwen3_32b_widths():
+    """The mixed run of the largest configuration in miniature: two blocks at the Qwen3-32B widths, one serve() call in
+    which eight rows decode at a context of 1,024 and more while a longer request (1,536 tokens) waits, is admitted
+    when the first row frees and is prefilled between two decode steps of the other rows.  Every request's
+    continuation is checked against the full-recompute forward."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+    print("engine: mixed decode + long prefill at Qwen3-32B widths, 2 layers", flush=True)
+    cfg = dict(QWEN3_32B, num_hidden_layers=2, max_position_embeddings=2048)
+    model = random_awq_qwen3(cfg, seed=31, std=0.02)
+    rg = torch.Generator().manual_seed(32)
+    B, P, LONG = 8, 1024, 1536
+    prompts = torch.randint(0, cfg["vocab_size"], (B, P), generator=rg).tolist()
+    long_prompt = torch.randint(0, cfg["vocab_size"], (LONG,), generator=rg).tolist()
+    reqs = [(p, 3 if i == 0 else 8) for i, p in enumerate(prompts)] + [(long_prompt, 4)]
+    eng = LLMEngine(model, max_batch=B, max_seq_len=LONG + 64, block_size=64, use_graph=True)
+    st = {}
+    got = eng.serve(reqs, stats=st, batch_prefill=True, max_prefill_tokens=4 * P)
+    assert [len(g) for g in got] == [m for _, m in reqs]
+    long_pf = [p for p in st["prefill_log"] if p[0] == LONG]
+    assert len(long_pf) == 1 and long_pf[0][1] == 1, st["prefill_log"]
+    assert 1 <= long_pf[0][2] < st["decode_steps"], "the long prefill must sit between decode steps of the other rows"
+    for (prompt, _), cont in zip(reqs, got):
+        _teacher_forced_check(model, [prompt], [cont])
+    assert eng.serve(reqs, batch_prefill=True, max_prefill_tokens=4 * P) == got
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("group_size,max_batch", [(64, 4), (128, 65), (32, 3)])
 def test_engine_shapes_outside_the_fused_decode_forms(group_size, max_batch):
     """Group sizes 32 / 64 and widths that are not multiples of 128 (the register-path GEMV, no q|k|v / gate|up / norm

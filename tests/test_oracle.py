@@ -330,3 +330,33 @@ def test_splitk_ref_closed_forms(dtype):
     y1 = o.from_bits16(a, dtype)
     y2 = o.from_bits16(o.linear_splitk_ref(x2, p["qweight"], p["qzeros"], p["qscales"], dtype, 8, 32), dtype)
     assert np.array_equal(y2, 2.0 * y1)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("g", [32, 128])
+def test_torch_cpu_path_equals_the_oracle(dtype, g):
+    """oracle/torch_cpu_path.py -- the restatement timed as the CPU baseline -- against the pinned numpy oracle: its
+    dequantised weight is the oracle's bit for bit, its product (fp32-upcast matmul) is the fp32-accumulation oracle's
+    up to the rounding of the output and the summation order."""
+    import torch
+    from conftest import make_case, make_x, random_packed
+    from oracle import torch_cpu_path as cpu
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    for p in (make_case(256, 72, g, dtype, seed=3), random_packed(384, 64, g, dtype, seed=4)):
+        qw, qz = torch.from_numpy(p["qweight"]), torch.from_numpy(p["qzeros"])
+        qs = torch.from_numpy(p["qscales"].view(np.int16)).view(tdt)
+        assert np.array_equal(cpu.unpack(qw).numpy(), o.unpack_awq(p["qweight"]))
+        w = cpu.dequant(qw, qs, qz)
+        assert w.dtype == tdt and np.array_equal(bits(w), o.dequant(p["qweight"], p["qzeros"], p["qscales"], dtype))
+        K = p["qweight"].shape[0]
+        xb = make_x(5, K, dtype, seed=6)
+        x = torch.from_numpy(xb.view(np.int16)).view(tdt)
+        ref = o.linear_fp32(xb, p["qweight"], p["qzeros"], p["qscales"], dtype)
+        y = cpu.linear(x, qw, qs, qz, upcast=True)
+        assert y.dtype == tdt
+        # the output is rounded to 16 bits (half an ulp: 2^-11 / 2^-8 of the value); 1e-3 with fp16
+        tol = 1e-3 if dtype == "f16" else 4e-3
+        assert o.max_rel_err(y.float().numpy(), ref) <= tol
+        # the native 16-bit matmul agrees with the reference's tolerance for the product (1e-2)
+        assert o.max_rel_err(cpu.linear(x, qw, qs, qz, upcast=False).float().numpy(), ref) <= 1e-2
