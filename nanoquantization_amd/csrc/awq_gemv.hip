@@ -542,45 +542,118 @@ __device__ __forceinline__ void gemv_reduce_store(f32x4 (&acc)[8 * V], int m_bas
     }
 }
 
+// out += partials of splits first .. splits - 1 at (row m, columns n0 .. n0 + 7), in split order; eight splits (two
+// 16-byte loads each) in flight at a time.
+__device__ __forceinline__ void add_split_partials(float (&out)[8], const float* __restrict__ partials, int first,
+                                                   int splits, int M, int m, int N, size_t n0) {
+    for (int s0 = first; s0 < splits; s0 += 8) {
+        f32x4 lo[8], hi[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int s = min(s0 + u, splits - 1);
+            const float* p = partials + ((size_t)s * M + m) * N + n0;
+            lo[u] = fetch_f32x4_nowait(p);
+            hi[u] = fetch_f32x4_nowait(p + 4);
+        }
+        fetch_wait(lo, hi);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (s0 + u < splits) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    out[c] += lo[u][c];
+                    out[4 + c] += hi[u][c];
+                }
+            }
+    }
+}
+
+__device__ __forceinline__ void fetch_wait4(f32x4 (&a)[4], f32x4 (&b)[4]) {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3])
+                 :
+                 : "memory");
+}
+
+// The last workgroup to arrive at a tile adds the partials of all splits, in split order, and stores y.
+// An item is one word (8 columns) of one row.  With at least half as many items as threads, a thread owns an item
+// and walks the splits itself, eight in flight.  With fewer (up to 8 rows of a 128-column tile in a workgroup of four
+// waves) that would leave most threads idle behind one memory round trip per eight splits -- 32 splits at one row:
+// four round trips in a row, 13.7 us for a launch that takes 10.3 with 8 splits --, so there the threads share the
+// fetch: thread (g, item) brings splits g, g + G, ... (up to four per round, G = threads / items), stages them in LDS
+// (`red`: 128 bytes per thread at least, free by now), and the item's thread adds them from there in split order:
+// one round trip for up to 4 * G splits, and the same bits, since the order of the additions is the same.
 template <typename T, int V, int WN, int WK, int kEpi = 0>
-__device__ __forceinline__ void gemv_split_tail(int* s_last, int group, int splits,
+__device__ __forceinline__ void gemv_split_tail(float* red, int* s_last, int group, int splits,
                                                 const uint16_t* __restrict__ bias,
                                                 uint16_t* __restrict__ y, float* __restrict__ partials,
                                                 int* __restrict__ counters, int M, int N, int act,
                                                 EpiArgs ea = EpiArgs{}) {
-    constexpr int WAVES = WN * WK;
+    constexpr int WAVES = WN * WK, NT = 64 * WAVES;
     const int words = N >> 3;
     if (!arrive_last(&counters[group], splits, s_last)) return;
     const int group_words = 16 * V * WN;
     const int w_begin = group * group_words;
     const int w_count = min(group_words, words - w_begin);
-    for (int idx = threadIdx.x; idx < M * w_count; idx += 64 * WAVES) {
-        const int m = idx / w_count, wc = idx - m * w_count;
+    const int items = M * w_count;
+    const bool shared_fetch = WAVES > 1 && items * 2 <= NT && splits > 1;   // uniform
+    const int G = shared_fetch ? NT / items : 1;
+    for (int i0 = 0; i0 < items; i0 += NT) {
+        const int idx = i0 + (int)threadIdx.x;
+        const bool owner = idx < items;
+        const int m = owner ? idx / w_count : 0, wc = owner ? idx - m * w_count : 0;
         const size_t n0 = (size_t)(w_begin + wc) * 8;
         float out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         u32x4 rv = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (kEpi == 2) rv = residual_load(y, m, N, n0, true);   // in flight beside the partials
-        // fetch 8 splits at a time (two 16-byte loads each) so that their loads overlap; add in split order
-        for (int s0 = 0; s0 < splits; s0 += 8) {
-            f32x4 lo[8], hi[8];
+        if constexpr (kEpi == 2) {
+            if (owner) rv = residual_load(y, m, N, n0, true);   // in flight beside the partials
+        }
+        if (shared_fetch) {
+            // (items <= NT / 2: a single pass of the outer loop)
+            const int g = (int)threadIdx.x / items, it = (int)threadIdx.x - g * items;
+            const int fm = it / w_count;
+            const size_t fn0 = (size_t)(w_begin + (it - fm * w_count)) * 8;
+            const bool fetcher = g < G;
+            f32x4* stage = reinterpret_cast<f32x4*>(red);   // [split of the round][item][2]
+            for (int s0 = 0; s0 < splits; s0 += 4 * G) {
+                const int ns = min(4 * G, splits - s0);
+                f32x4 lo[4], hi[4];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int s = min(s0 + u, splits - 1);
-                const float* p = partials + ((size_t)s * M + m) * N + n0;
-                lo[u] = fetch_f32x4_nowait(p);
-                hi[u] = fetch_f32x4_nowait(p + 4);
-            }
-            fetch_wait(lo, hi);
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (s0 + u < splits) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        out[c] += lo[u][c];
-                        out[4 + c] += hi[u][c];
+                for (int u = 0; u < 4; ++u) {
+                    lo[u] = hi[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    const int sr = g + u * G;   // split of this round
+                    if (fetcher && sr < ns) {
+                        const float* p = partials + ((size_t)(s0 + sr) * M + fm) * N + fn0;
+                        lo[u] = fetch_f32x4_nowait(p);
+                        hi[u] = fetch_f32x4_nowait(p + 4);
                     }
                 }
+                fetch_wait4(lo, hi);
+                if (s0 > 0) __syncthreads();   // the previous round has been added
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int sr = g + u * G;
+                    if (fetcher && sr < ns) {
+                        stage[(sr * items + it) * 2] = lo[u];
+                        stage[(sr * items + it) * 2 + 1] = hi[u];
+                    }
+                }
+                __syncthreads();
+                if (owner) {
+                    for (int sr = 0; sr < ns; ++sr) {
+                        const f32x4 a = stage[(sr * items + idx) * 2], b = stage[(sr * items + idx) * 2 + 1];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            out[c] += a[c];
+                            out[4 + c] += b[c];
+                        }
+                    }
+                }
+            }
+        } else if (owner) {
+            add_split_partials(out, partials, 0, splits, M, m, N, n0);
         }
+        if (!owner) continue;   // whole groups of 16 lanes (an item count is a multiple of 16 wherever lanes exchange)
         if constexpr (kEpi == 1) {   // w_count == 16 here: the 16 lanes of a head run the same iterations
             qkv_rope_store<T>(out, m, n0, true, *ea.qe);
             continue;
@@ -629,7 +702,7 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][8 * V], float* re
                                                      y, partials, M, N, act, ea);
     }
     if (splits == 1) return;
-    gemv_split_tail<T, V, WN, WK, kEpi>(s_last, group, splits, bias, y, partials, counters, M, N, act, ea);
+    gemv_split_tail<T, V, WN, WK, kEpi>(red, s_last, group, splits, bias, y, partials, counters, M, N, act, ea);
 }
 
 // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
@@ -869,27 +942,15 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     const bool zs_lane = lane < 16;
     const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
 
-    // Order of the loads of a chunk: the weights of steps 0..3 (two loads each), x, the zero words and the scales.
-    // The step-by-step form consumes them as they land and wants x first: one load for all four steps with at most 4
-    // rows, else one per step in front of that step's weights (on multi-chunk launches that order measured 7 % slower
-    // at 16 rows).
-    auto issue_dma = [&](int c) {
-        const int row0 = c * 128;
-        uint32_t* w_lds = reinterpret_cast<uint32_t*>(stage);
-        if (STREAM && x_few && x_lane)
-            __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + row0 + xsrc), AWQ_LPTR(stage + x_off), 16, 0, 0);
-#pragma unroll
-        for (int s = 0; s < CH; ++s) {
-            if (STREAM && !x_few && x_lane)
-                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + s * 32) + xsrc),
-                                                 AWQ_LPTR(stage + x_off + s * 64 * M), 16, 0, 0);
-            const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-                __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
-                                                 16, 0, 0);
-        }
-        if (!STREAM && x_lane) {
+    // Order of the loads of a chunk: the weights of steps 0..3 (two loads each), x, the zero words and the scales;
+    // the step-by-step form consumes them as they land and wants x first (on multi-chunk launches that order measured
+    // 7 % slower at 16 rows).  x is one load for all four steps with at most 4 rows, else one per step.
+    // The x loads and the zero/scale loads run under a lane mask, and the step-by-step form counts loads by hand:
+    // each masked group is ONE block, fenced off from the unmasked weight loads.  (With an x load in front of every
+    // step's weights the compiler threaded the four equal conditions into one divergent branch and issued the weight
+    // loads in between once per side of it -- two more loads in the wave's queue than the waits below count.)
+    auto issue_x = [&](int row0) {
+        if (x_lane) {
             if (x_few) {
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + row0 + xsrc), AWQ_LPTR(stage + x_off), 16, 0, 0);
             } else {
@@ -899,6 +960,22 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
                                                      AWQ_LPTR(stage + x_off + s * 64 * M), 16, 0, 0);
             }
         }
+        __builtin_amdgcn_wave_barrier();
+    };
+    auto issue_dma = [&](int c) {
+        const int row0 = c * 128;
+        uint32_t* w_lds = reinterpret_cast<uint32_t*>(stage);
+        if constexpr (STREAM) issue_x(row0);
+#pragma unroll
+        for (int s = 0; s < CH; ++s) {
+            const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
+                                                 16, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();
+        if constexpr (!STREAM) issue_x(row0);
         if (zs_lane) {
             const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
             __builtin_amdgcn_global_load_lds(AWQ_GPTR(qzeros + (size_t)gi * words + zsrc), AWQ_LPTR(stage + zs_off),
@@ -947,21 +1024,14 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
             u32x4 sv = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
             for (int s = 0; s < CH; ++s) {
-                // Loads still allowed in flight while step s is read: those issue_dma issues behind it -- the later
-                // steps' (kWLoads weight loads each, one more where x travels per step) and the zero words and scales.
-                // The counts come from the constants issue_dma's order is written with.
+                // Loads still allowed in flight while step s is read: those issue_dma issues behind step s's weights --
+                // the later steps' weights (kWLoads each) and the zero words and scales (x went out first).
                 constexpr int kWLoads = 2, kZsLoads = 2;
-                static_assert(3 * (kWLoads + 1) + kZsLoads <= 15, "the wait count is four bits wide here");
+                static_assert(3 * kWLoads + kZsLoads <= 15, "the wait count is four bits wide here");
                 static_assert(CH == 4, "one wait per step below");
-                if (x_few) {
-                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * kWLoads + kZsLoads));
-                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kWLoads + kZsLoads));
-                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (1 * kWLoads + kZsLoads));
-                } else {
-                    if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * (kWLoads + 1) + kZsLoads));
-                    if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (kWLoads + 1) + kZsLoads));
-                    if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (1 * (kWLoads + 1) + kZsLoads));
-                }
+                if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * kWLoads + kZsLoads));
+                if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kWLoads + kZsLoads));
+                if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (1 * kWLoads + kZsLoads));
                 if (s == 3) __builtin_amdgcn_s_waitcnt(0x0F70);
                 asm volatile("" ::: "memory");
                 uint32_t w[8];
@@ -1485,12 +1555,24 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         } else if (chunks <= 8) {
             v = kDma1x8;
         } else if (M <= 4) {
-            s = cdiv(3072, tiles * 4);
+            // About 2048 waves in four-wave workgroups and no more than 16 splits: every split of a tile bumps the
+            // same arrival counter, and those updates are served one after the other -- 9728 x 2560 at one row 13.7 us
+            // in 26 splits, 10.5 in 14; 17408 x 5120 17.5 us in 20, 16.3 in 13; 12288 x 4096 13.1 us in 24, 12.5 in 16.
+            // Eight-wave workgroups, i.e. half the splits for the same waves, on the longest K with few column tiles
+            // (25600 x 5120: 22.3 us in 25 splits of four waves, 20.4 in 13 of eight; on shorter K they lose:
+            // 4096 x 2048 8.3 us in 4 splits of eight waves against 7.4 in 8 of four).
             // short K: one chunk per wave (the step-by-step form), at most 10 splits (the tail is a larger share of
-            // a 6 us launch: 2048 x 1024 at one row 5.55 us in 8 splits, 5.23 in 4); long K: up to 32
-            const int64_t cap = chunks < 64 ? (chunks / 4 < 10 ? chunks / 4 : 10) : 32;
+            // a 6 us launch: 2048 x 1024 at one row 5.55 us in 8 splits, 5.23 in 4)
+            const int64_t cap = chunks < 64 ? (chunks / 4 < 10 ? chunks / 4 : 10) : 16;
+            int64_t wk = 4;
+            s = cdiv(2048, tiles * 4);
+            if (tiles <= 48 && chunks >= 160) {
+                wk = 8;
+                s = cdiv(4096, tiles * 8);
+            }
+            if (wk == 8) v = kDma1x8;
             if (s > cap) s = cap;
-            s = balance_splits(chunks, s, 4, cap);
+            s = balance_splits(chunks, s, wk, cap);
         } else {
             // 5..64 rows.  A CU streams at a fixed rate whatever the number of workgroups on it, so the launch lasts
             // as long as the CU with the most bytes: at least about 200 workgroups, and a count that fills whole

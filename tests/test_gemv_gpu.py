@@ -44,6 +44,20 @@ def test_gemv_decode_sweep_f16(K, N, M):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("K,N", [(1024, 2048), (2048, 1024)])
+def test_gemv_every_row_count_step_by_step_form(dtype, K, N):
+    """1..16 rows on decode-size shapes (one chunk per wave: the step-by-step form, which waits for its loads by
+    count).  Between 5 and 15 rows the activation loads run under a lane mask that cuts a wave in two."""
+    p = make_case(K, N, 128, dtype, seed=K + 3 * N)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    for M in range(1, 17):
+        print(f"gemv rows {dtype} M={M} K={K} N={N}", flush=True)
+        xb = make_x(M, K, dtype, seed=40 + M)
+        y = nq.awq_gemm(to_dev(xb, dtype), *dev, 8)
+        _check(y, xb, p, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_gemv_every_variant_and_split(dtype):
     L = _lib.lib()
     K, N = 1024, 1024
@@ -251,7 +265,7 @@ def test_gemv_splitk_exchange_endurance():
     L = _lib.lib()
     names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
     cases = []
-    for (M, K, N, dtype) in ((1, 2048, 1024, "f16"), (16, 5120, 25600, "bf16"), (32, 3072, 1024, "f16")):
+    for (M, K, N, dtype) in ((1, 2048, 1024, "f16"), (16, 4096, 4096, "bf16"), (32, 3072, 1024, "f16")):
         v, sp = ctypes.c_int(), ctypes.c_int()
         assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
         assert sp.value > 1 and not names[v.value].startswith("wide"), (M, K, N, names[v.value], sp.value)
