@@ -815,6 +815,8 @@ __host__ __device__ constexpr int dma_wave_bytes(int M) { return 8192 + 256 * M 
 // epilogue.  The extra arguments of a form stay out of the plain kernel's argument block (the launch-bound decode
 // GEMVs measured 0.2-0.5 us slower with them).
 constexpr int kModeQkv = 1, kModeNorm = 2, kModeResid = 4;
+// the step-by-step form takes the RMSNorm prologue for inputs of up to this many 128-column tiles (K <= 2048)
+constexpr int kNormStreamChunks = 16;
 template <int MODE>
 struct GemvExtra {};
 template <>
@@ -995,22 +997,49 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
     f32x4 acc[1][8];
 
     float rstd = 0.f;
+    u32x4 nw0[CH];   // step-by-step form with the prologue: the norm weights of the wave's one chunk
     if constexpr (NORM) {   // the lane's row: 1 / rms from the tile sums, added in tile order (eight loads in flight)
         const float* sp = ex.np.ssq + min(j, M - 1);
         float tot = 0.f;
-        for (int t0 = 0; t0 < total_chunks; t0 += 8) {
-            float v[8];
+        if constexpr (STREAM) {
+            // (launched with up to kNormStreamChunks tiles only.)  Every statistic and the chunk's norm weights are
+            // asked for BEFORE the chunk's loads: loads return in issue order, and anything issued behind the weights
+            // would keep the normalisation below waiting for the whole chunk.
+            float v[kNormStreamChunks];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = sp[(size_t)min(t0 + u, total_chunks - 1) * ex.np.m_stride];
-            if (t0 == 0 && c0 < c1) issue_dma(c0);   // behind the first statistics loads, ahead of their use
+            for (int u = 0; u < kNormStreamChunks; ++u) v[u] = sp[(size_t)min(u, total_chunks - 1) * ex.np.m_stride];
+            if (c0 < c1) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) tot += t0 + u < total_chunks ? v[u] : 0.f;
+                for (int s = 0; s < CH; ++s)
+                    nw0[s] = *reinterpret_cast<const u32x4*>(ex.np.weight + c0 * 128 + s * 32 + kb * 8);
+                issue_dma(c0);
+            }
+#pragma unroll
+            for (int u = 0; u < kNormStreamChunks; ++u) tot += u < total_chunks ? v[u] : 0.f;
+        } else {
+            for (int t0 = 0; t0 < total_chunks; t0 += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = sp[(size_t)min(t0 + u, total_chunks - 1) * ex.np.m_stride];
+                if (t0 == 0 && c0 < c1) issue_dma(c0);   // behind the first statistics loads, ahead of their use
+#pragma unroll
+                for (int u = 0; u < 8; ++u) tot += t0 + u < total_chunks ? v[u] : 0.f;
+            }
         }
         rstd = rsqrtf(tot / (float)K + ex.np.eps);
     } else {
         if (c0 < c1) issue_dma(c0);
     }
-    static_assert(!(STREAM && NORM), "the step-by-step form has no RMSNorm prologue");
+    // h = T(T(x * r) * w) for the 8 activations of one operand register quadruple
+    auto normalise = [&](u32x4& xa, const u32x4& nwv) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t xv = xa[i], wv = nwv[i];
+            const float lo = mul_round<T>(T::to_f32((uint16_t)(xv & 0xFFFFu)), rstd) * T::to_f32((uint16_t)(wv & 0xFFFFu));
+            const float hi = mul_round<T>(T::to_f32((uint16_t)(xv >> 16)), rstd) * T::to_f32((uint16_t)(wv >> 16));
+            xa[i] = T::pack2(lo, hi);
+        }
+    };
     int c_first = c0;
     if constexpr (STREAM) {
         // A wave with a single chunk (a decode-size launch: the chunk is all there is, and the loads of the eight
@@ -1022,13 +1051,24 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
             StepAcc sa;
             uint32_t zw = 0;
             u32x4 sv = u32x4{0u, 0u, 0u, 0u};
+            constexpr int kWLoads = 2, kZsLoads = 2;
+            static_assert(4 * kWLoads + kZsLoads <= 15, "the wait count is four bits wide here");
+            static_assert(CH == 4, "one wait per step below");
+            u32x4 xn[CH];
+            if constexpr (NORM) {
+                // x went out first: once it is there (the weights and the zeros/scales may all be on their way still)
+                // the four operand quadruples are normalised while the weights land
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (4 * kWLoads + kZsLoads));
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int s = 0; s < CH; ++s) xn[s] = *reinterpret_cast<const u32x4*>(stage + x_rd_off + s * x_rd_step);
+#pragma unroll
+                for (int s = 0; s < CH; ++s) normalise(xn[s], nw0[s]);
+            }
 #pragma unroll
             for (int s = 0; s < CH; ++s) {
                 // Loads still allowed in flight while step s is read: those issue_dma issues behind step s's weights --
                 // the later steps' weights (kWLoads each) and the zero words and scales (x went out first).
-                constexpr int kWLoads = 2, kZsLoads = 2;
-                static_assert(3 * kWLoads + kZsLoads <= 15, "the wait count is four bits wide here");
-                static_assert(CH == 4, "one wait per step below");
                 if (s == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * kWLoads + kZsLoads));
                 if (s == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kWLoads + kZsLoads));
                 if (s == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (1 * kWLoads + kZsLoads));
@@ -1037,7 +1077,9 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
                 uint32_t w[8];
 #pragma unroll
                 for (int r = 0; r < 8; ++r) w[r] = w_rd[s * 512 + r * 64];
-                const u32x4 xa = *reinterpret_cast<const u32x4*>(stage + x_rd_off + s * x_rd_step);
+                u32x4 xa;
+                if constexpr (NORM) xa = xn[s];
+                else xa = *reinterpret_cast<const u32x4*>(stage + x_rd_off + s * x_rd_step);
                 if (s == 3) {
                     zw = *reinterpret_cast<const uint32_t*>(stage + z_rd_off);
                     sv = *reinterpret_cast<const u32x4*>(stage + s_rd_off);
@@ -1081,16 +1123,7 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
         if (c + 1 < c1) issue_dma(c + 1);
         if constexpr (NORM) {
 #pragma unroll
-            for (int s = 0; s < CH; ++s)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t xv = d.xa[s][0][i], wv = nw[s][i];
-                    const float lo = mul_round<T>(T::to_f32((uint16_t)(xv & 0xFFFFu)), rstd) *
-                                     T::to_f32((uint16_t)(wv & 0xFFFFu));
-                    const float hi = mul_round<T>(T::to_f32((uint16_t)(xv >> 16)), rstd) *
-                                     T::to_f32((uint16_t)(wv >> 16));
-                    d.xa[s][0][i] = T::pack2(lo, hi);
-                }
+            for (int s = 0; s < CH; ++s) normalise(d.xa[s][0], nw[s]);
         }
         compute_chunk<T, 1, CH, 1>(d, acc);
     }
@@ -1406,7 +1439,9 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
                                    reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeResid>),
                                    reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, 0, true>),
                                    reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeQkv, true>),
-                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeResid, true>)};
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeResid, true>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeNorm, true>),
+                                   reinterpret_cast<const void*>(gemv_dma_kernel<T, WK, kModeQkv | kModeNorm, true>)};
             for (const void* f : forms) {
                 hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
                 if (e != hipSuccess) return e;
@@ -1450,12 +1485,16 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),     \
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters, \
                        M, N, K, g / 128, cps, splits, act, groups, pair_map, pf, EXTRA)
-    if (fu.qe && fu.np)
-        AWQ_DMA_LAUNCH(kModeQkv | kModeNorm, (GemvExtra<kModeQkv | kModeNorm>{*fu.qe, *fu.np}));
-    else if (fu.qe)
+    const bool norm_stream = stream_form && total_chunks <= kNormStreamChunks;
+    if (fu.qe && fu.np) {
+        if (norm_stream) AWQ_DMA_LAUNCH_FORM(kModeQkv | kModeNorm, true, (GemvExtra<kModeQkv | kModeNorm>{*fu.qe, *fu.np}));
+        else AWQ_DMA_LAUNCH(kModeQkv | kModeNorm, (GemvExtra<kModeQkv | kModeNorm>{*fu.qe, *fu.np}));
+    } else if (fu.qe)
         AWQ_DMA_LAUNCH_S(kModeQkv, (GemvExtra<kModeQkv>{*fu.qe}));
-    else if (fu.np)
-        AWQ_DMA_LAUNCH(kModeNorm, (GemvExtra<kModeNorm>{*fu.np}));
+    else if (fu.np) {
+        if (norm_stream) AWQ_DMA_LAUNCH_FORM(kModeNorm, true, (GemvExtra<kModeNorm>{*fu.np}));
+        else AWQ_DMA_LAUNCH(kModeNorm, (GemvExtra<kModeNorm>{*fu.np}));
+    }
     else if (fu.re)
         AWQ_DMA_LAUNCH_S(kModeResid, (GemvExtra<kModeResid>{*fu.re}));
     else
