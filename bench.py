@@ -15,9 +15,10 @@ the prefill GEMM TFLOP/s at the Qwen3-8B MLP shapes, the dequantise kernel, and 
 python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cfg5] [--only-cfg5] [--no-cpu]
 
 For a profiler or a counter collection to look at one kernel (no timing, no JSON line):
-python bench.py --one linear|dequant|copy K N M [--one-dtype bf16|f16] [--one-iters 6]
-launches that one problem a few times on the same seeded buffers (`copy`: a device copy of the packed weight,
-the known-size kernel the traffic counters are calibrated with).
+python bench.py --one linear|dequant|copy K N M [--one-dtype bf16|f16] [--one-iters 6] [--one-copies 1]
+launches that one problem a few times on seeded buffers, walking over `--one-copies` distinct packed weights (more
+than the 256 MB Infinity Cache holds: the launches stream from HBM as the timed sections do).  `copy`: a device copy
+of the packed weight, the known-size kernel the traffic counters are calibrated with.
 """
 from __future__ import annotations
 
@@ -34,9 +35,9 @@ sys.path.insert(0, ROOT)
 
 # HBM bytes per GEMV launch of the headline sweep, from two `rocprofv3 --pmc` runs of this file
 # (FETCH_SIZE, then WRITE_SIZE; profiles/gemv_cfg2_sweep_hbm_traffic.txt).  Each counter is scaled by
-# what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,011.5 -> 2047.3 B per count,
+# what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,012.8 -> 2047.2 B per count,
 # WRITE_SIZE 64,000 -> 1024 B per count.
-MEASURED_FETCH_BYTES_PER_LAUNCH = 1123.98 * 2047.3
+MEASURED_FETCH_BYTES_PER_LAUNCH = 1132.48 * 2047.2
 MEASURED_WRITE_BYTES_PER_LAUNCH = 100.68 * 1024.0
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
@@ -117,22 +118,25 @@ def time_eager(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
-def run_one(kind, K, N, M, dtype, iters, g=G):
-    """One problem, `iters` launches, nothing timed: the subject of a rocprofv3 run."""
+def run_one(kind, K, N, M, dtype, iters, copies=1, g=G):
+    """One problem, `iters` launches over `copies` distinct weights, nothing timed: the subject of a rocprofv3 run."""
     import nanoquantization_amd as nq
     dev = torch.device("cuda:0")
     tdt = torch.bfloat16 if dtype == "bf16" else torch.float16
     gen = torch.Generator(device=dev).manual_seed(K + N)
-    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device=dev, generator=gen)
-    qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, device=dev, generator=gen)
-    qs = (torch.rand(K // g, N, device=dev, generator=gen) * 0.02 + 0.001).to(tdt)
+    ws = []
+    for _ in range(max(1, copies)):
+        qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device=dev, generator=gen)
+        qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, device=dev, generator=gen)
+        qs = (torch.rand(K // g, N, device=dev, generator=gen) * 0.02 + 0.001).to(tdt)
+        ws.append((qw, qs, qz))
     x = torch.randn(max(M, 1), K, device=dev, generator=gen).to(tdt)
-    fn = {"linear": lambda: nq.awq_gemm(x, qw, qs, qz, 8),
-          "dequant": lambda: nq.awq_dequantize(qw, qs, qz), "copy": lambda: qw.clone()}[kind]
-    for _ in range(iters):
-        fn()
+    fn = {"linear": lambda w: nq.awq_gemm(x, w[0], w[1], w[2], 8),
+          "dequant": lambda w: nq.awq_dequantize(*w), "copy": lambda w: w[0].clone()}[kind]
+    for i in range(iters):
+        fn(ws[i % len(ws)])
     torch.cuda.synchronize()
-    print(f"{kind} K={K} N={N} M={M} {dtype}: {iters} launches")
+    print(f"{kind} K={K} N={N} M={M} {dtype}: {iters} launches over {len(ws)} weight copies")
 
 
 def gemm_kernel_name(M, N, K, dtype_name, g=G):
@@ -152,12 +156,32 @@ def gemm_kernel_name(M, N, K, dtype_name, g=G):
     return f"{kern} (plan {name}, split {sp.value})"
 
 
+def gemv_kernel_name(M, N, K, dtype_name, g=G):
+    """The kernel awq_gemv runs for a decode problem, from the library's own plan."""
+    import ctypes
+    from nanoquantization_amd import _lib
+    L = _lib.lib()
+    v, sp = ctypes.c_int(), ctypes.c_int()
+    if L.awq_gemv_plan(M, N, K, g, ctypes.byref(v), ctypes.byref(sp)) != 0:
+        return "?"
+    name = L.awq_gemv_variant_name(v.value).decode()
+    T = "F16" if dtype_name == "f16" else "BF16"
+    if name.startswith("wide"):
+        kern = f"awq::gemv_wide_kernel<{T},2,{name[-1]}> + awq::gemv_wide_reduce_kernel<{T}>"
+    elif name.startswith("dma"):
+        kern = f"awq::gemv_dma_kernel<{T},{name[5]},plain>"
+    else:
+        kern = f"awq::gemv_kernel<{T}> ({name})"
+    return f"{kern} (plan {name}, split {sp.value})"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--one", nargs=4, metavar=("KIND", "K", "N", "M"),
                     help="launch one problem a few times for a profiler: linear|dequant|copy K N M")
     ap.add_argument("--one-dtype", choices=["bf16", "f16"], default="bf16")
     ap.add_argument("--one-iters", type=int, default=6)
+    ap.add_argument("--one-copies", type=int, default=1)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -190,7 +214,7 @@ def main():
         kind, K1, N1, M1 = args.one[0], int(args.one[1]), int(args.one[2]), int(args.one[3])
         if kind not in ("linear", "dequant", "copy"):
             ap.error("--one KIND must be linear, dequant or copy")
-        run_one(kind, K1, N1, M1, args.one_dtype, args.one_iters)
+        run_one(kind, K1, N1, M1, args.one_dtype, args.one_iters, args.one_copies)
         return
     tdt = torch.float16
     torch.manual_seed(0)
@@ -222,7 +246,7 @@ def main():
         "achieved": avg_bytes / (avg_launch_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": avg_bytes / (avg_launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "traffic": MEASURED_FETCH_BYTES_PER_LAUNCH + MEASURED_WRITE_BYTES_PER_LAUNCH,
-        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 2.30 MB + write 0.10 MB) from rocprofv3 "
+        "traffic_note": "bytes per launch crossing the L2/fabric boundary (fetch 2.32 MB + write 0.10 MB) from rocprofv3 "
                         "FETCH_SIZE / WRITE_SIZE, copy-calibrated.  The counters sit between the L2s and the fabric "
                         "and cannot tell Infinity Cache hits from HBM reads: about 0.87 MB of the fetch is the prefetch "
                         "(spare workgroups read the next launch's weights once to park them in the Infinity Cache, "
@@ -274,16 +298,19 @@ def main():
                 us = time_graph(fn, 10, 2) * 1e3 / len(copies)
                 gbs = packed_bytes(K, N) / us / 1e3
                 (large if M <= 16 else batched)[f"{K}x{N}_M{M}"] = {
-                    "us": round(us, 2), "GBs": round(gbs, 1), "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4)}
+                    "us": round(us, 2), "GBs": round(gbs, 1), "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4),
+                    "kernel": gemv_kernel_name(M, N, K, "f16")}
             del copies
             torch.cuda.empty_cache()
         out["batched_decode_gemv"] = {
             "kernel": "awq::gemv_wide_kernel + awq::gemv_wide_reduce_kernel", "unit": "GB/s of packed weights",
-            "note": "17..64 rows (cfg5 decodes at 64): not HBM-bound (the same time with cache-resident weights); counters of "
-                    "this regime: vector ALU 39 %, MFMA 23 %, LDS 36 % busy, waves issuing 38 % of their lifetime",
+            "note": "17..64 rows (cfg5 decodes at 64): bound by the SIMDs' issue ports (MFMA + unpack + fold + load-to-LDS "
+                    "instructions of two lock-stepped waves per SIMD) plus the K splits' fp32 partial round trip, not by HBM",
             "cases": batched}
         best = max(v["GBs"] for v in large.values())
-        out["roofline_large"] = {"kernel": "awq::gemv_dma_kernel", "bound": "hbm", "achieved": best,
+        best_large = max(large, key=lambda k: large[k]["GBs"])
+        out["roofline_large"] = {"kernel": large[best_large]["kernel"] + f" at {best_large} (each case names its own)",
+                                 "bound": "hbm", "achieved": best,
                                  "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best / HBM_PEAK_GBS,
                                  "workload": "Qwen3-32B MLP shapes (68.1 MB packed), HBM-streaming over 6 copies",
                                  "cases": large}

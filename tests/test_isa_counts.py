@@ -1,0 +1,41 @@
+"""The step-by-step form of the staged GEMV waits for its loads by count (s_waitcnt vmcnt(N) with N worked out by
+hand from the order the loads are issued in).  The compiler is free to restructure branches around the load-to-LDS
+instructions -- it once threaded four equal lane-mask conditions into one divergent branch and issued the weight loads
+in between once per side, two more loads than the waits counted, a silent race between 5 and 15 rows.  This test
+compiles the kernel file to gfx950 assembly (no GPU needed) and counts the load-to-LDS instructions of every
+instantiation: 14 per chunk issue (1 or 4 of x sharing their first instruction, 8 of weights, 2 of zeros/scales)."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from nanoquantization_amd import build as nq_build
+
+
+@pytest.mark.skipif(shutil.which(nq_build.HIPCC) is None and not os.path.exists(nq_build.HIPCC), reason="hipcc not found")
+def test_staged_gemv_issues_each_load_once(tmp_path):
+    src = os.path.join(nq_build.CSRC, "awq_gemv.hip")
+    out = tmp_path / "awq_gemv.s"
+    flags = [f for f in nq_build.FLAGS if f not in ("-shared", "-fPIC")]
+    cmd = [nq_build.HIPCC, *flags, *nq_build.EXTRA.get("awq_gemv.hip", []), "--cuda-device-only", "-S", src, "-o", str(out)]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-2000:]
+    asm = out.read_text()
+    names = re.findall(r"^(_ZN3awq15gemv_dma_kernel[^:\s]*):", asm, re.M)
+    assert len(names) >= 32, names            # 2 types x 2 wave counts x the forms
+    seen_stream = seen_chunked = 0
+    for name in names:
+        begin = asm.index("\n" + name + ":")
+        body = asm[begin:asm.index(".Lfunc_end", begin)]
+        loads = len(re.findall(r"\bglobal_load_lds_dword", body))
+        # template arguments: <T, WK, MODE, STREAM>; the mangled name spells STREAM as Lb1 / Lb0
+        stream = re.search(r"ELi\dELi\dELb(\d)", name).group(1) == "1"
+        if stream:
+            assert loads == 14, (name, loads)      # issued once: the wave has one chunk
+            seen_stream += 1
+        else:
+            assert loads == 28, (name, loads)      # the first chunk's issue and the one in the loop
+            seen_chunked += 1
+    assert seen_stream >= 10 and seen_chunked >= 10
