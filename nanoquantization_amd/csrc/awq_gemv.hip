@@ -1155,9 +1155,10 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int M, int N, int K, int chunks_per_group, int chunks_per_split, int splits, int act) {
-    constexpr int CH = 4, WN = 4, HMT = MT / 2;
+    // HMT: pieces of x a wave brings per chunk (with one m-tile the four pieces go to waves 0..3, one each)
+    constexpr int CH = 4, WN = 4, HMT = MT >= 2 ? MT / 2 : 1;
     static_assert(DEPTH >= 2 && DEPTH <= 3, "two or three staging buffers");
-    static_assert(MT == 2 || MT == 4, "m-tiles per workgroup");
+    static_assert(MT == 1 || MT == 2 || MT == 4, "m-tiles per workgroup");
     extern __shared__ __attribute__((aligned(16))) float red[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1188,15 +1189,18 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
     uint32_t xsrc[HMT];
 #pragma unroll
     for (int i = 0; i < HMT; ++i) {
-        const int o = wave * HMT + i;
+        const int o = MT >= 2 ? wave * HMT + i : (wave & 3);
         x_s[i] = o / MT;
         x_mt[i] = o % MT;
         xsrc[i] = (uint32_t)min(16 * x_mt[i] + (lane >> 2), M - 1) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
     }
+    const bool x_wave = MT >= 2 || wave < 4;   // uniform
     const uint32_t zsrc = (uint32_t)(tile * 16 + (lane & 15));
     const bool zs_lane = lane < 16;
 
-    constexpr int kDmaOps = CH + HMT + 1;   // per wave and chunk
+    // per wave and chunk (an upper bound where a wave brings no x; only a third buffer waits by this count)
+    constexpr int kDmaOps = CH + HMT + 1;
+    static_assert(MT >= 2 || DEPTH == 2, "one m-tile: the waves' load counts differ, two buffers only");
     auto issue_dma = [&](int c, int buf) {
         const int row0 = c * 128;
         char* base = stage + buf * buf_bytes;
@@ -1210,10 +1214,12 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
                                                  16, 0, 0);
         }
+        if (x_wave) {
 #pragma unroll
-        for (int i = 0; i < HMT; ++i)
-            __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + x_s[i] * 32) + xsrc[i]),
-                                             AWQ_LPTR(base + x_s[i] * x_step + x_mt[i] * 1024), 16, 0, 0);
+            for (int i = 0; i < HMT; ++i)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + x_s[i] * 32) + xsrc[i]),
+                                                 AWQ_LPTR(base + x_s[i] * x_step + x_mt[i] * 1024), 16, 0, 0);
+        }
         if (zs_lane) {
             const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
             if (bh == 0)
@@ -1271,6 +1277,30 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
             // with every read consumed
             buf = (buf + 1 == DEPTH) ? 0 : buf + 1;
             compute_chunk_bytes<T, CH, MT, BH>(d, acc);
+        }
+        if constexpr (MT == 1) {
+            // One m-tile: the odd half hands its four fragments to its partner, which stores whole words.
+            __syncthreads();   // staging is free
+            float* xch1 = red + (size_t)wn * (16 * 64);
+            if (BH == 1) {
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) xch1[(f * 4 + r) * 64 + lane] = acc[0][f][r];
+            }
+            __syncthreads();
+            if (BH == 0) {
+                f32x4 acc8[8];
+#pragma unroll
+                for (int f = 0; f < 4; ++f) {
+                    acc8[2 * f] = acc[0][f];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc8[2 * f + 1][r] = xch1[(f * 4 + r) * 64 + lane];
+                }
+                gemv_reduce_store<T, 1, WN, 1, true>(acc8, 0, red, lane, wn, group, split, splits, bias, y, partials, M, N,
+                                                     act);
+            }
+            return;
         }
         // Exchange: this wave stores m-tiles BH*HMT .. and sends its fragments of the other m-tiles to its
         // partner (wave ^ 4).  xch[wave][(ml*4 + f)*4 + r][lane]
@@ -1362,8 +1392,9 @@ static const GemvVariant kGemvVariants[] = {
     // shared staged chunk, eight waves as 4 column tiles x 2 byte halves: wide d<DEPTH> m<MT>
     {"wided2m4", 1, 8, false, 4, 2, 4, true},
     {"wided2m2", 1, 8, false, 4, 2, 2, true},
+    {"wided2m1", 1, 8, false, 4, 2, 1, true},
 };
-enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5 };
+enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = kDma1x4;
 
@@ -1591,6 +1622,16 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             v = M > 32 ? kWideM4 : kWideM2;
             s = 256 / (N / 512);
             if (s > chunks / 4) s = chunks / 4;
+        } else if (allow_shared_chunk && M >= 5 && M <= 16 && N % 512 == 0 && N >= 24576 && K * N >= 96000000ll) {
+            // 5..16 rows on the widest weights (gate|up of Qwen3-8B and larger): the shared-chunk kernel with one
+            // m-tile -- the staged kernel's waves bring their own x, 4 KiB per chunk beside 8 KiB of weights at 16
+            // rows; shared by eight waves it is 0.5 KiB per wave.  5120 x 25600 at 8 / 16 rows 22.7 / 25.0 -> 21.3 /
+            // 21.9 us, 5120 x 51200 40.2 / 46.2 -> 36.6 / 39.5, 4096 x 24576 20.0 / 22.0 -> 18.8 / 19.5; below
+            // these widths (25600 x 5120, 5120 x 10240) its K splits' partial round trip costs more than it saves.
+            v = kWideM1;
+            s = 256 / (N / 512);
+            if (s < 2) s = 2;
+            if (s > chunks / 4) s = chunks / 4;
         } else if (chunks <= 8) {
             v = kDma1x8;
         } else if (M <= 4) {
@@ -1605,6 +1646,10 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             const int64_t cap = chunks < 64 ? (chunks / 4 < 10 ? chunks / 4 : 10) : 16;
             int64_t wk = 4;
             s = cdiv(2048, tiles * 4);
+            // and no more than two chunks per wave: a wave takes its chunks one after the other, each a round trip
+            // of its own (5120 x 51200 at one row 41.5 us in 2 splits -- five chunks per wave --, 32.5 in 5 or 6;
+            // 5120 x 34816 32.9 -> 24.9 us)
+            if (s < cdiv(chunks, 8) && cdiv(chunks, 8) <= cap) s = cdiv(chunks, 8);
             if (tiles <= 48 && chunks >= 160) {
                 wk = 8;
                 s = cdiv(4096, tiles * 8);
@@ -1739,6 +1784,10 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         case kWideM4:
             e = f16 ? launch_gemv_wide<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
                     : launch_gemv_wide<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            break;
+        case kWideM1:
+            e = f16 ? launch_gemv_wide<F16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
+                    : launch_gemv_wide<BF16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
             break;
         case kWideM2:
             e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)

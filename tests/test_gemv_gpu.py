@@ -152,6 +152,36 @@ def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N):
     assert torch.equal(y, _linear("awq_linear", to_dev(xb, dtype), *dev, bd))
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [5, 9, 16])
+def test_gemv_shared_chunk_one_m_tile(dtype, M):
+    """5..16 rows on the widest weights (N >= 24576): the default dispatch takes the shared-chunk kernel with one m-tile
+    (the odd byte halves hand their fragments to their partners, a second pass adds the K splits); with and without a
+    bias, against the oracle, and forced with other split counts (same oracle)."""
+    import ctypes
+    K, N = 4096, 24576
+    L = _lib.lib()
+    names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
+    v, sp = ctypes.c_int(), ctypes.c_int()
+    assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
+    assert names[v.value] == "wided2m1" and sp.value == 5, (names[v.value], sp.value)
+    print(f"gemv shared-chunk, one m-tile {dtype} M={M} K={K} N={N}", flush=True)
+    p = random_packed(K, N, 128, dtype, seed=K + N + M)
+    xb = make_x(M, K, dtype, seed=M)
+    bias = np.linspace(-1, 1, N).astype(np.float32)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    from nanoquantization_amd.layers.gemm import _linear
+    bd = to_dev(o.to_bits16(bias, dtype), dtype)
+    xd = to_dev(xb, dtype)
+    y = _linear("awq_linear", xd, *dev, bd)
+    _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
+    assert torch.equal(y, _linear("awq_linear", xd, *dev, bd))
+    y0 = nq.awq_gemm(xd, *dev, 8)
+    _check(y0, xb, p, dtype)
+    for split in (1, 2, 8):
+        _check(awq_gemv_variant(xd, *dev, v.value, split), xb, p, dtype)
+
+
 def test_gemv_reference_test_shape():
     # the reference's own GEMM test: K=1024, N=2048, g=32, 8 tokens, atol=1.0 against x @ w_dq.T
     # (awq/tests/dequantization_kernel.py:108-138)

@@ -166,7 +166,8 @@ def test_dispatch_plans_are_consistent():
                 else:
                     assert M <= 16
                 if name.startswith("wide"):
-                    assert M > 16 and N % 512 == 0 and K * N >= 50 << 20
+                    assert M >= 5 and N % 512 == 0 and K * N >= 50 << 20
+                    assert (name == "wided2m1") == (M <= 16) and (name == "wided2m4") == (M > 32)
                     assert N // 512 * s <= 256 + N // 512            # about one workgroup per CU
                 if not staged_ok:
                     assert not name.startswith(("dma", "wide"))
@@ -194,10 +195,15 @@ def test_dispatch_plans_are_consistent():
             assert L.awq_gemm_ex_workspace_bytes(M, N, K, v, s) == L.awq_gemm_workspace_bytes(M, N, K)
             assert L.awq_gemm_workspace_bytes(M, N, K) <= L.awq_linear_workspace_bytes(M, N, K)
     # the whole-rounds rule for 5..64 rows: 272 column tiles are cut so that the workgroups fill the 256 CUs evenly
-    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 5120, 128)
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 2048, 128)
     assert rc == 0 and gemv_names[v] == "dma1x4" and s >= 3
     wgs = 34816 // 128 * s
     assert wgs / (256 * -(-wgs // 256)) >= 0.8
+    # 5..16 rows on the widest weights: the shared-chunk kernel with one m-tile, about one workgroup per CU
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 5120, 128)
+    assert rc == 0 and gemv_names[v] == "wided2m1" and s == 3
+    rc, v, s = _plan(L.awq_gemv_plan, 4, 34816, 5120, 128)      # up to four rows: the one-tile kernel, two chunks per wave
+    assert rc == 0 and gemv_names[v] == "dma1x4" and s == 5
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
     # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
     rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120, 128, _lib.AWQ_BF16)
