@@ -1147,19 +1147,23 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
 // ALU port (one instruction per SIMD every four cycles: about 270 unpack, 140 scale/zero and 2 x 144 MFMA
 // issue slots per 128 x 128 weights at 64 rows), not the memory.
 // At the end the two halves exchange fragments through LDS so that each stores whole words of half the rows.
+// A K split leaves fp32 partials that a second kernel adds in split order -- or, TAIL (one m-tile, a few rows), the
+// last workgroup of the 512 columns to arrive, as in the one-tile kernel.
 __host__ __device__ constexpr int wide_buf_bytes(int MT) { return 4096 * MT + 4 * 8704; }
 
-template <typename T, int DEPTH, int MT>
+template <typename T, int DEPTH, int MT, bool TAIL = false>
 __global__ __launch_bounds__(512) void gemv_wide_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
-    int M, int N, int K, int chunks_per_group, int chunks_per_split, int splits, int act) {
+    int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split, int splits, int act) {
     // HMT: pieces of x a wave brings per chunk (with one m-tile the four pieces go to waves 0..3, one each)
     constexpr int CH = 4, WN = 4, HMT = MT >= 2 ? MT / 2 : 1;
     static_assert(DEPTH >= 2 && DEPTH <= 3, "two or three staging buffers");
     static_assert(MT == 1 || MT == 2 || MT == 4, "m-tiles per workgroup");
+    static_assert(!TAIL || MT == 1, "the in-kernel tail of a K split: one m-tile only");
     extern __shared__ __attribute__((aligned(16))) float red[];
+    __shared__ int s_last;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave & 3, bh = wave >> 2;
@@ -1297,8 +1301,12 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
 #pragma unroll
                     for (int r = 0; r < 4; ++r) acc8[2 * f + 1][r] = xch1[(f * 4 + r) * 64 + lane];
                 }
-                gemv_reduce_store<T, 1, WN, 1, true>(acc8, 0, red, lane, wn, group, split, splits, bias, y, partials, M, N,
-                                                     act);
+                gemv_reduce_store<T, 1, WN, 1, !TAIL>(acc8, 0, red, lane, wn, group, split, splits, bias, y, partials, M,
+                                                      N, act);
+            }
+            if constexpr (TAIL) {   // the last workgroup of the 512 columns to arrive adds the splits
+                if (splits > 1)
+                    gemv_split_tail<T, 1, WN, 2>(red, &s_last, group, splits, bias, y, partials, counters, M, N, act);
             }
             return;
         }
@@ -1536,19 +1544,21 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     return hipGetLastError();
 }
 
-template <typename T, int DEPTH, int MT>
-static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
-                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
-                                   int g, void* workspace, int split_k, hipStream_t stream, int act) {
+template <typename T, int DEPTH, int MT, bool TAIL>
+static hipError_t launch_gemv_wide_form(const void* x, const int32_t* qweight, const void* qscales,
+                                        const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
+                                        int g, void* workspace, int split_k, hipStream_t stream, int act) {
     const int groups = N / 512;
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
     const int splits = (int)cdiv(total_chunks, cps);
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes)
                                 : nullptr;
+    int* counters = reinterpret_cast<int*>(workspace);
     constexpr size_t lds = (size_t)DEPTH * wide_buf_bytes(MT);
     static_assert(lds <= 160 * 1024 - 1024, "staging buffers exceed the LDS");
-    auto kern = gemv_wide_kernel<T, DEPTH, MT>;
+    static_assert(!TAIL || lds >= 512 * 128, "the tail stages 128 bytes per thread");
+    auto kern = gemv_wide_kernel<T, DEPTH, MT, TAIL>;
     static bool raised = false;  // once per process and instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1560,13 +1570,32 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
     hipLaunchKernelGGL(kern, dim3(groups, splits), dim3(512), lds, stream,
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
-                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials,
+                       reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
                        M, N, K, g / 128, cps, splits, act);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || splits == 1) return e;
+    if (e != hipSuccess || splits == 1 || TAIL) return e;
     hipLaunchKernelGGL(gemv_wide_reduce_kernel<T>, dim3((unsigned)cdiv((int64_t)M * (N / 8), 256)), dim3(256), 0, stream, partials,
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, splits, act);
     return hipGetLastError();
+}
+
+// Up to kWideTailRows rows the K splits of the one-m-tile form are added by the last workgroup of the 512 columns to
+// arrive, above (and with more m-tiles) by a second kernel: that one workgroup's serial tail grows with rows x splits
+// (5120 x 25600 in five splits: 19.6 us against 20.4 at one row, 20.9 / 21.3 at four, 22.0 / 21.3 at eight,
+// 25.3 / 22.1 at sixteen).
+constexpr int kWideTailRows = 4;
+
+template <typename T, int DEPTH, int MT>
+static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
+                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
+                                   int g, void* workspace, int split_k, hipStream_t stream, int act) {
+    if constexpr (MT == 1) {
+        if (M <= kWideTailRows)
+            return launch_gemv_wide_form<T, DEPTH, MT, true>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace,
+                                                             split_k, stream, act);
+    }
+    return launch_gemv_wide_form<T, DEPTH, MT, false>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace,
+                                                      split_k, stream, act);
 }
 
 // Upper bound that does not depend on the group size: the kernel never uses
@@ -1613,6 +1642,26 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int v = kDma1x4;
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
+        // Split count of the shared-chunk kernel with the in-kernel tail (M <= 4), 0 = the one-tile kernel runs.  A CU
+        // streams at a fixed rate, so the launch lasts rounds x chunks per split (workgroups come in rounds of one per
+        // CU), plus a tail per row and split (0.06 of a chunk's time).  Taken at one or two rows; at three and four
+        // only where five splits or fewer do and N >= 28672 (5120 x 51200 at four rows 36.0 -> 34.7 us, 8192 x 28672
+        // 34.4 -> 32.7; but 5120 x 25600 20.6 -> 20.9, 5120 x 34816 in ten splits 27.3 -> 29.9).
+        int64_t wide1_tail_splits = 0;
+        if (allow_shared_chunk && M <= kWideTailRows && N % 512 == 0 && N >= 24576 && K * N >= 96000000ll && chunks >= 8) {
+            double best = 1e30;
+            const int64_t hi = chunks / 4 < 10 ? chunks / 4 : 10;
+            for (int64_t c = 2; c <= hi; ++c) {
+                const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
+                if (splits != c) continue;
+                const double cost = (double)(cdiv(N / 512 * splits, 256) * cps) + 0.06 * (double)(M * splits);
+                if (cost < best - 1e-9) {
+                    best = cost;
+                    wide1_tail_splits = c;
+                }
+            }
+            if (M > 2 && (wide1_tail_splits > 5 || N < 28672)) wide1_tail_splits = 0;
+        }
         if (allow_shared_chunk && M > 16 && M <= 64 && N % 512 == 0 && N >= 5120 &&
             K * N >= (M > 48 ? (50ll << 20) : (M > 32 ? 64000000ll : 95000000ll))) {
             // 17..64 rows on the largest weights (from sweeps: the fused gate|up of Qwen3-8B and the MLP of
@@ -1622,6 +1671,13 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             v = M > 32 ? kWideM4 : kWideM2;
             s = 256 / (N / 512);
             if (s > chunks / 4) s = chunks / 4;
+        } else if (wide1_tail_splits > 0) {
+            // up to four rows on the same weights: the shared-chunk kernel again (its row pieces are 256 bytes where
+            // the one-tile kernel's are 64, and a bare read of 64-byte pieces streams 10 % slower), the K splits
+            // added by the last workgroup to arrive.  One row: 5120 x 25600 19.9 -> 19.6 us, 4096 x 24576 18.1 ->
+            // 17.1, 5120 x 51200 35.5 -> 33.3, 8192 x 28672 33.4 -> 31.6, 4096 x 28672 20.2 -> 18.4.
+            v = kWideM1;
+            s = wide1_tail_splits;
         } else if (allow_shared_chunk && M >= 5 && M <= 16 && N % 512 == 0 && N >= 24576 && K * N >= 96000000ll) {
             // 5..16 rows on the widest weights (gate|up of Qwen3-8B and larger): the shared-chunk kernel with one
             // m-tile -- the staged kernel's waves bring their own x, 4 KiB per chunk beside 8 KiB of weights at 16

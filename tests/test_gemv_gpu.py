@@ -153,18 +153,20 @@ def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("M", [5, 9, 16])
-def test_gemv_shared_chunk_one_m_tile(dtype, M):
-    """5..16 rows on the widest weights (N >= 24576): the default dispatch takes the shared-chunk kernel with one m-tile
-    (the odd byte halves hand their fragments to their partners, a second pass adds the K splits); with and without a
-    bias, against the oracle, and forced with other split counts (same oracle)."""
+@pytest.mark.parametrize("M,K,N,splits", [(1, 4096, 24576, 5), (2, 4096, 24576, 5), (5, 4096, 24576, 5),
+                                          (9, 4096, 24576, 5), (16, 4096, 24576, 5), (3, 4096, 28672, 4),
+                                          (4, 4096, 28672, 4)])
+def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
+    """Up to 16 rows on the widest weights (N >= 24576): the default dispatch takes the shared-chunk kernel with one
+    m-tile (the odd byte halves hand their fragments to their partners; the K splits are added by the last workgroup
+    to arrive at up to four rows, by a second pass above); with and without a bias, against the oracle, and forced
+    with other split counts (same oracle)."""
     import ctypes
-    K, N = 4096, 24576
     L = _lib.lib()
     names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
     v, sp = ctypes.c_int(), ctypes.c_int()
     assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
-    assert names[v.value] == "wided2m1" and sp.value == 5, (names[v.value], sp.value)
+    assert names[v.value] == "wided2m1" and sp.value == splits, (names[v.value], sp.value)
     print(f"gemv shared-chunk, one m-tile {dtype} M={M} K={K} N={N}", flush=True)
     p = random_packed(K, N, 128, dtype, seed=K + N + M)
     xb = make_x(M, K, dtype, seed=M)
@@ -287,18 +289,19 @@ def test_gemv_row_blocks_up_to_128_rows(dt):
 
 
 def test_gemv_splitk_exchange_endurance():
-    """About 500 launches cycling three split-K problems (1, 16 and 32 rows) back to back on one stream, sharing one
-    workspace: the cross-workgroup exchange of partials (write-through stores, arrival counter, last arriver adds in
-    split order, counter left at zero) must give the bits of the first launch every time.  Stops at the first
-    mismatch."""
+    """About 670 launches cycling four split-K problems (1, 16 and 32 rows on the one-tile kernels, 2 rows on the
+    shared-chunk kernel's in-kernel tail) back to back on one stream, sharing one workspace: the cross-workgroup
+    exchange of partials (write-through stores, arrival counter, last arriver adds in split order, counter left at
+    zero) must give the bits of the first launch every time.  Stops at the first mismatch."""
     import ctypes
     L = _lib.lib()
     names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
     cases = []
-    for (M, K, N, dtype) in ((1, 2048, 1024, "f16"), (16, 4096, 4096, "bf16"), (32, 3072, 1024, "f16")):
+    for (M, K, N, dtype) in ((1, 2048, 1024, "f16"), (16, 4096, 4096, "bf16"), (32, 3072, 1024, "f16"),
+                             (2, 4096, 24576, "bf16")):
         v, sp = ctypes.c_int(), ctypes.c_int()
         assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
-        assert sp.value > 1 and not names[v.value].startswith("wide"), (M, K, N, names[v.value], sp.value)
+        assert sp.value > 1 and (names[v.value] == "wided2m1") == (N == 24576), (M, K, N, names[v.value], sp.value)
         gen = torch.Generator(device="cuda").manual_seed(M + K)
         tdt = torch.float16 if dtype == "f16" else torch.bfloat16
         qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)
@@ -318,11 +321,11 @@ def test_gemv_splitk_exchange_endurance():
     for c in cases:
         launch(c)
         first.append(c[-1].clone())
-    print("gemv split-K endurance: 168 rounds of 3 launches", flush=True)
+    print("gemv split-K endurance: 168 rounds of 4 launches", flush=True)
     for rnd in range(168):
         for c in cases:
             c[-1].fill_(float("nan"))
-        for c in cases:      # three launches back to back: the second starts while the first's tail may still run
+        for c in cases:      # launches back to back: the second starts while the first's tail may still run
             launch(c)
         for i, c in enumerate(cases):
             assert torch.equal(c[-1], first[i]), f"round {rnd}: launch {i} (M={c[0]} K={c[1]} N={c[2]}) changed bits"
