@@ -1401,8 +1401,10 @@ static const GemvVariant kGemvVariants[] = {
     {"wided2m4", 1, 8, false, 4, 2, 4, true},
     {"wided2m2", 1, 8, false, 4, 2, 2, true},
     {"wided2m1", 1, 8, false, 4, 2, 1, true},
+    // the same with the K splits added by the last workgroup to arrive instead of a second kernel: ...t
+    {"wided2m1t", 1, 8, false, 4, 2, 1, true},
 };
-enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6 };
+enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6, kWideM1T = 7 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = kDma1x4;
 
@@ -1544,10 +1546,15 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
     return hipGetLastError();
 }
 
-template <typename T, int DEPTH, int MT, bool TAIL>
-static hipError_t launch_gemv_wide_form(const void* x, const int32_t* qweight, const void* qscales,
-                                        const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
-                                        int g, void* workspace, int split_k, hipStream_t stream, int act) {
+// The one-m-tile form comes with either way of adding its K splits (variants wided2m1 / wided2m1t): the last
+// workgroup's serial tail grows with rows x splits -- 5120 x 25600 in five splits: 19.6 us with the tail against 20.4
+// with the second pass at one row, 20.9 / 21.3 at four, 22.0 / 21.3 at eight, 25.3 / 22.1 at sixteen.
+constexpr int kWideTailRows = 4;   // the default dispatch takes the tail up to here
+
+template <typename T, int DEPTH, int MT, bool TAIL = false>
+static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
+                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
+                                   int g, void* workspace, int split_k, hipStream_t stream, int act) {
     const int groups = N / 512;
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
@@ -1577,25 +1584,6 @@ static hipError_t launch_gemv_wide_form(const void* x, const int32_t* qweight, c
     hipLaunchKernelGGL(gemv_wide_reduce_kernel<T>, dim3((unsigned)cdiv((int64_t)M * (N / 8), 256)), dim3(256), 0, stream, partials,
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, splits, act);
     return hipGetLastError();
-}
-
-// Up to kWideTailRows rows the K splits of the one-m-tile form are added by the last workgroup of the 512 columns to
-// arrive, above (and with more m-tiles) by a second kernel: that one workgroup's serial tail grows with rows x splits
-// (5120 x 25600 in five splits: 19.6 us against 20.4 at one row, 20.9 / 21.3 at four, 22.0 / 21.3 at eight,
-// 25.3 / 22.1 at sixteen).
-constexpr int kWideTailRows = 4;
-
-template <typename T, int DEPTH, int MT>
-static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
-                                   const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
-                                   int g, void* workspace, int split_k, hipStream_t stream, int act) {
-    if constexpr (MT == 1) {
-        if (M <= kWideTailRows)
-            return launch_gemv_wide_form<T, DEPTH, MT, true>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace,
-                                                             split_k, stream, act);
-    }
-    return launch_gemv_wide_form<T, DEPTH, MT, false>(x, qweight, qscales, qzeros, bias, y, M, N, K, g, workspace,
-                                                      split_k, stream, act);
 }
 
 // Upper bound that does not depend on the group size: the kernel never uses
@@ -1676,7 +1664,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             // the one-tile kernel's are 64, and a bare read of 64-byte pieces streams 10 % slower), the K splits
             // added by the last workgroup to arrive.  One row: 5120 x 25600 19.9 -> 19.6 us, 4096 x 24576 18.1 ->
             // 17.1, 5120 x 51200 35.5 -> 33.3, 8192 x 28672 33.4 -> 31.6, 4096 x 28672 20.2 -> 18.4.
-            v = kWideM1;
+            v = kWideM1T;
             s = wide1_tail_splits;
         } else if (allow_shared_chunk && M >= 5 && M <= 16 && N % 512 == 0 && N >= 24576 && K * N >= 96000000ll) {
             // 5..16 rows on the widest weights (gate|up of Qwen3-8B and larger): the shared-chunk kernel with one
@@ -1844,6 +1832,10 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         case kWideM1:
             e = f16 ? launch_gemv_wide<F16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
                     : launch_gemv_wide<BF16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            break;
+        case kWideM1T:
+            e = f16 ? launch_gemv_wide<F16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
+                    : launch_gemv_wide<BF16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
             break;
         case kWideM2:
             e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)

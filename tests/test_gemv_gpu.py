@@ -166,7 +166,7 @@ def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
     names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
     v, sp = ctypes.c_int(), ctypes.c_int()
     assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
-    assert names[v.value] == "wided2m1" and sp.value == splits, (names[v.value], sp.value)
+    assert names[v.value] == ("wided2m1t" if M <= 4 else "wided2m1") and sp.value == splits, (names[v.value], sp.value)
     print(f"gemv shared-chunk, one m-tile {dtype} M={M} K={K} N={N}", flush=True)
     p = random_packed(K, N, 128, dtype, seed=K + N + M)
     xb = make_x(M, K, dtype, seed=M)
@@ -180,8 +180,9 @@ def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
     assert torch.equal(y, _linear("awq_linear", xd, *dev, bd))
     y0 = nq.awq_gemm(xd, *dev, 8)
     _check(y0, xb, p, dtype)
-    for split in (1, 2, 8):
-        _check(awq_gemv_variant(xd, *dev, v.value, split), xb, p, dtype)
+    for vn in ("wided2m1", "wided2m1t"):      # either way of adding the K splits, at every row count
+        for split in (1, 2, 8):
+            _check(awq_gemv_variant(xd, *dev, names.index(vn), split), xb, p, dtype)
 
 
 def test_gemv_reference_test_shape():
@@ -301,7 +302,7 @@ def test_gemv_splitk_exchange_endurance():
                              (2, 4096, 24576, "bf16")):
         v, sp = ctypes.c_int(), ctypes.c_int()
         assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
-        assert sp.value > 1 and (names[v.value] == "wided2m1") == (N == 24576), (M, K, N, names[v.value], sp.value)
+        assert sp.value > 1 and (names[v.value] == "wided2m1t") == (N == 24576), (M, K, N, names[v.value], sp.value)
         gen = torch.Generator(device="cuda").manual_seed(M + K)
         tdt = torch.float16 if dtype == "f16" else torch.bfloat16
         qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)

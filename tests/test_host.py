@@ -167,7 +167,8 @@ def test_dispatch_plans_are_consistent():
                     assert M <= 16
                 if name.startswith("wide"):
                     assert N % 512 == 0 and K * N >= 50 << 20
-                    assert (name == "wided2m1") == (M <= 16) and (name == "wided2m4") == (M > 32)
+                    assert (name == "wided2m1t") == (M <= 4) and (name == "wided2m1") == (5 <= M <= 16)
+                    assert (name == "wided2m4") == (M > 32)
                     if M >= 5:
                         assert N // 512 * s <= 256 + N // 512        # about one workgroup per CU
                     else:                                            # in-kernel tail: up to two rounds of workgroups
@@ -210,9 +211,9 @@ def test_dispatch_plans_are_consistent():
     # one or two rows there: the shared-chunk kernel with the in-kernel tail, split so that whole rounds of workgroups
     # carry the fewest chunks each (68 groups x 7 splits = 476 workgroups: two rounds of six chunks)
     rc, v, s = _plan(L.awq_gemv_plan, 1, 34816, 5120, 128)
-    assert rc == 0 and gemv_names[v] == "wided2m1" and s == 7
+    assert rc == 0 and gemv_names[v] == "wided2m1t" and s == 7
     rc, v, s = _plan(L.awq_gemv_plan, 4, 51200, 5120, 128)      # 100 groups x 5 splits: two full rounds, also at four rows
-    assert rc == 0 and gemv_names[v] == "wided2m1" and s == 5
+    assert rc == 0 and gemv_names[v] == "wided2m1t" and s == 5
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
     # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
     rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120, 128, _lib.AWQ_BF16)
