@@ -78,8 +78,8 @@ size_t awq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* Decode regime, 1 <= M <= 16 (up to 128 rows where N % 128 == 0 and group_size % 128 == 0: batched
  * decode, as blocks of 16 rows): y = x @ dequant(W) (+ bias), fp32 accumulation, split-K with a
- * fixed-order (run-to-run bit-stable) reduction, inside the kernel or, for 17..64 rows on the largest
- * weights, as a second kernel on the same stream.
+ * fixed-order (run-to-run bit-stable) reduction, inside the kernel or, from 5 rows on the widest and
+ * from 17 rows on the largest weights, as a second kernel on the same stream.
  * Replaces awq_gemm(x, qweight, qscales, qzeros, split_k_iters) for small M:
  * nanoquantization/layers/gemm.py:329-379 (kernel :183-326, torch.zeros :361,
  * out.sum :378). */
