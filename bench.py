@@ -166,10 +166,10 @@ def gemv_kernel_name(M, N, K, dtype_name, g=G):
         return "?"
     name = L.awq_gemv_variant_name(v.value).decode()
     T = "F16" if dtype_name == "f16" else "BF16"
-    if name == "wided2m1t":   # the K splits are added inside the kernel
-        kern = f"awq::gemv_wide_kernel<{T},2,1,true>"
+    if name.startswith("wide") and name.endswith("t"):   # wided<DEPTH>m<MT>t: the K splits are added inside the kernel
+        kern = f"awq::gemv_wide_kernel<{T},{name[5]},{name[7]},true>"
     elif name.startswith("wide"):
-        kern = f"awq::gemv_wide_kernel<{T},2,{name[-1]},false> + awq::gemv_wide_reduce_kernel<{T}>"
+        kern = f"awq::gemv_wide_kernel<{T},{name[5]},{name[7]},false> + awq::gemv_wide_reduce_kernel<{T}>"
     elif name.startswith("dma"):
         kern = f"awq::gemv_dma_kernel<{T},{name[5]},plain>"
     else:

@@ -1204,7 +1204,15 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
 
     // per wave and chunk (an upper bound where a wave brings no x; only a third buffer waits by this count)
     constexpr int kDmaOps = CH + HMT + 1;
-    static_assert(MT >= 2 || DEPTH == 2, "one m-tile: the waves' load counts differ, two buffers only");
+    // one m-tile: waves 4..7 bring no x, one load fewer per chunk
+    const bool full_count = MT >= 2 || wave < 4;   // uniform
+    auto wait_chunks_in_flight = [&](int n) {   // all but the loads of the n newest chunks have landed
+#define AWQ_WIDE_WAIT(K) __builtin_amdgcn_s_waitcnt(0x0F70 | ((K) & 15) | (((K) >> 4) << 14))
+        if (n == 0) AWQ_WIDE_WAIT(0);
+        else if (full_count) AWQ_WIDE_WAIT(kDmaOps);
+        else AWQ_WIDE_WAIT(kDmaOps - 1);
+#undef AWQ_WIDE_WAIT
+    };
     auto issue_dma = [&](int c, int buf) {
         const int row0 = c * 128;
         char* base = stage + buf * buf_bytes;
@@ -1218,12 +1226,16 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256),
                                                  16, 0, 0);
         }
+        // the three-buffer form counts its loads (wait_chunks_in_flight): every block below is issued once per wave,
+        // fenced off from its neighbours so that no branch is threaded through another block's loads
+        __builtin_amdgcn_wave_barrier();
         if (x_wave) {
 #pragma unroll
             for (int i = 0; i < HMT; ++i)
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + x_s[i] * 32) + xsrc[i]),
                                                  AWQ_LPTR(base + x_s[i] * x_step + x_mt[i] * 1024), 16, 0, 0);
         }
+        __builtin_amdgcn_wave_barrier();
         if (zs_lane) {
             const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
             if (bh == 0)
@@ -1255,8 +1267,7 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
         int buf = 0;
         for (int c = c0; c < c1; ++c) {
             const int newer = min(c1 - 1 - c, DEPTH - 2);
-            if (newer == 0) __builtin_amdgcn_s_waitcnt(0x0F70);                                   // vmcnt(0)
-            else __builtin_amdgcn_s_waitcnt(0x0F70 | (kDmaOps & 15) | ((kDmaOps >> 4) << 14));    // vmcnt(kDmaOps)
+            wait_chunks_in_flight(newer);
             asm volatile("" ::: "memory");
             // every wave's share of the chunk is in LDS, and every wave is done reading the buffer of chunk c-1.
             // A bare barrier: __syncthreads() would first wait for every outstanding load, i.e. for the chunks
@@ -1403,8 +1414,12 @@ static const GemvVariant kGemvVariants[] = {
     {"wided2m1", 1, 8, false, 4, 2, 1, true},
     // the same with the K splits added by the last workgroup to arrive instead of a second kernel: ...t
     {"wided2m1t", 1, 8, false, 4, 2, 1, true},
+    // one m-tile with three staging buffers (two chunks in flight): for launches of one workgroup per CU at most
+    {"wided3m1", 1, 8, false, 4, 3, 1, true},
+    {"wided3m1t", 1, 8, false, 4, 3, 1, true},
 };
-enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6, kWideM1T = 7 };
+enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6, kWideM1T = 7,
+       kWideD3M1 = 8, kWideD3M1T = 9 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = kDma1x4;
 
@@ -1733,6 +1748,16 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             }
         }
         if (s < 1) s = 1;
+        if (v == kWideM1 || v == kWideM1T) {
+            // One workgroup per CU at most and enough chunks per split to fill the pipeline: three staging buffers, two
+            // chunks in flight while one is multiplied (5120 x 25600 in five splits 19.5 -> 18.4 us at one row,
+            // 22.0 -> 21.6 at 16; 8192 x 28672 in four 32.9 -> 29.2 / 33.2 -> 32.3; 5120 x 51200 at 16 rows in two
+            // 40.4 -> 36.7).  With more workgroups than CUs two of the two-buffer form share a CU and do better
+            // (5120 x 51200 at one row in five splits: 32.8 against 35.1 us), and on short splits the deeper prologue
+            // does not pay (4096 x 24576, seven chunks per split, at 8 / 16 rows: 18.8 / 19.7 against 19.2 / 20.0).
+            const int64_t cps = cdiv(chunks, s), splits = cdiv(chunks, cps);
+            if (N / 512 * splits <= 256 && cps >= (v == kWideM1T ? 6 : 8)) v = v == kWideM1T ? kWideD3M1T : kWideD3M1;
+        }
         *variant = v;
         *split_k = (int)s;
         return;
@@ -1836,6 +1861,14 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         case kWideM1T:
             e = f16 ? launch_gemv_wide<F16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
                     : launch_gemv_wide<BF16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            break;
+        case kWideD3M1T:
+            e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
+                    : launch_gemv_wide<BF16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            break;
+        case kWideD3M1:
+            e = f16 ? launch_gemv_wide<F16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
+                    : launch_gemv_wide<BF16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
             break;
         case kWideM2:
             e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)

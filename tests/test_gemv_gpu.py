@@ -166,7 +166,7 @@ def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
     names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
     v, sp = ctypes.c_int(), ctypes.c_int()
     assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
-    assert names[v.value] == ("wided2m1t" if M <= 4 else "wided2m1") and sp.value == splits, (names[v.value], sp.value)
+    assert names[v.value].endswith("m1t" if M <= 4 else "m1") and sp.value == splits, (names[v.value], sp.value)
     print(f"gemv shared-chunk, one m-tile {dtype} M={M} K={K} N={N}", flush=True)
     p = random_packed(K, N, 128, dtype, seed=K + N + M)
     xb = make_x(M, K, dtype, seed=M)
@@ -178,11 +178,18 @@ def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
     y = _linear("awq_linear", xd, *dev, bd)
     _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
     assert torch.equal(y, _linear("awq_linear", xd, *dev, bd))
-    y0 = nq.awq_gemm(xd, *dev, 8)
-    _check(y0, xb, p, dtype)
-    for vn in ("wided2m1", "wided2m1t"):      # either way of adding the K splits, at every row count
+    ref = o.linear_fp32(xb, p["qweight"], p["qzeros"], p["qscales"], dtype, None)   # once: 100 M weights on the CPU
+
+    def check_plain(yv, what):
+        err = o.max_rel_err(o.from_bits16(to_bits(yv), dtype), ref)
+        assert err <= TIGHT[dtype], (what, err)
+
+    check_plain(nq.awq_gemm(xd, *dev, 8), "default")
+    for vn in ("wided2m1", "wided2m1t", "wided3m1", "wided3m1t"):   # two or three staging buffers, either way of adding the K splits
         for split in (1, 2, 8):
-            _check(awq_gemv_variant(xd, *dev, names.index(vn), split), xb, p, dtype)
+            yv = awq_gemv_variant(xd, *dev, names.index(vn), split)
+            check_plain(yv, (vn, split))
+            assert torch.equal(yv, awq_gemv_variant(xd, *dev, names.index(vn), split)), (vn, split)
 
 
 def test_gemv_reference_test_shape():
@@ -302,7 +309,7 @@ def test_gemv_splitk_exchange_endurance():
                              (2, 4096, 24576, "bf16")):
         v, sp = ctypes.c_int(), ctypes.c_int()
         assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
-        assert sp.value > 1 and (names[v.value] == "wided2m1t") == (N == 24576), (M, K, N, names[v.value], sp.value)
+        assert sp.value > 1 and names[v.value].endswith("m1t") == (N == 24576), (M, K, N, names[v.value], sp.value)
         gen = torch.Generator(device="cuda").manual_seed(M + K)
         tdt = torch.float16 if dtype == "f16" else torch.bfloat16
         qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda", generator=gen)

@@ -167,8 +167,11 @@ def test_dispatch_plans_are_consistent():
                     assert M <= 16
                 if name.startswith("wide"):
                     assert N % 512 == 0 and K * N >= 50 << 20
-                    assert (name == "wided2m1t") == (M <= 4) and (name == "wided2m1") == (5 <= M <= 16)
+                    assert name.endswith("m1t") == (M <= 4) and name.endswith("m1") == (5 <= M <= 16)
                     assert (name == "wided2m4") == (M > 32)
+                    if name[5] == "3":      # three staging buffers: one workgroup per CU at most
+                        cps = -(-chunks // s)
+                        assert N // 512 * -(-chunks // cps) <= 256 and cps >= 6
                     if M >= 5:
                         assert N // 512 * s <= 256 + N // 512        # about one workgroup per CU
                     else:                                            # in-kernel tail: up to two rounds of workgroups
@@ -204,8 +207,8 @@ def test_dispatch_plans_are_consistent():
     wgs = 34816 // 128 * s
     assert wgs / (256 * -(-wgs // 256)) >= 0.8
     # 5..16 rows on the widest weights: the shared-chunk kernel with one m-tile, about one workgroup per CU
-    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 5120, 128)
-    assert rc == 0 and gemv_names[v] == "wided2m1" and s == 3
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 5120, 128)      # 68 groups x 3 splits of 14 chunks: three buffers
+    assert rc == 0 and gemv_names[v] == "wided3m1" and s == 3
     rc, v, s = _plan(L.awq_gemv_plan, 4, 34816, 5120, 128)      # three or four rows: the one-tile kernel, two chunks per wave
     assert rc == 0 and gemv_names[v] == "dma1x4" and s == 5
     # one or two rows there: the shared-chunk kernel with the in-kernel tail, split so that whole rounds of workgroups
@@ -214,6 +217,8 @@ def test_dispatch_plans_are_consistent():
     assert rc == 0 and gemv_names[v] == "wided2m1t" and s == 7
     rc, v, s = _plan(L.awq_gemv_plan, 4, 51200, 5120, 128)      # 100 groups x 5 splits: two full rounds, also at four rows
     assert rc == 0 and gemv_names[v] == "wided2m1t" and s == 5
+    rc, v, s = _plan(L.awq_gemv_plan, 1, 25600, 5120, 128)      # 50 groups x 5 splits = 250 workgroups: three buffers
+    assert rc == 0 and gemv_names[v] == "wided3m1t" and s == 5
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
     # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
     rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120, 128, _lib.AWQ_BF16)
