@@ -1645,19 +1645,24 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int v = kDma1x4;
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
-        // Split count of the shared-chunk kernel with the in-kernel tail (M <= 4), 0 = the one-tile kernel runs.  A CU
+        // Split count of the shared-chunk kernel with the in-kernel tail (M <= 4; N >= 8192 and 80 M weights or more:
+        // 5120 x 20480 at one row 20.3 -> 16.9 us, 8192 x 14336 20.2 -> 18.5, 8192 x 10240 17.6 -> 15.8, 12288 x 8192
+        // 19.5 -> 17.9, 5120 x 17408 15.8 -> 15.4; 4096 x 14336 and smaller lose), 0 = the one-tile kernel runs.  A CU
         // streams at a fixed rate, so the launch lasts rounds x chunks per split (workgroups come in rounds of one per
         // CU), plus a tail per row and split (0.06 of a chunk's time).  Taken at one or two rows; at three and four
         // only where five splits or fewer do and N >= 28672 (5120 x 51200 at four rows 36.0 -> 34.7 us, 8192 x 28672
         // 34.4 -> 32.7; but 5120 x 25600 20.6 -> 20.9, 5120 x 34816 in ten splits 27.3 -> 29.9).
         int64_t wide1_tail_splits = 0;
-        if (allow_shared_chunk && M <= kWideTailRows && N % 512 == 0 && N >= 24576 && K * N >= 96000000ll && chunks >= 8) {
+        if (allow_shared_chunk && M <= kWideTailRows && N % 512 == 0 && N >= 8192 && K * N >= 80000000ll && chunks >= 8) {
             double best = 1e30;
-            const int64_t hi = chunks / 4 < 10 ? chunks / 4 : 10;
+            const int64_t hi = chunks / 4 < 16 ? chunks / 4 : 16;
             for (int64_t c = 2; c <= hi; ++c) {
                 const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
                 if (splits != c) continue;
-                const double cost = (double)(cdiv(N / 512 * splits, 256) * cps) + 0.06 * (double)(M * splits);
+                const int64_t wgs = N / 512 * splits;
+                // (one workgroup per CU at most runs the three-buffer form, 5 % faster: see the choice of depth below)
+                const double cost = ((double)(cdiv(wgs, 256) * cps) + 0.06 * (double)(M * splits)) *
+                                    (wgs <= 256 && cps >= 6 ? 0.95 : 1.0);
                 if (cost < best - 1e-9) {
                     best = cost;
                     wide1_tail_splits = c;
@@ -1681,12 +1686,14 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             // 17.1, 5120 x 51200 35.5 -> 33.3, 8192 x 28672 33.4 -> 31.6, 4096 x 28672 20.2 -> 18.4.
             v = kWideM1T;
             s = wide1_tail_splits;
-        } else if (allow_shared_chunk && M >= 5 && M <= 16 && N % 512 == 0 && N >= 24576 && K * N >= 96000000ll) {
-            // 5..16 rows on the widest weights (gate|up of Qwen3-8B and larger): the shared-chunk kernel with one
-            // m-tile -- the staged kernel's waves bring their own x, 4 KiB per chunk beside 8 KiB of weights at 16
-            // rows; shared by eight waves it is 0.5 KiB per wave.  5120 x 25600 at 8 / 16 rows 22.7 / 25.0 -> 21.3 /
-            // 21.9 us, 5120 x 51200 40.2 / 46.2 -> 36.6 / 39.5, 4096 x 24576 20.0 / 22.0 -> 18.8 / 19.5; below
-            // these widths (25600 x 5120, 5120 x 10240) its K splits' partial round trip costs more than it saves.
+        } else if (allow_shared_chunk && M >= 5 && M <= 16 && N % 512 == 0 && N >= 10240 && K * N >= 80000000ll) {
+            // 5..16 rows on wide, large weights (the MLP gate|up of Qwen3-8B and larger, fused or not): the shared-chunk
+            // kernel with one m-tile -- the staged kernel's waves bring their own x, 4 KiB per chunk beside 8 KiB of
+            // weights at 16 rows; shared by eight waves it is 0.5 KiB per wave.  5120 x 25600 at 8 / 16 rows 22.7 /
+            // 25.0 -> 21.3 / 21.9 us, 5120 x 51200 40.2 / 46.2 -> 36.6 / 39.5, 4096 x 24576 20.0 / 22.0 -> 18.8 / 19.5,
+            // 5120 x 20480 21.8 / 23.1 -> 19.4 / 20.3, 8192 x 14336 24.2 / 25.7 -> 21.4 / 22.1, 8192 x 10240 20.1 /
+            // 21.1 -> 19.2 / 19.7; on narrower or smaller weights (12288 x 8192: 19.9 / 21.5 -> 21.1 / 22.3, 4096 x
+            // 12288, 5120 x 10240, 25600 x 5120) its K splits' partial round trip costs more than it saves.
             v = kWideM1;
             s = 256 / (N / 512);
             if (s < 2) s = 2;

@@ -155,9 +155,9 @@ def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N):
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("M,K,N,splits", [(1, 4096, 24576, 5), (2, 4096, 24576, 5), (5, 4096, 24576, 5),
                                           (9, 4096, 24576, 5), (16, 4096, 24576, 5), (3, 4096, 28672, 4),
-                                          (4, 4096, 28672, 4)])
+                                          (4, 4096, 28672, 4), (1, 12288, 8192, 16), (16, 5120, 20480, 6)])
 def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
-    """Up to 16 rows on the widest weights (N >= 24576): the default dispatch takes the shared-chunk kernel with one
+    """Up to 16 rows on wide, large weights (80 M and more): the default dispatch takes the shared-chunk kernel with one
     m-tile (the odd byte halves hand their fragments to their partners; the K splits are added by the last workgroup
     to arrive at up to four rows, by a second pass above); with and without a bias, against the oracle, and forced
     with other split counts (same oracle)."""

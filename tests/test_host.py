@@ -147,7 +147,8 @@ def test_dispatch_plans_are_consistent():
     gemv_names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
     gemm_names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
     shapes = [(1024, 2048), (1024, 1024), (2048, 1024), (1024, 3072), (3072, 1024), (4096, 12288), (12288, 4096),
-              (5120, 25600), (25600, 5120), (5120, 10240), (8192, 5120), (5120, 34816), (4096, 24576), (128, 128),
+              (5120, 25600), (25600, 5120), (5120, 10240), (8192, 5120), (5120, 34816), (4096, 24576), (5120, 20480),
+              (8192, 14336), (12288, 8192), (128, 128),
               (256, 8), (1024, 1032), (3072, 136)]
     for K, N in shapes:
         for M in (1, 2, 4, 5, 8, 16, 17, 32, 33, 48, 64):
@@ -175,7 +176,7 @@ def test_dispatch_plans_are_consistent():
                     if M >= 5:
                         assert N // 512 * s <= 256 + N // 512        # about one workgroup per CU
                     else:                                            # in-kernel tail: up to two rounds of workgroups
-                        assert N >= 24576 and s <= 10 and (M <= 2 or (s <= 5 and N >= 28672))
+                        assert N >= 8192 and K * N >= 80000000 and s <= 16 and (M <= 2 or (s <= 5 and N >= 28672))
                 if not staged_ok:
                     assert not name.startswith(("dma", "wide"))
                 if g == 128:   # awq_gemv_workspace_bytes takes no group size: it must cover this plan
@@ -219,6 +220,14 @@ def test_dispatch_plans_are_consistent():
     assert rc == 0 and gemv_names[v] == "wided2m1t" and s == 5
     rc, v, s = _plan(L.awq_gemv_plan, 1, 25600, 5120, 128)      # 50 groups x 5 splits = 250 workgroups: three buffers
     assert rc == 0 and gemv_names[v] == "wided3m1t" and s == 5
+    # wide mid-size weights (80 M and more) take it too: 16 groups x 16 splits at one row, 40 groups x 6 at 16 rows;
+    # 12288 x 8192 at 16 rows and anything smaller stay with the one-tile kernel
+    rc, v, s = _plan(L.awq_gemv_plan, 1, 8192, 12288, 128)
+    assert rc == 0 and gemv_names[v] == "wided3m1t" and s == 16
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 20480, 5120, 128)
+    assert rc == 0 and gemv_names[v] == "wided2m1" and s == 6
+    assert gemv_names[_plan(L.awq_gemv_plan, 16, 8192, 12288, 128)[1]] == "dma1x4"
+    assert gemv_names[_plan(L.awq_gemv_plan, 1, 14336, 4096, 128)[1]] == "dma1x4"
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
     # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
     rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120, 128, _lib.AWQ_BF16)
