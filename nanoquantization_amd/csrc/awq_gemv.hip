@@ -1149,16 +1149,17 @@ __global__ __launch_bounds__(64 * WK) void gemv_dma_kernel(
 // At the end the two halves exchange fragments through LDS so that each stores whole words of half the rows.
 // A K split leaves fp32 partials that a second kernel adds in split order -- or, TAIL (one m-tile, a few rows), the
 // last workgroup of the 512 columns to arrive, as in the one-tile kernel.
-__host__ __device__ constexpr int wide_buf_bytes(int MT) { return 4096 * MT + 4 * 8704; }
+__host__ __device__ constexpr int wide_buf_bytes(int MT, int WN = 4) { return 4096 * MT + WN * 8704; }
 
-template <typename T, int DEPTH, int MT, bool TAIL = false>
-__global__ __launch_bounds__(512) void gemv_wide_kernel(
+template <typename T, int DEPTH, int MT, bool TAIL = false, int WN = 4>
+__global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ qweight,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split, int splits, int act) {
     // HMT: pieces of x a wave brings per chunk (with one m-tile the four pieces go to waves 0..3, one each)
-    constexpr int CH = 4, WN = 4, HMT = MT >= 2 ? MT / 2 : 1;
+    constexpr int CH = 4, HMT = MT >= 2 ? MT / 2 : 1;
+    static_assert(WN == 4 || (WN == 2 && MT == 1), "512 columns, or 256 with one m-tile");
     static_assert(DEPTH >= 2 && DEPTH <= 3, "two or three staging buffers");
     static_assert(MT == 1 || MT == 2 || MT == 4, "m-tiles per workgroup");
     static_assert(!TAIL || MT == 1, "the in-kernel tail of a K split: one m-tile only");
@@ -1166,7 +1167,7 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
     __shared__ int s_last;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wn = wave & 3, bh = wave >> 2;
+    const int wn = wave % WN, bh = wave / WN;
     const int j = lane & 15, kb = lane >> 4;
     const int words = N >> 3;
     const int group = blockIdx.x, split = blockIdx.y;
@@ -1176,7 +1177,7 @@ __global__ __launch_bounds__(512) void gemv_wide_kernel(
     const int c0 = split * chunks_per_split;
     const int c1 = min(c0 + chunks_per_split, total_chunks);
 
-    constexpr int buf_bytes = wide_buf_bytes(MT);
+    constexpr int buf_bytes = wide_buf_bytes(MT, WN);
     constexpr int x_step = 1024 * MT;
     char* stage = reinterpret_cast<char*>(red);
     const int w_off = 4096 * MT + wn * 8704, zs_off = w_off + 8192;
@@ -1417,9 +1418,14 @@ static const GemvVariant kGemvVariants[] = {
     // one m-tile with three staging buffers (two chunks in flight): for launches of one workgroup per CU at most
     {"wided3m1", 1, 8, false, 4, 3, 1, true},
     {"wided3m1t", 1, 8, false, 4, 3, 1, true},
+    // the one-m-tile forms on 256 columns per workgroup (four waves: 2 column tiles x 2 byte halves): wide2d...
+    {"wide2d2m1", 1, 4, false, 2, 2, 1, true},
+    {"wide2d2m1t", 1, 4, false, 2, 2, 1, true},
+    {"wide2d3m1", 1, 4, false, 2, 3, 1, true},
+    {"wide2d3m1t", 1, 4, false, 2, 3, 1, true},
 };
 enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6, kWideM1T = 7,
-       kWideD3M1 = 8, kWideD3M1T = 9 };
+       kWideD3M1 = 8, kWideD3M1T = 9, kWide2D2M1 = 10, kWide2D2M1T = 11, kWide2D3M1 = 12, kWide2D3M1T = 13 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = kDma1x4;
 
@@ -1566,21 +1572,21 @@ static hipError_t launch_gemv_dma(const void* x, const int32_t* qweight, const v
 // with the second pass at one row, 20.9 / 21.3 at four, 22.0 / 21.3 at eight, 25.3 / 22.1 at sixteen.
 constexpr int kWideTailRows = 4;   // the default dispatch takes the tail up to here
 
-template <typename T, int DEPTH, int MT, bool TAIL = false>
+template <typename T, int DEPTH, int MT, bool TAIL = false, int WN = 4>
 static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
                                    const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                                    int g, void* workspace, int split_k, hipStream_t stream, int act) {
-    const int groups = N / 512;
+    const int groups = N / (128 * WN);
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
     const int splits = (int)cdiv(total_chunks, cps);
     float* partials = workspace ? reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + kCounterBytes)
                                 : nullptr;
     int* counters = reinterpret_cast<int*>(workspace);
-    constexpr size_t lds = (size_t)DEPTH * wide_buf_bytes(MT);
+    constexpr size_t lds = (size_t)DEPTH * wide_buf_bytes(MT, WN);
     static_assert(lds <= 160 * 1024 - 1024, "staging buffers exceed the LDS");
-    static_assert(!TAIL || lds >= 512 * 128, "the tail stages 128 bytes per thread");
-    auto kern = gemv_wide_kernel<T, DEPTH, MT, TAIL>;
+    static_assert(!TAIL || lds >= 128 * WN * 128, "the tail stages 128 bytes per thread");
+    auto kern = gemv_wide_kernel<T, DEPTH, MT, TAIL, WN>;
     static bool raised = false;  // once per process and instantiation
     if (!raised) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1589,7 +1595,7 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
         raised = true;
     }
     (void)hipGetLastError();
-    hipLaunchKernelGGL(kern, dim3(groups, splits), dim3(512), lds, stream,
+    hipLaunchKernelGGL(kern, dim3(groups, splits), dim3(128 * WN), lds, stream,
                        reinterpret_cast<const uint16_t*>(x), reinterpret_cast<const uint32_t*>(qweight),
                        reinterpret_cast<const uint16_t*>(qscales), reinterpret_cast<const uint32_t*>(qzeros),
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), partials, counters,
@@ -1634,6 +1640,93 @@ static int64_t balance_splits(int64_t chunks, int64_t s, int64_t wk, int64_t cap
     return best;
 }
 
+// The one-m-tile forms of the shared-chunk kernel for up to 16 rows on large weights: which one, and its K split
+// (0 = the one-tile staged kernel runs).  The one-tile kernel's waves each bring their own x (4 KiB per chunk beside
+// 8 KiB of weights at 16 rows) and fetch 64-byte row pieces; in a shared-chunk workgroup x is staged once and the row
+// pieces are 128 or 256 bytes wide.  From sweeps of every form x split on 17 weights of 50..260 M elements:
+//  * N >= 28672 (the fused gate|up of Qwen3-14B/32B, 8192 x 28672): 512 columns per workgroup.  Few splits fill the
+//    chip there, and every split costs a tail (per row) or partial traffic.  Up to four rows with the in-kernel tail,
+//    the split count from a cost in chunk times -- rounds of 256 workgroups x chunks per split + 0.06 per row and
+//    split, 5 % off where one workgroup per CU lets the three-buffer form run -- (5120 x 51200 at one row 35.5 -> 32.2
+//    us in five splits, 8192 x 28672 33.4 -> 28.6 in four, 5120 x 34816 26.0 -> 24.4 in seven); at three and four rows
+//    only where five splits or fewer do (5120 x 34816 in ten: 27.3 -> 29.9).  5..16 rows: second pass, about one
+//    workgroup per CU (5120 x 51200 at 16 rows 46.2 -> 36.6 us, 5120 x 34816 34.7 -> 28.3, 8192 x 28672 -> 32.2).
+//  * 8192 <= N < 28672 and 64 Mi weights or more (56 M from five rows on: 6144 x 10240 at 8 rows 16.5 -> 14.4 us,
+//    4096 x 14336 15.9 -> 14.1, while at up to four rows both lose 0.5 us): 256 columns per workgroup (four waves).  Plan A: two buffers,
+//    about 500 workgroups (two or three share a CU); plan B: about one workgroup per CU (at least 85 % of them),
+//    three buffers if a split has six chunks or more.  Up to eight rows with the tail while rows x splits <= 64 -- A,
+//    or B where A needs eleven splits or more -- (one row: 5120 x 25600 19.9 -> 17.6 us, 5120 x 17408 15.8 -> 14.1,
+//    12288 x 8192 19.5 -> 16.0, 8192 x 8192 15.5 -> 12.9, 4096 x 22016 19.3 -> 15.4, 3584 x 18944 15.4 -> 12.8; four
+//    rows: 8192 x 10240 18.2 -> 16.4, 12288 x 8192 20.3 -> 18.1, 5120 x 25600 20.6 -> 18.3; eight: 22.7 -> 19.1),
+//    beyond that B with the second pass (12288 x 8192 at 16 rows 21.6 -> 18.9 us, 8192 x 8192 17.2 -> 15.8,
+//    8192 x 10240 19.7 -> 18.3, 6144 x 16384 21.8 -> 18.6), else the 512-column form if that fills the CUs
+//    (4096 x 24576: 19.4), else A (5120 x 25600 21.2 -> 20.7, 5120 x 17408 18.4 -> 17.7).  Smaller weights (4096 x
+//    12288, 12288 x 4096, 8192 x 5120, 5120 x 12288) and narrower ones (16384 x 4096, 25600 x 5120, 8192 x 7168:
+//    28..56 column tiles) lose up to 2 us to the one-tile kernel.
+static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, int* variant) {
+    if (chunks < 8) return 0;
+    auto normalised = [&](int64_t c) { return cdiv(chunks, cdiv(chunks, c)); };   // the split count a launch ends up with
+    // 512 columns per workgroup, second pass: about one workgroup per CU
+    auto wide512_pass = [&]() -> int64_t {
+        int64_t c = 256 / (N / 512);
+        if (c < 2) c = 2;
+        if (c > chunks / 4) c = chunks / 4;
+        const int64_t cps = cdiv(chunks, c);
+        *variant = (N / 512 * normalised(c) <= 256 && cps >= 8) ? kWideD3M1 : kWideM1;
+        return c;
+    };
+    if (N >= 28672) {
+        if (N % 512 != 0 || K * N < 80000000ll) return 0;
+        if (M > kWideTailRows) return wide512_pass();
+        double best = 1e30;
+        int64_t best_c = 0;
+        bool best_d3 = false;
+        const int64_t hi = chunks / 4 < 16 ? chunks / 4 : 16;
+        for (int64_t c = 2; c <= hi; ++c) {
+            const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
+            if (splits != c) continue;
+            const int64_t wgs = N / 512 * splits;
+            const bool d3 = wgs <= 256 && cps >= 6;
+            const double cost = ((double)(cdiv(wgs, 256) * cps) + 0.06 * (double)(M * splits)) * (d3 ? 0.95 : 1.0);
+            if (cost < best - 1e-9) {
+                best = cost;
+                best_c = c;
+                best_d3 = d3;
+            }
+        }
+        if (best_c == 0 || (M > 2 && best_c > 5)) return 0;
+        *variant = best_d3 ? kWideD3M1T : kWideM1T;
+        return best_c;
+    }
+    if (N % 256 != 0 || N < 8192 || K * N < (M <= 4 ? (64ll << 20) : 56000000ll)) return 0;
+    const int64_t groups = N / 256;
+    int64_t sa = 512 / groups;
+    if (sa > 25) sa = 25;
+    if (sa > chunks / 4) sa = chunks / 4;
+    if (sa < 2) return 0;
+    sa = normalised(sa);
+    int64_t sb = 256 / groups;
+    if (sb > chunks / 4) sb = chunks / 4;
+    const bool b_valid = sb >= 2 && normalised(sb) * groups >= 218;
+    if (b_valid) sb = normalised(sb);
+    const bool b_d3 = b_valid && cdiv(chunks, sb) >= 6;
+    if (M <= 8) {
+        const bool use_b = b_valid && sa >= 11;
+        const int64_t c = use_b ? sb : sa;
+        if (M * c <= 64) {
+            *variant = use_b ? (b_d3 ? kWide2D3M1T : kWide2D2M1T) : kWide2D2M1T;
+            return c;
+        }
+    }
+    if (b_valid) {
+        *variant = b_d3 ? kWide2D3M1 : kWide2D2M1;
+        return sb;
+    }
+    if (N % 512 == 0 && (256 / (N / 512)) * (N / 512) >= 230 && K * N >= 80000000ll) return wide512_pass();
+    *variant = kWide2D2M1;
+    return sa;
+}
+
 static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, int* split_k,
                       bool allow_shared_chunk = true) {
     const int64_t chunks = K / 128 > 0 ? K / 128 : 1;
@@ -1645,31 +1738,10 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int v = kDma1x4;
         int64_t s = 1;
         const int64_t row_blocks = cdiv(M, 16);   // above 16 rows the one-m-tile kernels run one block of 16 per z
-        // Split count of the shared-chunk kernel with the in-kernel tail (M <= 4; N >= 8192 and 80 M weights or more:
-        // 5120 x 20480 at one row 20.3 -> 16.9 us, 8192 x 14336 20.2 -> 18.5, 8192 x 10240 17.6 -> 15.8, 12288 x 8192
-        // 19.5 -> 17.9, 5120 x 17408 15.8 -> 15.4; 4096 x 14336 and smaller lose), 0 = the one-tile kernel runs.  A CU
-        // streams at a fixed rate, so the launch lasts rounds x chunks per split (workgroups come in rounds of one per
-        // CU), plus a tail per row and split (0.06 of a chunk's time).  Taken at one or two rows; at three and four
-        // only where five splits or fewer do and N >= 28672 (5120 x 51200 at four rows 36.0 -> 34.7 us, 8192 x 28672
-        // 34.4 -> 32.7; but 5120 x 25600 20.6 -> 20.9, 5120 x 34816 in ten splits 27.3 -> 29.9).
-        int64_t wide1_tail_splits = 0;
-        if (allow_shared_chunk && M <= kWideTailRows && N % 512 == 0 && N >= 8192 && K * N >= 80000000ll && chunks >= 8) {
-            double best = 1e30;
-            const int64_t hi = chunks / 4 < 16 ? chunks / 4 : 16;
-            for (int64_t c = 2; c <= hi; ++c) {
-                const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
-                if (splits != c) continue;
-                const int64_t wgs = N / 512 * splits;
-                // (one workgroup per CU at most runs the three-buffer form, 5 % faster: see the choice of depth below)
-                const double cost = ((double)(cdiv(wgs, 256) * cps) + 0.06 * (double)(M * splits)) *
-                                    (wgs <= 256 && cps >= 6 ? 0.95 : 1.0);
-                if (cost < best - 1e-9) {
-                    best = cost;
-                    wide1_tail_splits = c;
-                }
-            }
-            if (M > 2 && (wide1_tail_splits > 5 || N < 28672)) wide1_tail_splits = 0;
-        }
+        // Up to 16 rows on large weights: the one-m-tile forms of the shared-chunk kernel (pick_one_m_tile), 0 = none.
+        int64_t m1_splits = 0;
+        int m1_variant = 0;
+        if (allow_shared_chunk && M <= 16) m1_splits = pick_one_m_tile(M, N, K, chunks, &m1_variant);
         if (allow_shared_chunk && M > 16 && M <= 64 && N % 512 == 0 && N >= 5120 &&
             K * N >= (M > 48 ? (50ll << 20) : (M > 32 ? 64000000ll : 95000000ll))) {
             // 17..64 rows on the largest weights (from sweeps: the fused gate|up of Qwen3-8B and the MLP of
@@ -1679,25 +1751,9 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             v = M > 32 ? kWideM4 : kWideM2;
             s = 256 / (N / 512);
             if (s > chunks / 4) s = chunks / 4;
-        } else if (wide1_tail_splits > 0) {
-            // up to four rows on the same weights: the shared-chunk kernel again (its row pieces are 256 bytes where
-            // the one-tile kernel's are 64, and a bare read of 64-byte pieces streams 10 % slower), the K splits
-            // added by the last workgroup to arrive.  One row: 5120 x 25600 19.9 -> 19.6 us, 4096 x 24576 18.1 ->
-            // 17.1, 5120 x 51200 35.5 -> 33.3, 8192 x 28672 33.4 -> 31.6, 4096 x 28672 20.2 -> 18.4.
-            v = kWideM1T;
-            s = wide1_tail_splits;
-        } else if (allow_shared_chunk && M >= 5 && M <= 16 && N % 512 == 0 && N >= 10240 && K * N >= 80000000ll) {
-            // 5..16 rows on wide, large weights (the MLP gate|up of Qwen3-8B and larger, fused or not): the shared-chunk
-            // kernel with one m-tile -- the staged kernel's waves bring their own x, 4 KiB per chunk beside 8 KiB of
-            // weights at 16 rows; shared by eight waves it is 0.5 KiB per wave.  5120 x 25600 at 8 / 16 rows 22.7 /
-            // 25.0 -> 21.3 / 21.9 us, 5120 x 51200 40.2 / 46.2 -> 36.6 / 39.5, 4096 x 24576 20.0 / 22.0 -> 18.8 / 19.5,
-            // 5120 x 20480 21.8 / 23.1 -> 19.4 / 20.3, 8192 x 14336 24.2 / 25.7 -> 21.4 / 22.1, 8192 x 10240 20.1 /
-            // 21.1 -> 19.2 / 19.7; on narrower or smaller weights (12288 x 8192: 19.9 / 21.5 -> 21.1 / 22.3, 4096 x
-            // 12288, 5120 x 10240, 25600 x 5120) its K splits' partial round trip costs more than it saves.
-            v = kWideM1;
-            s = 256 / (N / 512);
-            if (s < 2) s = 2;
-            if (s > chunks / 4) s = chunks / 4;
+        } else if (m1_splits > 0) {
+            v = m1_variant;
+            s = m1_splits;
         } else if (chunks <= 8) {
             v = kDma1x8;
         } else if (M <= 4) {
@@ -1709,20 +1765,36 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             // 4096 x 2048 8.3 us in 4 splits of eight waves against 7.4 in 8 of four).
             // short K: one chunk per wave (the step-by-step form), at most 10 splits (the tail is a larger share of
             // a 6 us launch: 2048 x 1024 at one row 5.55 us in 8 splits, 5.23 in 4)
-            const int64_t cap = chunks < 64 ? (chunks / 4 < 10 ? chunks / 4 : 10) : 16;
+            // (that limit is for launches of a few microseconds; from 32 Mi weights on up to 16 again: 6144 x 10240
+            // at one row 15.4 us in 7 splits, two chunks per wave, 12.9 in 12)
+            const int64_t short_cap = K * N >= (32ll << 20) ? 16 : 10;
+            const int64_t cap = chunks < 64 ? (chunks / 4 < short_cap ? chunks / 4 : short_cap) : 16;
             int64_t wk = 4;
             s = cdiv(2048, tiles * 4);
             // and no more than two chunks per wave: a wave takes its chunks one after the other, each a round trip
             // of its own (5120 x 51200 at one row 41.5 us in 2 splits -- five chunks per wave --, 32.5 in 5 or 6;
             // 5120 x 34816 32.9 -> 24.9 us)
             if (s < cdiv(chunks, 8) && cdiv(chunks, 8) <= cap) s = cdiv(chunks, 8);
-            if (tiles <= 48 && chunks >= 160) {
-                wk = 8;
-                s = cdiv(4096, tiles * 8);
-            }
-            if (wk == 8) v = kDma1x8;
             if (s > cap) s = cap;
             s = balance_splits(chunks, s, wk, cap);
+            if (tiles <= 56 && chunks >= 64) {
+                // (long K, few column tiles: eight-wave workgroups where their split wastes no more wave slots than the
+                // four-wave one -- 16384 x 4096 17.6 -> 14.1 us in 16 splits, 14336 x 4096 14.2 -> 13.3, 8192 x 7168
+                // 13.1 -> 12.2, 12288 x 4096 12.55 -> 12.2; 17408 x 5120 keeps four waves: 13 splits of 11 chunks are
+                // 3, 3, 3, 2 per wave there and 2, 2, 2, 1, 1, 1, 1, 1 on eight: 16.3 against 16.9 us)
+                auto wasted = [&](int64_t c, int64_t waves) {
+                    const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
+                    return 1.0 - (double)chunks / (double)(splits * waves * cdiv(cps, waves));
+                };
+                int64_t s8 = cdiv(4096, tiles * 8);
+                if (s8 > cap) s8 = cap;
+                s8 = balance_splits(chunks, s8, 8, cap);
+                if (wasted(s8, 8) <= wasted(s, 4) + 1e-9) {
+                    wk = 8;
+                    s = s8;
+                    v = kDma1x8;
+                }
+            }
         } else {
             // 5..64 rows.  A CU streams at a fixed rate whatever the number of workgroups on it, so the launch lasts
             // as long as the CU with the most bytes: at least about 200 workgroups, and a count that fills whole
@@ -1755,16 +1827,6 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             }
         }
         if (s < 1) s = 1;
-        if (v == kWideM1 || v == kWideM1T) {
-            // One workgroup per CU at most and enough chunks per split to fill the pipeline: three staging buffers, two
-            // chunks in flight while one is multiplied (5120 x 25600 in five splits 19.5 -> 18.4 us at one row,
-            // 22.0 -> 21.6 at 16; 8192 x 28672 in four 32.9 -> 29.2 / 33.2 -> 32.3; 5120 x 51200 at 16 rows in two
-            // 40.4 -> 36.7).  With more workgroups than CUs two of the two-buffer form share a CU and do better
-            // (5120 x 51200 at one row in five splits: 32.8 against 35.1 us), and on short splits the deeper prologue
-            // does not pay (4096 x 24576, seven chunks per split, at 8 / 16 rows: 18.8 / 19.7 against 19.2 / 20.0).
-            const int64_t cps = cdiv(chunks, s), splits = cdiv(chunks, cps);
-            if (N / 512 * splits <= 256 && cps >= (v == kWideM1T ? 6 : 8)) v = v == kWideM1T ? kWideD3M1T : kWideD3M1;
-        }
         *variant = v;
         *split_k = (int)s;
         return;
@@ -1869,6 +1931,16 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
             e = f16 ? launch_gemv_wide<F16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
                     : launch_gemv_wide<BF16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
             break;
+#define AWQ_WIDE2_CASE(ID, DD, TT)                                                                                      \
+        case ID:                                                                                                        \
+            e = f16 ? launch_gemv_wide<F16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act) \
+                    : launch_gemv_wide<BF16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act); \
+            break;
+        AWQ_WIDE2_CASE(kWide2D2M1, 2, false)
+        AWQ_WIDE2_CASE(kWide2D2M1T, 2, true)
+        AWQ_WIDE2_CASE(kWide2D3M1, 3, false)
+        AWQ_WIDE2_CASE(kWide2D3M1T, 3, true)
+#undef AWQ_WIDE2_CASE
         case kWideD3M1T:
             e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
                     : launch_gemv_wide<BF16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);

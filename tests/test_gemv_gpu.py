@@ -153,20 +153,22 @@ def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("M,K,N,splits", [(1, 4096, 24576, 5), (2, 4096, 24576, 5), (5, 4096, 24576, 5),
-                                          (9, 4096, 24576, 5), (16, 4096, 24576, 5), (3, 4096, 28672, 4),
-                                          (4, 4096, 28672, 4), (1, 12288, 8192, 16), (16, 5120, 20480, 6)])
-def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
-    """Up to 16 rows on wide, large weights (80 M and more): the default dispatch takes the shared-chunk kernel with one
-    m-tile (the odd byte halves hand their fragments to their partners; the K splits are added by the last workgroup
-    to arrive at up to four rows, by a second pass above); with and without a bias, against the oracle, and forced
-    with other split counts (same oracle)."""
+@pytest.mark.parametrize("M,K,N,plan", [(1, 4096, 24576, "wide2d2m1t/5"), (5, 4096, 24576, "wide2d2m1t/5"),
+                                        (9, 4096, 24576, "wided2m1/5"), (16, 4096, 24576, "wided2m1/5"),
+                                        (3, 4096, 28672, "wided3m1t/4"), (16, 4096, 28672, "wided3m1/4"),
+                                        (1, 12288, 8192, "wide2d3m1t/8"), (8, 12288, 8192, "wide2d3m1t/8"),
+                                        (16, 5120, 20480, "wide2d3m1/3"), (2, 5120, 17408, "wide2d2m1t/7")])
+def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, plan):
+    """Up to 16 rows on wide, large weights: the default dispatch takes a one-m-tile form of the shared-chunk kernel
+    (512 or 256 columns per workgroup; the odd byte halves hand their fragments to their partners; two or three
+    staging buffers; the K splits added by the last workgroup to arrive or by a second pass).  The planned form with
+    and without a bias, and every form forced with other split counts, against the oracle; run-to-run equal bits."""
     import ctypes
     L = _lib.lib()
     names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
     v, sp = ctypes.c_int(), ctypes.c_int()
     assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
-    assert names[v.value].endswith("m1t" if M <= 4 else "m1") and sp.value == splits, (names[v.value], sp.value)
+    assert f"{names[v.value]}/{sp.value}" == plan
     print(f"gemv shared-chunk, one m-tile {dtype} M={M} K={K} N={N}", flush=True)
     p = random_packed(K, N, 128, dtype, seed=K + N + M)
     xb = make_x(M, K, dtype, seed=M)
@@ -185,7 +187,9 @@ def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, splits):
         assert err <= TIGHT[dtype], (what, err)
 
     check_plain(nq.awq_gemm(xd, *dev, 8), "default")
-    for vn in ("wided2m1", "wided2m1t", "wided3m1", "wided3m1t"):   # two or three staging buffers, either way of adding the K splits
+    forms = [n for n in names if n.startswith("wide") and n.endswith(("m1", "m1t"))]
+    assert len(forms) == 8, forms
+    for vn in forms:
         for split in (1, 2, 8):
             yv = awq_gemv_variant(xd, *dev, names.index(vn), split)
             check_plain(yv, (vn, split))

@@ -148,7 +148,7 @@ def test_dispatch_plans_are_consistent():
     gemm_names = [L.awq_gemm_variant_name(i).decode() for i in range(L.awq_gemm_variant_count())]
     shapes = [(1024, 2048), (1024, 1024), (2048, 1024), (1024, 3072), (3072, 1024), (4096, 12288), (12288, 4096),
               (5120, 25600), (25600, 5120), (5120, 10240), (8192, 5120), (5120, 34816), (4096, 24576), (5120, 20480),
-              (8192, 14336), (12288, 8192), (128, 128),
+              (8192, 14336), (12288, 8192), (8192, 8192), (6144, 10240), (16384, 4096), (128, 128),
               (256, 8), (1024, 1032), (3072, 136)]
     for K, N in shapes:
         for M in (1, 2, 4, 5, 8, 16, 17, 32, 33, 48, 64):
@@ -167,16 +167,21 @@ def test_dispatch_plans_are_consistent():
                 else:
                     assert M <= 16
                 if name.startswith("wide"):
-                    assert N % 512 == 0 and K * N >= 50 << 20
-                    assert name.endswith("m1t") == (M <= 4) and name.endswith("m1") == (5 <= M <= 16)
-                    assert (name == "wided2m4") == (M > 32)
-                    if name[5] == "3":      # three staging buffers: one workgroup per CU at most
-                        cps = -(-chunks // s)
-                        assert N // 512 * -(-chunks // cps) <= 256 and cps >= 6
-                    if M >= 5:
-                        assert N // 512 * s <= 256 + N // 512        # about one workgroup per CU
-                    else:                                            # in-kernel tail: up to two rounds of workgroups
-                        assert N >= 8192 and K * N >= 80000000 and s <= 16 and (M <= 2 or (s <= 5 and N >= 28672))
+                    cols = 256 if name.startswith("wide2") else 512      # columns per workgroup
+                    assert N % cols == 0 and K * N >= 50 << 20
+                    one = name.endswith(("m1", "m1t"))
+                    assert one == (M <= 16) and name.endswith("m4") == (M > 32)
+                    cps = -(-chunks // s)
+                    wgs = N // cols * -(-chunks // cps)
+                    if name.endswith("t"):                               # in-kernel tail: few rows x splits
+                        assert M <= 8 and M * s <= 64 and s <= 25
+                        assert wgs <= 560
+                    elif one or M > 16:
+                        assert wgs <= 256 + N // cols or cols == 256     # second pass: about one workgroup per CU
+                    if "d3" in name:                                     # three staging buffers
+                        assert one and cps >= 6 and (wgs <= 256 or cols == 256)
+                    if cols == 256:
+                        assert 8192 <= N < 28672
                 if not staged_ok:
                     assert not name.startswith(("dma", "wide"))
                 if g == 128:   # awq_gemv_workspace_bytes takes no group size: it must cover this plan
@@ -207,27 +212,27 @@ def test_dispatch_plans_are_consistent():
     assert rc == 0 and gemv_names[v] == "dma1x4" and s >= 3
     wgs = 34816 // 128 * s
     assert wgs / (256 * -(-wgs // 256)) >= 0.8
-    # 5..16 rows on the widest weights: the shared-chunk kernel with one m-tile, about one workgroup per CU
-    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 5120, 128)      # 68 groups x 3 splits of 14 chunks: three buffers
+    # up to 16 rows on wide, large weights: the one-m-tile forms of the shared-chunk kernel
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 34816, 5120, 128)      # N >= 28672: 512 columns, 68 groups x 3 splits of 14 chunks
     assert rc == 0 and gemv_names[v] == "wided3m1" and s == 3
-    rc, v, s = _plan(L.awq_gemv_plan, 4, 34816, 5120, 128)      # three or four rows: the one-tile kernel, two chunks per wave
+    rc, v, s = _plan(L.awq_gemv_plan, 4, 34816, 5120, 128)       # three or four rows there: ten splits would be too many
     assert rc == 0 and gemv_names[v] == "dma1x4" and s == 5
-    # one or two rows there: the shared-chunk kernel with the in-kernel tail, split so that whole rounds of workgroups
-    # carry the fewest chunks each (68 groups x 7 splits = 476 workgroups: two rounds of six chunks)
-    rc, v, s = _plan(L.awq_gemv_plan, 1, 34816, 5120, 128)
+    rc, v, s = _plan(L.awq_gemv_plan, 1, 34816, 5120, 128)       # one row: 68 x 7 = 476 workgroups, two rounds of six chunks
     assert rc == 0 and gemv_names[v] == "wided2m1t" and s == 7
-    rc, v, s = _plan(L.awq_gemv_plan, 4, 51200, 5120, 128)      # 100 groups x 5 splits: two full rounds, also at four rows
+    rc, v, s = _plan(L.awq_gemv_plan, 4, 51200, 5120, 128)       # 100 groups x 5 splits: two full rounds, also at four rows
     assert rc == 0 and gemv_names[v] == "wided2m1t" and s == 5
-    rc, v, s = _plan(L.awq_gemv_plan, 1, 25600, 5120, 128)      # 50 groups x 5 splits = 250 workgroups: three buffers
-    assert rc == 0 and gemv_names[v] == "wided3m1t" and s == 5
-    # wide mid-size weights (80 M and more) take it too: 16 groups x 16 splits at one row, 40 groups x 6 at 16 rows;
-    # 12288 x 8192 at 16 rows and anything smaller stay with the one-tile kernel
-    rc, v, s = _plan(L.awq_gemv_plan, 1, 8192, 12288, 128)
-    assert rc == 0 and gemv_names[v] == "wided3m1t" and s == 16
-    rc, v, s = _plan(L.awq_gemv_plan, 16, 20480, 5120, 128)
-    assert rc == 0 and gemv_names[v] == "wided2m1" and s == 6
-    assert gemv_names[_plan(L.awq_gemv_plan, 16, 8192, 12288, 128)[1]] == "dma1x4"
-    assert gemv_names[_plan(L.awq_gemv_plan, 1, 14336, 4096, 128)[1]] == "dma1x4"
+    rc, v, s = _plan(L.awq_gemv_plan, 1, 25600, 5120, 128)       # N < 28672: 256 columns, 100 groups x 5 splits
+    assert rc == 0 and gemv_names[v] == "wide2d2m1t" and s == 5
+    rc, v, s = _plan(L.awq_gemv_plan, 8, 25600, 5120, 128)       # the tail while rows x splits <= 64
+    assert rc == 0 and gemv_names[v] == "wide2d2m1t" and s == 5
+    rc, v, s = _plan(L.awq_gemv_plan, 4, 8192, 12288, 128)       # eleven splits or more for 500 workgroups: one per CU instead
+    assert rc == 0 and gemv_names[v] == "wide2d3m1t" and s == 8
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 8192, 12288, 128)      # and the second pass beyond 64 rows x splits
+    assert rc == 0 and gemv_names[v] == "wide2d3m1" and s == 8
+    rc, v, s = _plan(L.awq_gemv_plan, 16, 24576, 4096, 128)      # 96 groups of 256 fill 75 % of the CUs in two splits: 512 columns
+    assert rc == 0 and gemv_names[v] == "wided2m1" and s == 5
+    assert gemv_names[_plan(L.awq_gemv_plan, 1, 4096, 16384, 128)[1]] == "dma1x8"      # narrow weights: the one-tile kernel
+    assert gemv_names[_plan(L.awq_gemv_plan, 16, 12288, 4096, 128)[1]] == "dma1x4"     # and small ones
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
     # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
     rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120, 128, _lib.AWQ_BF16)
