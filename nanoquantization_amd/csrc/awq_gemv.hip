@@ -1777,7 +1777,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             if (s < cdiv(chunks, 8) && cdiv(chunks, 8) <= cap) s = cdiv(chunks, 8);
             if (s > cap) s = cap;
             s = balance_splits(chunks, s, wk, cap);
-            if (tiles <= 56 && chunks >= 64) {
+            if (tiles <= 56 && chunks > 64) {
                 // (long K, few column tiles: eight-wave workgroups where their split wastes no more wave slots than the
                 // four-wave one -- 16384 x 4096 17.6 -> 14.1 us in 16 splits, 14336 x 4096 14.2 -> 13.3, 8192 x 7168
                 // 13.1 -> 12.2, 12288 x 4096 12.55 -> 12.2; 17408 x 5120 keeps four waves: 13 splits of 11 chunks are
@@ -1786,14 +1786,26 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
                     const int64_t cps = cdiv(chunks, c), splits = cdiv(chunks, cps);
                     return 1.0 - (double)chunks / (double)(splits * waves * cdiv(cps, waves));
                 };
+                // (two eight-wave workgroups fit a CU: beyond about 512 of them a third round starts -- 13824 x 5120 in
+                // 14 splits, 560 workgroups, 14.9 us against 13.7 in 12 splits of four waves)
+                int64_t cap8 = 540 / tiles < cap ? 540 / tiles : cap;
                 int64_t s8 = cdiv(4096, tiles * 8);
-                if (s8 > cap) s8 = cap;
-                s8 = balance_splits(chunks, s8, 8, cap);
+                if (s8 > cap8) s8 = cap8;
+                s8 = balance_splits(chunks, s8, 8, cap8);
                 if (wasted(s8, 8) <= wasted(s, 4) + 1e-9) {
                     wk = 8;
                     s = s8;
                     v = kDma1x8;
                 }
+            } else if (tiles <= 64 && chunks >= 48 && chunks <= 64 &&
+                       (tiles * 8 <= 256 || tiles * 8 * 20 >= 256 * cdiv(tiles * 8, 256) * 17)) {
+                // 6144 <= K <= 8192 on up to 64 column tiles: eight splits of eight waves, one chunk per wave at most
+                // (the step-by-step form) -- 6144 x 4096 10.4 -> 8.8 us, 8192 x 4096 10.0 -> 9.4, 8192 x 2048 9.6 -> 9.0,
+                // 7168 x 8192 14.4 -> 13.0 --, where those workgroups come in whole rounds of the CUs (40 or 48 tiles
+                // make 1.25 / 1.5 rounds: 8192 x 5120 11.1 -> 11.7, 6144 x 6144 10.5 -> 11.0)
+                wk = 8;
+                s = 8;
+                v = kDma1x8;
             }
         } else {
             // 5..64 rows.  A CU streams at a fixed rate whatever the number of workgroups on it, so the launch lasts
