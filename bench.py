@@ -23,6 +23,7 @@ of the packed weight, the known-size kernel the traffic counters are calibrated 
 from __future__ import annotations
 
 import argparse
+import re
 import json
 import os
 import sys
@@ -166,10 +167,12 @@ def gemv_kernel_name(M, N, K, dtype_name, g=G):
         return "?"
     name = L.awq_gemv_variant_name(v.value).decode()
     T = "F16" if dtype_name == "f16" else "BF16"
-    if name.startswith("wide") and name.endswith("t"):   # wided<DEPTH>m<MT>t: the K splits are added inside the kernel
-        kern = f"awq::gemv_wide_kernel<{T},{name[5]},{name[7]},true>"
-    elif name.startswith("wide"):
-        kern = f"awq::gemv_wide_kernel<{T},{name[5]},{name[7]},false> + awq::gemv_wide_reduce_kernel<{T}>"
+    wide = re.fullmatch(r"wide(2?)d(\d)m(\d)(t?)", name)   # wide[2]d<DEPTH>m<MT>[t]: 256 columns per workgroup, in-kernel tail
+    if wide:
+        wn = 2 if wide.group(1) else 4
+        kern = f"awq::gemv_wide_kernel<{T},{wide.group(2)},{wide.group(3)},{'true' if wide.group(4) else 'false'},{wn}>"
+        if not wide.group(4):   # the K splits are added by a second kernel
+            kern += f" + awq::gemv_wide_reduce_kernel<{T}>"
     elif name.startswith("dma"):
         kern = f"awq::gemv_dma_kernel<{T},{name[5]},plain>"
     else:
