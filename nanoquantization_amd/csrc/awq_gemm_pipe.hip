@@ -406,9 +406,21 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float* __re
     const float* p = partials + ((size_t)r << 16) + row * 256 + col;
     const size_t plane = (size_t)plan.tail_tiles << 16;
     f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
-    for (int s = 0; s < plan.splits; ++s) {
-        lo += *reinterpret_cast<const f32x4*>(p + s * plane);
-        hi += *reinterpret_cast<const f32x4*>(p + s * plane + 4);
+    // four slices' loads in flight at a time, added in slice order
+    for (int s0 = 0; s0 < plan.splits; s0 += 4) {
+        f32x4 a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t off = (size_t)min(s0 + u, plan.splits - 1) * plane;
+            a[u] = *reinterpret_cast<const f32x4*>(p + off);
+            b[u] = *reinterpret_cast<const f32x4*>(p + off + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (s0 + u < plan.splits) {
+                lo += a[u];
+                hi += b[u];
+            }
     }
     float out[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     if (plan.act) {

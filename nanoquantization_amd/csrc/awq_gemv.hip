@@ -1371,9 +1371,22 @@ __global__ __launch_bounds__(256) void gemv_wide_reduce_kernel(const float* __re
     const size_t plane = (size_t)M * N;
     const float* p = partials + (size_t)m * N + n0;
     f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
-    for (int s = 0; s < splits; ++s) {
-        lo += *reinterpret_cast<const f32x4*>(p + s * plane);
-        hi += *reinterpret_cast<const f32x4*>(p + s * plane + 4);
+    // eight splits' loads in flight at a time (a loop of load, add, load, add is one memory round trip per split:
+    // 4.7 us for five splits of 16 rows x 25600 columns), added in split order all the same
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        f32x4 a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const size_t off = (size_t)min(s0 + u, splits - 1) * plane;
+            a[u] = *reinterpret_cast<const f32x4*>(p + off);
+            b[u] = *reinterpret_cast<const f32x4*>(p + off + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (s0 + u < splits) {
+                lo += a[u];
+                hi += b[u];
+            }
     }
     float out[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     if (act) {
