@@ -1157,9 +1157,10 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, float* __restrict__ partials,
     int* __restrict__ counters, int M, int N, int K, int chunks_per_group, int chunks_per_split, int splits, int act) {
-    // HMT: pieces of x a wave brings per chunk (with one m-tile the four pieces go to waves 0..3, one each)
-    constexpr int CH = 4, HMT = MT >= 2 ? MT / 2 : 1;
-    static_assert(WN == 4 || (WN == 2 && MT == 1), "512 columns, or 256 with one m-tile");
+    // XP: pieces of x a wave brings per chunk (with one m-tile the four pieces go to waves 0..3, one each);
+    // HMT: m-tiles each of the two byte-half waves of a column tile stores at the end
+    constexpr int CH = 4, XP = MT >= 2 ? 4 * MT / (2 * WN) : 1, HMT = MT >= 2 ? MT / 2 : 1;
+    static_assert(WN == 4 || WN == 2, "512 or 256 columns per workgroup");
     static_assert(DEPTH >= 2 && DEPTH <= 3, "two or three staging buffers");
     static_assert(MT == 1 || MT == 2 || MT == 4, "m-tiles per workgroup");
     static_assert(!TAIL || MT == 1, "the in-kernel tail of a K split: one m-tile only");
@@ -1189,12 +1190,12 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
         const int slot = h * 16 + dsl;
         wsrc[h] = (uint32_t)((slot & 3) * 8 + (slot >> 2)) * (uint32_t)words + (uint32_t)(tile * 16 + dq * 4);
     }
-    // x: the 4*MT (step, m-tile) pieces of 16 rows x 64 B are dealt to the 8 waves, HMT each
-    int x_s[HMT], x_mt[HMT];
-    uint32_t xsrc[HMT];
+    // x: the 4*MT (step, m-tile) pieces of 16 rows x 64 B are dealt to the 2*WN waves, XP each
+    int x_s[XP], x_mt[XP];
+    uint32_t xsrc[XP];
 #pragma unroll
-    for (int i = 0; i < HMT; ++i) {
-        const int o = MT >= 2 ? wave * HMT + i : (wave & 3);
+    for (int i = 0; i < XP; ++i) {
+        const int o = MT >= 2 ? wave * XP + i : (wave & 3);
         x_s[i] = o / MT;
         x_mt[i] = o % MT;
         xsrc[i] = (uint32_t)min(16 * x_mt[i] + (lane >> 2), M - 1) * (uint32_t)K + (uint32_t)(lane & 3) * 8u;
@@ -1204,7 +1205,7 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
     const bool zs_lane = lane < 16;
 
     // per wave and chunk (an upper bound where a wave brings no x; only a third buffer waits by this count)
-    constexpr int kDmaOps = CH + HMT + 1;
+    constexpr int kDmaOps = CH + XP + 1;
     // one m-tile: waves 4..7 bring no x, one load fewer per chunk
     const bool full_count = MT >= 2 || wave < 4;   // uniform
     auto wait_chunks_in_flight = [&](int n) {   // all but the loads of the n newest chunks have landed
@@ -1232,7 +1233,7 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
         __builtin_amdgcn_wave_barrier();
         if (x_wave) {
 #pragma unroll
-            for (int i = 0; i < HMT; ++i)
+            for (int i = 0; i < XP; ++i)
                 __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + x_s[i] * 32) + xsrc[i]),
                                                  AWQ_LPTR(base + x_s[i] * x_step + x_mt[i] * 1024), 16, 0, 0);
         }
@@ -1323,7 +1324,7 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
             return;
         }
         // Exchange: this wave stores m-tiles BH*HMT .. and sends its fragments of the other m-tiles to its
-        // partner (wave ^ 4).  xch[wave][(ml*4 + f)*4 + r][lane]
+        // partner (wave ^ WN).  xch[wave][(ml*4 + f)*4 + r][lane]
         __syncthreads();   // staging is free
         float* xch = red;
         constexpr int PER_WAVE = HMT * 16 * 64;
@@ -1344,7 +1345,7 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
                 acc8[2 * f + BH] = acc[mt][f];
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    acc8[2 * f + 1 - BH][r] = xch[(wave ^ 4) * PER_WAVE + ((ml * 4 + f) * 4 + r) * 64 + lane];
+                    acc8[2 * f + 1 - BH][r] = xch[(wave ^ WN) * PER_WAVE + ((ml * 4 + f) * 4 + r) * 64 + lane];
             }
             if (16 * mt < M)
                 gemv_reduce_store<T, 1, WN, 1, true>(acc8, 16 * mt, red, lane, wn, group, split, splits, bias, y,
@@ -1436,9 +1437,12 @@ static const GemvVariant kGemvVariants[] = {
     {"wide2d2m1t", 1, 4, false, 2, 2, 1, true},
     {"wide2d3m1", 1, 4, false, 2, 3, 1, true},
     {"wide2d3m1t", 1, 4, false, 2, 3, 1, true},
+    // 256 columns, two m-tiles (17..32 rows)
+    {"wide2d2m2", 1, 4, false, 2, 2, 2, true},
+    {"wide2d3m2", 1, 4, false, 2, 3, 2, true},
 };
 enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6, kWideM1T = 7,
-       kWideD3M1 = 8, kWideD3M1T = 9, kWide2D2M1 = 10, kWide2D2M1T = 11, kWide2D3M1 = 12, kWide2D3M1T = 13 };
+       kWideD3M1 = 8, kWideD3M1T = 9, kWide2D2M1 = 10, kWide2D2M1T = 11, kWide2D3M1 = 12, kWide2D3M1T = 13, kWide2D2M2 = 14, kWide2D3M2 = 15 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = kDma1x4;
 
@@ -1740,6 +1744,36 @@ static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, 
     return sa;
 }
 
+// 17..32 rows: the shared-chunk kernel on 256 columns per workgroup with two m-tiles (four waves: two or three of
+// these smaller workgroups share a CU and run out of step, where the eight waves of a 512-column workgroup pass one
+// barrier per chunk together), second pass for the K splits.  Split as for up to 16 rows: about one workgroup per CU
+// if that fills 85 % of them (plan B; three buffers where a split has six chunks or more), else about 500 (plan A).
+// For N < 28672 and 48 M weights or more -- against the row blocks of the one-tile kernel or the 512-column form at
+// 24 / 32 rows: 5120 x 17408 27.6 / 28.9 -> 20.3 / 21.8 us, 17408 x 5120 26.5 / 27.0 -> 21.4 / 22.4, 8192 x 8192
+// 22.3 / 22.8 -> 17.0 / 17.8, 5120 x 10240 19.6 / 20.2 -> 16.4 / 16.6, 12288 x 4096 18.5 -> 16.1 / 16.7, 6144 x 8192
+// 17.8 / 18.3 -> 15.6 / 16.4, 5120 x 25600 26.6 / 26.8 -> 25.1; 5120 x 51200 stays with 512 columns (44.6 against
+// 46.6).  With four m-tiles (33..64 rows) the form was measured too and is not used: within 5 % of the 512-column
+// one where it wins (5120 x 10240 at 64 rows 27.3 -> 25.3 us, 5120 x 17408 32.3 -> 31.7), 10..20 % slower with few
+// long splits (8192 x 14336 in four: 43.0 against 37.9).
+static int64_t pick_shared_256(int64_t M, int64_t N, int64_t K, int64_t chunks, int* variant) {
+    if (M > 32 || N % 256 != 0 || chunks < 8 || N < 4096 || N >= 28672 || K * N < 48000000ll) return 0;
+    auto normalised = [&](int64_t c) { return cdiv(chunks, cdiv(chunks, c)); };
+    const int64_t groups = N / 256;
+    int64_t sb = 256 / groups;
+    if (sb > chunks / 4) sb = chunks / 4;
+    if (sb >= 2 && normalised(sb) * groups >= 218) {
+        sb = normalised(sb);
+        *variant = cdiv(chunks, sb) >= 6 ? kWide2D3M2 : kWide2D2M2;
+        return sb;
+    }
+    int64_t sa = 512 / groups;
+    if (sa > 25) sa = 25;
+    if (sa > chunks / 4) sa = chunks / 4;
+    if (sa < 1) return 0;
+    *variant = kWide2D2M2;
+    return normalised(sa);
+}
+
 static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, int* split_k,
                       bool allow_shared_chunk = true) {
     const int64_t chunks = K / 128 > 0 ? K / 128 : 1;
@@ -1755,7 +1789,8 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int64_t m1_splits = 0;
         int m1_variant = 0;
         if (allow_shared_chunk && M <= 16) m1_splits = pick_one_m_tile(M, N, K, chunks, &m1_variant);
-        if (allow_shared_chunk && M > 16 && M <= 64 && N % 512 == 0 && N >= 5120 &&
+        if (allow_shared_chunk && M > 16 && M <= 32) m1_splits = pick_shared_256(M, N, K, chunks, &m1_variant);
+        if (m1_splits == 0 && allow_shared_chunk && M > 16 && M <= 64 && N % 512 == 0 && N >= 5120 &&
             K * N >= (M > 48 ? (50ll << 20) : (M > 32 ? 64000000ll : 95000000ll))) {
             // 17..64 rows on the largest weights (from sweeps: the fused gate|up of Qwen3-8B and the MLP of
             // Qwen3-14B/32B and, above 32 rows, the 32B fused q/k/v): eight-wave workgroups of 512 columns sharing the staged chunk, K split so that about
@@ -1966,6 +2001,14 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         AWQ_WIDE2_CASE(kWide2D3M1, 3, false)
         AWQ_WIDE2_CASE(kWide2D3M1T, 3, true)
 #undef AWQ_WIDE2_CASE
+#define AWQ_WIDE2M_CASE(ID, DD, MM)                                                                                     \
+        case ID:                                                                                                        \
+            e = f16 ? launch_gemv_wide<F16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act) \
+                    : launch_gemv_wide<BF16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act); \
+            break;
+        AWQ_WIDE2M_CASE(kWide2D2M2, 2, 2)
+        AWQ_WIDE2M_CASE(kWide2D3M2, 3, 2)
+#undef AWQ_WIDE2M_CASE
         case kWideD3M1T:
             e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
                     : launch_gemv_wide<BF16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);

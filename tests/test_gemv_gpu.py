@@ -135,11 +135,21 @@ def test_gemv_batched_decode_rows(dtype, M):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("M,K,N", [(64, 4096, 6144), (33, 4096, 6144), (24, 8192, 5120), (17, 8192, 5120)])
-def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N):
-    # 17..64 rows on weights large enough for the default dispatch to take the shared-chunk kernel
-    # (eight waves per 512 columns, K split, second-pass reduction), with a bias
-    print(f"gemv shared-chunk {dtype} M={M} K={K} N={N}", flush=True)
+@pytest.mark.parametrize("M,K,N,plan", [(64, 4096, 6144, "dma1x4"), (33, 4096, 6144, "dma1x4"), (24, 8192, 5120, "dma1x4"),
+                                        (17, 8192, 5120, "dma1x4"), (24, 8192, 8192, "wide2d3m2/8"),
+                                        (32, 5120, 17408, "wide2d2m2/7"), (17, 12288, 4096, "wide2d3m2/16"),
+                                        (64, 5120, 17408, "wided2m4/7"), (32, 4096, 28672, "wided2m2/4")])
+def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N, plan):
+    # 17..64 rows, with a bias: blocks of 16 rows on the one-tile kernel, and on larger weights the shared-chunk kernel
+    # (256 columns x two m-tiles with two or three staging buffers; 512 columns x two or four m-tiles), K split,
+    # second-pass reduction
+    import ctypes
+    L = _lib.lib()
+    names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
+    v, sp = ctypes.c_int(), ctypes.c_int()
+    assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
+    assert f"{names[v.value]}/{sp.value}".startswith(plan), (names[v.value], sp.value)
+    print(f"gemv {names[v.value]} {dtype} M={M} K={K} N={N}", flush=True)
     p = random_packed(K, N, 128, dtype, seed=K + N + M)
     xb = make_x(M, K, dtype, seed=M)
     bias = np.linspace(-1, 1, N).astype(np.float32)

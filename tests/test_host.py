@@ -168,7 +168,7 @@ def test_dispatch_plans_are_consistent():
                     assert M <= 16
                 if name.startswith("wide"):
                     cols = 256 if name.startswith("wide2") else 512      # columns per workgroup
-                    assert N % cols == 0 and K * N >= 50 << 20
+                    assert N % cols == 0 and K * N >= 48000000
                     one = name.endswith(("m1", "m1t"))
                     assert one == (M <= 16) and name.endswith("m4") == (M > 32)
                     cps = -(-chunks // s)
@@ -179,9 +179,9 @@ def test_dispatch_plans_are_consistent():
                     elif one or M > 16:
                         assert wgs <= 256 + N // cols or cols == 256     # second pass: about one workgroup per CU
                     if "d3" in name:                                     # three staging buffers
-                        assert one and cps >= 6 and (wgs <= 256 or cols == 256)
+                        assert (one or name == "wide2d3m2") and cps >= 6 and (wgs <= 256 or cols == 256)
                     if cols == 256:
-                        assert 8192 <= N < 28672
+                        assert (8192 if one else 4096) <= N < 28672 and M <= 32
                 if not staged_ok:
                     assert not name.startswith(("dma", "wide"))
                 if g == 128:   # awq_gemv_workspace_bytes takes no group size: it must cover this plan
@@ -231,6 +231,10 @@ def test_dispatch_plans_are_consistent():
     assert rc == 0 and gemv_names[v] == "wide2d3m1" and s == 8
     rc, v, s = _plan(L.awq_gemv_plan, 16, 24576, 4096, 128)      # 96 groups of 256 fill 75 % of the CUs in two splits: 512 columns
     assert rc == 0 and gemv_names[v] == "wided2m1" and s == 5
+    rc, v, s = _plan(L.awq_gemv_plan, 32, 8192, 8192, 128)       # 17..32 rows: 256 columns x two m-tiles, one workgroup per CU
+    assert rc == 0 and gemv_names[v] == "wide2d3m2" and s == 8
+    rc, v, s = _plan(L.awq_gemv_plan, 24, 17408, 5120, 128)      # 68 groups: about 500 workgroups instead
+    assert rc == 0 and gemv_names[v] == "wide2d2m2" and s == 7
     assert gemv_names[_plan(L.awq_gemv_plan, 1, 4096, 16384, 128)[1]] == "dma1x8"      # narrow weights: the one-tile kernel
     assert gemv_names[_plan(L.awq_gemv_plan, 16, 12288, 4096, 128)[1]] == "dma1x4"     # and small ones
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so

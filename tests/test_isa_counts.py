@@ -42,13 +42,17 @@ def test_staged_gemv_issues_each_load_once(tmp_path):
     # The shared-chunk kernel with three staging buffers counts too.  Per issue site a wave runs 4 weight loads, its x
     # load (one m-tile: one piece, brought by waves 0..3) and one of the two zero/scale loads; the two byte-half paths of
     # the kernel keep their own weight loads and share the zero/scale block -- and the x load where only some waves
-    # run it (512 columns: 8 + 1 + 2 instructions per site; 256 columns: 8 + 2 + 2), DEPTH sites.
+    # run it (512 columns: 8 + 1 + 2 instructions per site; 256 columns: 8 + 2 + 2; 256 columns and two m-tiles:
+    # 8 + 4 + 2), DEPTH sites.
     wide = re.findall(r"^(_ZN3awq16gemv_wide_kernel[^:\s]*):", asm, re.M)
-    deep = [n for n in wide if re.search(r"ELi3ELi1ELb[01]ELi[24]E", n)]
-    assert len(deep) == 8, wide               # 2 types x (second pass, in-kernel tail) x (512, 256 columns)
+    deep = [n for n in wide if re.search(r"ELi3ELi[12]ELb[01]ELi[24]E", n)]
+    assert len(deep) == 10, wide              # 2 types x ((second pass, in-kernel tail) x (512, 256 columns) + 256 columns x two m-tiles)
     for name in deep:
         begin = asm.index("\n" + name + ":")
         body = asm[begin:asm.index(".Lfunc_end", begin)]
         loads = len(re.findall(r"\bglobal_load_lds_dword", body))
-        per_site = 11 if re.search(r"ELb[01]ELi4E", name) else 12
+        if re.search(r"ELi3ELi2E", name):      # two m-tiles on 256 columns: two x pieces per wave on either path
+            per_site = 8 + 4 + 2
+        else:
+            per_site = 11 if re.search(r"ELb[01]ELi4E", name) else 12
         assert loads == 3 * per_site, (name, loads)
