@@ -38,7 +38,7 @@ sys.path.insert(0, ROOT)
 # (FETCH_SIZE, then WRITE_SIZE; profiles/gemv_cfg2_sweep_hbm_traffic.txt).  Each counter is scaled by
 # what it reads for a device-to-device copy of 65,536,000 bytes: FETCH_SIZE 32,012.8 -> 2047.2 B per count,
 # WRITE_SIZE 64,000 -> 1024 B per count.
-MEASURED_FETCH_BYTES_PER_LAUNCH = 1128.51 * 2047.2
+MEASURED_FETCH_BYTES_PER_LAUNCH = 1129.27 * 2047.2
 MEASURED_WRITE_BYTES_PER_LAUNCH = 100.68 * 1024.0
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published

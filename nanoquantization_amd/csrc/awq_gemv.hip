@@ -1715,7 +1715,10 @@ static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, 
         *variant = best_d3 ? kWideD3M1T : kWideM1T;
         return best_c;
     }
-    if (N % 256 != 0 || N < 8192 || K * N < (M <= 4 ? (64ll << 20) : 56000000ll)) return 0;
+    if (N % 256 != 0 || K * N < (M <= 4 ? (64ll << 20) : 56000000ll)) return 0;
+    // (narrower weights only from five rows on and 120 M weights: 25600 x 5120 at 16 rows 26.2 -> 24.8 us; at up to
+    // four rows, and on 17408 x 5120 or 16384 x 4096 at any row count, the one-tile kernel is as fast or faster)
+    if (N < 8192 && (N < 5120 || M < 5 || K * N < 120000000ll)) return 0;
     const int64_t groups = N / 256;
     int64_t sa = 512 / groups;
     if (sa > 25) sa = 25;
