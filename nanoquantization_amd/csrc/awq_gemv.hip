@@ -1668,8 +1668,9 @@ static int64_t balance_splits(int64_t chunks, int64_t s, int64_t wk, int64_t cap
 //    us in five splits, 8192 x 28672 33.4 -> 28.6 in four, 5120 x 34816 26.0 -> 24.4 in seven); at three and four rows
 //    only where five splits or fewer do (5120 x 34816 in ten: 27.3 -> 29.9).  5..16 rows: second pass, about one
 //    workgroup per CU (5120 x 51200 at 16 rows 46.2 -> 36.6 us, 5120 x 34816 34.7 -> 28.3, 8192 x 28672 -> 32.2).
-//  * 8192 <= N < 28672 and 64 Mi weights or more (56 M from five rows on: 6144 x 10240 at 8 rows 16.5 -> 14.4 us,
-//    4096 x 14336 15.9 -> 14.1, while at up to four rows both lose 0.5 us): 256 columns per workgroup (four waves).  Plan A: two buffers,
+//  * 8192 <= N < 28672 and 64 Mi weights or more (52 M from five rows, 50 M from nine rows on: 5120 x 10240 at 8 / 16
+//    rows 15.2 / 16.2 -> 13.9 / 14.3 us, 6144 x 10240 at 8 rows 16.5 -> 14.4, while at up to four rows these lose 0.5 us
+//    and 4096 x 12288 at 8 rows 12.4 -> 13.7): 256 columns per workgroup (four waves).  Plan A: two buffers,
 //    about 500 workgroups (two or three share a CU); plan B: about one workgroup per CU (at least 85 % of them),
 //    three buffers if a split has six chunks or more.  Up to eight rows with the tail while rows x splits <= 64 -- A,
 //    or B where A needs eleven splits or more -- (one row: 5120 x 25600 19.9 -> 17.6 us, 5120 x 17408 15.8 -> 14.1,
@@ -1715,13 +1716,14 @@ static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, 
         *variant = best_d3 ? kWideD3M1T : kWideM1T;
         return best_c;
     }
-    if (N % 256 != 0 || K * N < (M <= 4 ? (64ll << 20) : 56000000ll)) return 0;
-    // (narrower weights only from five rows on and 120 M weights: 25600 x 5120 at 16 rows 26.2 -> 24.8 us; at up to
-    // four rows, and on 17408 x 5120 or 16384 x 4096 at any row count, the one-tile kernel is as fast or faster)
-    if (N < 8192 && (N < 5120 || M < 5 || K * N < 120000000ll)) return 0;
+    if (N % 256 != 0 || K * N < (M <= 4 ? (64ll << 20) : (M <= 8 ? 52000000ll : 50000000ll))) return 0;
+    // (40 to 63 column tiles: at one and two rows from 80 M weights on -- 25600 x 5120 22.0 -> 20.3 us, 17408 x 5120
+    // 17.5 -> 16.4 in 20 splits --, from five rows on from 120 M -- 25600 x 5120 at 16 rows 26.2 -> 24.8 us; otherwise, and
+    // on 16384 x 4096 at any row count, the one-tile kernel is as fast or faster)
+    if (N < 8192 && (N < 5120 || (M <= 2 ? K * N < 80000000ll : (M < 5 || K * N < 120000000ll)))) return 0;
     const int64_t groups = N / 256;
     int64_t sa = 512 / groups;
-    if (sa > 25) sa = 25;
+    if (sa > 20) sa = 20;
     if (sa > chunks / 4) sa = chunks / 4;
     if (sa < 2) return 0;
     sa = normalised(sa);
@@ -1731,7 +1733,7 @@ static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, 
     if (b_valid) sb = normalised(sb);
     const bool b_d3 = b_valid && cdiv(chunks, sb) >= 6;
     if (M <= 8) {
-        const bool use_b = b_valid && sa >= 11;
+        const bool use_b = b_valid && sa >= 11 && N >= 8192;
         const int64_t c = use_b ? sb : sa;
         if (M * c <= 64) {
             *variant = use_b ? (b_d3 ? kWide2D3M1T : kWide2D2M1T) : kWide2D2M1T;
@@ -1869,6 +1871,12 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             // 65..128 rows (five to eight blocks of 16, small weights only): the blocks fill the chip, a split only
             // adds its tail (2048 x 2048 at 128 rows: 8.6 us unsplit, 9.4 in two)
             const int64_t cap = M > 64 && wgs >= 64 ? 1 : (chunks / 4 > 1 ? chunks / 4 : 1);
+            // From 17 rows on, weights under 32 Mi elements (16 MB packed: the linears of Qwen3-1.7B / 4B) are not
+            // streaming-bound, and with 150 workgroups or more any split only adds its tail -- 2560 x 9728 at 64 rows
+            // 27.2 us in five splits, 16.8 unsplit (304 workgroups); at 32 rows 16.2 -> 13.1; 2048 x 6144 at 64 rows
+            // 12.3 -> 9.7; likewise four row blocks of 128 tiles or more: 2560 x 19456 at 64 rows 33.4 -> 23.4.
+            const bool unsplit = row_blocks >= 2 && wgs >= 150 &&
+                                 (K * N < (32ll << 20) || (row_blocks >= 4 && wgs >= 512));
             int64_t s0 = wgs < 200 ? cdiv(200, wgs) : 1;
             if (s0 > cap) s0 = cap;
             const int64_t hi = s0 + 5 < cap ? s0 + 5 : cap;
@@ -1888,6 +1896,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
                     s = c;
                 }
             }
+            if (unsplit) s = 1;
         }
         if (s < 1) s = 1;
         *variant = v;

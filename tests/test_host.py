@@ -236,7 +236,7 @@ def test_dispatch_plans_are_consistent():
     rc, v, s = _plan(L.awq_gemv_plan, 24, 17408, 5120, 128)      # 68 groups: about 500 workgroups instead
     assert rc == 0 and gemv_names[v] == "wide2d2m2" and s == 7
     assert gemv_names[_plan(L.awq_gemv_plan, 1, 4096, 16384, 128)[1]] == "dma1x8"      # narrow weights: the one-tile kernel
-    assert gemv_names[_plan(L.awq_gemv_plan, 16, 12288, 4096, 128)[1]] == "dma1x4"     # and small ones
+    assert gemv_names[_plan(L.awq_gemv_plan, 8, 12288, 4096, 128)[1]] == "dma1x4"      # and small ones
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
     # 200 tiles are cut in two (400 workgroups, one round) or five (1000, two full rounds), never in three (600)
     rc, v, s = _plan(L.awq_gemm_plan, 128, 25600, 5120, 128, _lib.AWQ_BF16)
