@@ -1897,6 +1897,17 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
                 }
             }
             if (unsplit) s = 1;
+            // K of 4096..8192: eight-wave workgroups with one chunk per wave (the step-by-step form) where they make
+            // 150..256 workgroups, at most one per CU -- 4096 x 2560 at 32 rows 12.7 -> 9.9 us, 4096 x 8192 at 16 rows
+            // 11.6 -> 10.9, 8192 x 4096 at 8 rows 11.9 -> 10.5, 5120 x 5120 at 8 rows 10.8 -> 10.0; with more
+            // workgroups than that the four-wave split is faster (4096 x 8192 at 32 rows 14.6 against 17.3 us).
+            if (chunks >= 32 && chunks <= 64 && row_blocks <= 2) {
+                const int64_t s8 = cdiv(chunks, 8);
+                if (wgs * s8 >= 150 && wgs * s8 <= 256) {
+                    v = kDma1x8;
+                    s = s8;
+                }
+            }
         }
         if (s < 1) s = 1;
         *variant = v;
