@@ -308,9 +308,11 @@ def main():
             del copies
             torch.cuda.empty_cache()
         out["batched_decode_gemv"] = {
-            "kernel": "awq::gemv_wide_kernel + awq::gemv_wide_reduce_kernel", "unit": "GB/s of packed weights",
+            "kernel": "awq::gemv_wide_kernel + awq::gemv_wide_reduce_kernel (each case names its own form)",
+            "unit": "GB/s of packed weights",
             "note": "17..64 rows (cfg5 decodes at 64): bound by the SIMDs' issue ports (MFMA + unpack + fold + load-to-LDS "
-                    "instructions of two lock-stepped waves per SIMD) plus the K splits' fp32 partial round trip, not by HBM",
+                    "instructions; at 33..64 rows the 244 registers a wave holds leave two waves per SIMD) plus the K "
+                    "splits' fp32 partial round trip, not by HBM",
             "cases": batched}
         best = max(v["GBs"] for v in large.values())
         best_large = max(large, key=lambda k: large[k]["GBs"])

@@ -1160,6 +1160,11 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
     // XP: pieces of x a wave brings per chunk (with one m-tile the four pieces go to waves 0..3, one each);
     // HMT: m-tiles each of the two byte-half waves of a column tile stores at the end
     constexpr int CH = 4, XP = MT >= 2 ? 4 * MT / (2 * WN) : 1, HMT = MT >= 2 ? MT / 2 : 1;
+    // Four m-tiles on 256 columns take a chunk one 32-row step at a time (below): two such workgroups share a CU, one
+    // wave each per SIMD, and a wave that first brings all its loads and then reads the whole chunk from LDS leaves its
+    // SIMD to the other workgroup's wave alone.  (Measured on the other forms too: no gain with eight waves per
+    // workgroup, which pass a barrier per chunk together, nor with two m-tiles, where three waves share a SIMD.)
+    constexpr bool STEP = WN == 2 && MT == 4;
     static_assert(WN == 4 || WN == 2, "512 or 256 columns per workgroup");
     static_assert(DEPTH >= 2 && DEPTH <= 3, "two or three staging buffers");
     static_assert(MT == 1 || MT == 2 || MT == 4, "m-tiles per workgroup");
@@ -1249,6 +1254,36 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
         }
     };
 
+    // STEP: the same loads in four parts, one per 32-row step of the chunk being multiplied (zeros/scales and half the
+    // weights, the other half, then x)
+    auto issue_dma_part = [&](int c, int buf, int part) {
+        const int row0 = c * 128;
+        char* base = stage + buf * buf_bytes;
+        if (part < 2) {
+            uint32_t* w_lds = reinterpret_cast<uint32_t*>(base + w_off);
+            const int s = bh * (CH / 2) + part;
+            const uint32_t* wp = qweight + (size_t)(row0 + s * 32) * words;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                __builtin_amdgcn_global_load_lds(AWQ_GPTR(wp + wsrc[h]), AWQ_LPTR(w_lds + s * 512 + h * 256), 16, 0, 0);
+            if (part == 0 && zs_lane) {
+                const int gi = chunks_per_group == 1 ? c : c / chunks_per_group;
+                if (bh == 0)
+                    __builtin_amdgcn_global_load_lds(AWQ_GPTR(qzeros + (size_t)gi * words + zsrc),
+                                                     AWQ_LPTR(base + zs_off), 4, 0, 0);
+                else
+                    __builtin_amdgcn_global_load_lds(AWQ_GPTR(scales + ((size_t)gi * words + zsrc) * 8),
+                                                     AWQ_LPTR(base + zs_off + 64), 16, 0, 0);
+            }
+        } else if (x_wave) {
+#pragma unroll
+            for (int i = 0; i < XP; ++i)
+                if ((XP == 1 ? 2 : 2 + (i & 1)) == part)
+                    __builtin_amdgcn_global_load_lds(AWQ_GPTR(x + (row0 + x_s[i] * 32) + xsrc[i]),
+                                                     AWQ_LPTR(base + x_s[i] * x_step + x_mt[i] * 1024), 16, 0, 0);
+        }
+    };
+
     const int w_rd_off = w_off + (kb * 16 + j) * 4;
     int x_rd_off[MT];
 #pragma unroll
@@ -1276,9 +1311,78 @@ __global__ __launch_bounds__(128 * WN) void gemv_wide_kernel(
             // in flight too; the LDS itself needs no fence (DMA data is there once vmcnt has counted it).
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (c + DEPTH - 1 < c1) issue_dma(c + DEPTH - 1, buf == 0 ? DEPTH - 1 : buf - 1);
             const char* base = stage + buf * buf_bytes;
             const uint32_t* w_rd = reinterpret_cast<const uint32_t*>(base + w_rd_off);
+            if constexpr (STEP) {
+                // One 32-row step at a time: the LDS reads of step s + 1 and a part of the next chunk's loads go out
+                // before step s is multiplied.  The MFMA chains and the fold are those of compute_chunk_bytes.
+                const bool more = c + DEPTH - 1 < c1;
+                const int nbuf = buf == 0 ? DEPTH - 1 : buf - 1;
+                const u32x4 ones = u32x4{T::ones2, T::ones2, T::ones2, T::ones2};
+                const f32x4 zero4 = f32x4{0.f, 0.f, 0.f, 0.f};
+                const AndOr emb_lo(Embed<T>::kMaskLo, Embed<T>::kMagicLo), emb_hi(Embed<T>::kMaskHi, Embed<T>::kMagicHi);
+                uint32_t w[2][8];
+                u32x4 xa[2][MT];
+                f32x4 dones[MT], dq[2][2][MT];
+                auto lds_step = [&](int s, int slot) {
+#pragma unroll
+                    for (int r = 0; r < 8; ++r) w[slot][r] = w_rd[s * 512 + r * 64];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        xa[slot][mt] = *reinterpret_cast<const u32x4*>(base + x_rd_off[mt] + s * x_step);
+                };
+                lds_step(0, 0);
+                const uint32_t zw = *reinterpret_cast<const uint32_t*>(base + z_rd_off);
+                const u32x4 sv = *reinterpret_cast<const u32x4*>(base + s_rd_off);
+#pragma unroll
+                for (int s = 0; s < CH; ++s) {
+                    if (s + 1 < CH) lds_step(s + 1, (s + 1) & 1);
+                    if (more) issue_dma_part(c + DEPTH - 1, nbuf, s);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) dones[mt] = T::mfma16(xa[s & 1][mt], ones, s ? dones[mt] : zero4);
+#pragma unroll
+                    for (int bi = 0; bi < 2; ++bi) {
+                        const int b = 2 * BH + bi;
+                        u32x4 flo, fhi;
+#pragma unroll
+                        for (int rp = 0; rp < 4; ++rp) {
+                            const uint32_t p = __builtin_amdgcn_perm(w[s & 1][2 * rp + 1], w[s & 1][2 * rp],
+                                                                     0x0c000c00u | (uint32_t)b | ((4u + b) << 16));
+                            flo[rp] = emb_lo(Embed<T>::pre_lo(p));
+                            fhi[rp] = emb_hi(Embed<T>::pre_hi(p));
+                        }
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) {
+                            dq[bi][0][mt] = T::mfma16(xa[s & 1][mt], flo, s ? dq[bi][0][mt] : zero4);
+                            dq[bi][1][mt] = T::mfma16(xa[s & 1][mt], fhi, s ? dq[bi][1][mt] : zero4);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int bi = 0; bi < 2; ++bi) {
+                    constexpr int kLoCol[4] = {0, 4, 1, 5}, kHiCol[4] = {2, 6, 3, 7};
+                    const int b = 2 * BH + bi;
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int col = h ? kHiCol[b] : kLoCol[b];
+                        const float mul = h ? Embed<T>::kMulHi : Embed<T>::kMulLo;
+                        const float off = h ? Embed<T>::kOffHi : Embed<T>::kOffLo;
+                        const float zf = (float)((zw >> nibble_shift(col)) & 0xFu) * mul + off;
+                        const uint32_t pair = sv[col >> 1];
+                        const float sc = T::to_f32((uint16_t)((col & 1) ? (pair >> 16) : (pair & 0xFFFFu))) * (1.f / mul);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                acc[mt][2 * bi + h][r] += sc * (dq[bi][h][mt][r] - zf * dones[mt][r]);
+                    }
+                }
+                buf = (buf + 1 == DEPTH) ? 0 : buf + 1;
+                continue;
+            }
+            if (c + DEPTH - 1 < c1) issue_dma(c + DEPTH - 1, buf == 0 ? DEPTH - 1 : buf - 1);
             Chunk<1, CH, MT> d;
 #pragma unroll
             for (int s = 0; s < CH; ++s) {
@@ -1440,9 +1544,12 @@ static const GemvVariant kGemvVariants[] = {
     // 256 columns, two m-tiles (17..32 rows)
     {"wide2d2m2", 1, 4, false, 2, 2, 2, true},
     {"wide2d3m2", 1, 4, false, 2, 3, 2, true},
+    // 256 columns, four m-tiles (33..64 rows), a chunk taken one 32-row step at a time
+    {"wide2d2m4", 1, 4, false, 2, 2, 4, true},
 };
 enum { kV1W4P = 0, kV2W4 = 1, kDma1x4 = 2, kDma1x8 = 3, kWideM4 = 4, kWideM2 = 5, kWideM1 = 6, kWideM1T = 7,
-       kWideD3M1 = 8, kWideD3M1T = 9, kWide2D2M1 = 10, kWide2D2M1T = 11, kWide2D3M1 = 12, kWide2D3M1T = 13, kWide2D2M2 = 14, kWide2D3M2 = 15 };
+       kWideD3M1 = 8, kWideD3M1T = 9, kWide2D2M1 = 10, kWide2D2M1T = 11, kWide2D3M1 = 12, kWide2D3M1T = 13, kWide2D2M2 = 14, kWide2D3M2 = 15,
+       kWide2D2M4 = 16 };
 constexpr int kNumGemvVariants = sizeof(kGemvVariants) / sizeof(kGemvVariants[0]);
 constexpr int kFirstDmaVariant = kDma1x4;
 
@@ -1757,25 +1864,34 @@ static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, 
 // 24 / 32 rows: 5120 x 17408 27.6 / 28.9 -> 20.3 / 21.8 us, 17408 x 5120 26.5 / 27.0 -> 21.4 / 22.4, 8192 x 8192
 // 22.3 / 22.8 -> 17.0 / 17.8, 5120 x 10240 19.6 / 20.2 -> 16.4 / 16.6, 12288 x 4096 18.5 -> 16.1 / 16.7, 6144 x 8192
 // 17.8 / 18.3 -> 15.6 / 16.4, 5120 x 25600 26.6 / 26.8 -> 25.1; 5120 x 51200 stays with 512 columns (44.6 against
-// 46.6).  With four m-tiles (33..64 rows) the form was measured too and is not used: within 5 % of the 512-column
-// one where it wins (5120 x 10240 at 64 rows 27.3 -> 25.3 us, 5120 x 17408 32.3 -> 31.7), 10..20 % slower with few
-// long splits (8192 x 14336 in four: 43.0 against 37.9).
+// 46.6).
+// 33..64 rows: the same with four m-tiles, 244 registers a wave, so two workgroups a CU and one wave of each per SIMD;
+// the kernel then takes a chunk step by step.  From 45 M weights and 3584 columns on, any N; plan B from 92 % of the
+// CUs and up to 12 chunks a split (with 87 % and 16 chunks 4096 x 28672 runs 38.6 us, 36.9 in 448 workgroups of 8
+// chunks; 25600 x 5120 at 40 rows 37.6 us in 12 splits of 17 chunks, 33.7 in 25 of 8).  Against the
+// 512-column form or the one-tile kernel's row blocks at 64 rows: 8192 x 8192 30.4 -> 26.1 us, 5120 x 10240 27.8 ->
+// 23.7, 13824 x 5120 31.4 -> 27.2, 18944 x 3584 31.6 -> 27.7, 8192 x 10240 33.8 -> 29.9, 4096 x 12288 25.9 -> 23.5,
+// 5120 x 17408 34.1 -> 32.5, 4096 x 28672 39.6 -> 36.9, 5120 x 25600 40.8 -> 39.1, 5120 x 51200 70.7 -> 65.6; at 40
+// and 48 rows equal to 10 % faster (12288 x 4096 at 48 rows 25.0 -> 21.5); 4096 x 8192 and 5120 x 8192 keep the row
+// blocks (17.2 and 19.9 against 22.5 and 21.8).
 static int64_t pick_shared_256(int64_t M, int64_t N, int64_t K, int64_t chunks, int* variant) {
-    if (M > 32 || N % 256 != 0 || chunks < 8 || N < 4096 || N >= 28672 || K * N < 48000000ll) return 0;
+    if (M > 64 || N % 256 != 0 || chunks < 8) return 0;
+    const bool four = M > 32;   // m-tiles: four, else two
+    if (four ? (N < 3584 || K * N < 45000000ll) : (N < 4096 || N >= 28672 || K * N < 48000000ll)) return 0;
     auto normalised = [&](int64_t c) { return cdiv(chunks, cdiv(chunks, c)); };
     const int64_t groups = N / 256;
     int64_t sb = 256 / groups;
     if (sb > chunks / 4) sb = chunks / 4;
-    if (sb >= 2 && normalised(sb) * groups >= 218) {
+    if (sb >= 2 && normalised(sb) * groups >= (four ? 236 : 218) && (!four || cdiv(chunks, sb) <= 12)) {
         sb = normalised(sb);
-        *variant = cdiv(chunks, sb) >= 6 ? kWide2D3M2 : kWide2D2M2;
+        *variant = four ? kWide2D2M4 : (cdiv(chunks, sb) >= 6 ? kWide2D3M2 : kWide2D2M2);
         return sb;
     }
     int64_t sa = 512 / groups;
     if (sa > 25) sa = 25;
     if (sa > chunks / 4) sa = chunks / 4;
     if (sa < 1) return 0;
-    *variant = kWide2D2M2;
+    *variant = four ? kWide2D2M4 : kWide2D2M2;
     return normalised(sa);
 }
 
@@ -1794,7 +1910,7 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
         int64_t m1_splits = 0;
         int m1_variant = 0;
         if (allow_shared_chunk && M <= 16) m1_splits = pick_one_m_tile(M, N, K, chunks, &m1_variant);
-        if (allow_shared_chunk && M > 16 && M <= 32) m1_splits = pick_shared_256(M, N, K, chunks, &m1_variant);
+        if (allow_shared_chunk && M > 16 && M <= 64) m1_splits = pick_shared_256(M, N, K, chunks, &m1_variant);
         if (m1_splits == 0 && allow_shared_chunk && M > 16 && M <= 64 && N % 512 == 0 && N >= 5120 &&
             K * N >= (M > 48 ? (50ll << 20) : (M > 32 ? 64000000ll : 95000000ll))) {
             // 17..64 rows on the largest weights (from sweeps: the fused gate|up of Qwen3-8B and the MLP of
@@ -2031,6 +2147,7 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
             break;
         AWQ_WIDE2M_CASE(kWide2D2M2, 2, 2)
         AWQ_WIDE2M_CASE(kWide2D3M2, 3, 2)
+        AWQ_WIDE2M_CASE(kWide2D2M4, 2, 4)
 #undef AWQ_WIDE2M_CASE
         case kWideD3M1T:
             e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)

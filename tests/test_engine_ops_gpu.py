@@ -231,7 +231,8 @@ def test_silu_mul(dtype, rows, inter):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,inter", [(1, 1024, 3072), (32, 1024, 3072), (16, 2048, 1024), (64, 5120, 1280), (3, 4096, 64),
-                                           (48, 4096, 3072), (24, 8192, 2560)])   # the last two: shared-chunk kernel
+                                           (48, 4096, 3072), (24, 8192, 2560), (64, 8192, 4096), (40, 5120, 8704)])
+# (from 24 rows x 8192 on: the shared-chunk kernel, whose second pass applies the gate)
 def test_gemv_swiglu_equals_unfused(dtype, M, K, inter):
     """Gate and up interleaved + gated epilogue must give, bit for bit, what the plain GEMV over gate|up side by
     side followed by the SiLU*up kernel gives (a column's sum does not depend on where the column sits)."""

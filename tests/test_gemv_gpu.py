@@ -138,11 +138,11 @@ def test_gemv_batched_decode_rows(dtype, M):
 @pytest.mark.parametrize("M,K,N,plan", [(64, 4096, 6144, "dma1x4"), (33, 4096, 6144, "dma1x4"), (24, 8192, 5120, "dma1x4"),
                                         (17, 8192, 5120, "dma1x4"), (24, 8192, 8192, "wide2d3m2/8"),
                                         (32, 5120, 17408, "wide2d2m2/7"), (17, 12288, 4096, "wide2d3m2/16"),
-                                        (64, 5120, 17408, "wided2m4/7"), (32, 4096, 28672, "wided2m2/4")])
+                                        (64, 5120, 17408, "wide2d2m4/7"), (32, 4096, 28672, "wided2m2/4")])
 def test_gemv_batched_decode_rows_large_weights(dtype, M, K, N, plan):
     # 17..64 rows, with a bias: blocks of 16 rows on the one-tile kernel, and on larger weights the shared-chunk kernel
-    # (256 columns x two m-tiles with two or three staging buffers; 512 columns x two or four m-tiles), K split,
-    # second-pass reduction
+    # (256 columns x two m-tiles with two or three staging buffers or x four m-tiles; 512 columns x two m-tiles),
+    # K split, second-pass reduction
     import ctypes
     L = _lib.lib()
     names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
@@ -204,6 +204,39 @@ def test_gemv_shared_chunk_one_m_tile(dtype, M, K, N, plan):
             yv = awq_gemv_variant(xd, *dev, names.index(vn), split)
             check_plain(yv, (vn, split))
             assert torch.equal(yv, awq_gemv_variant(xd, *dev, names.index(vn), split)), (vn, split)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,K,N,plan", [(64, 8192, 8192, "wide2d2m4/8"), (33, 4096, 12288, "wide2d2m4/5"),
+                                        (50, 5120, 17408, "wide2d2m4/7"), (48, 12288, 4096, "wide2d2m4/16")])
+def test_gemv_shared_chunk_four_m_tiles(dtype, M, K, N, plan):
+    """33..64 rows on 45 M weights or more: 256 columns per workgroup, four m-tiles, a chunk taken one 32-row step at
+    a time.  The planned form with a bias against the oracle; forced with other split counts it must give, bit for
+    bit, what the 512-column form gives (the same MFMA chains and the same fold per column), run after run."""
+    import ctypes
+    L = _lib.lib()
+    names = [L.awq_gemv_variant_name(i).decode() for i in range(L.awq_gemv_variant_count())]
+    v, sp = ctypes.c_int(), ctypes.c_int()
+    assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(v), ctypes.byref(sp)) == 0
+    assert f"{names[v.value]}/{sp.value}" == plan
+    print(f"gemv shared-chunk, four m-tiles {dtype} M={M} K={K} N={N}", flush=True)
+    p = random_packed(K, N, 128, dtype, seed=K + N + M)
+    xb = make_x(M, K, dtype, seed=M)
+    bias = np.linspace(-1, 1, N).astype(np.float32)
+    dev = [to_dev(p["qweight"]), to_dev(p["qscales"], dtype), to_dev(p["qzeros"])]
+    from nanoquantization_amd.layers.gemm import _linear
+    bd = to_dev(o.to_bits16(bias, dtype), dtype)
+    xd = to_dev(xb, dtype)
+    y = _linear("awq_linear", xd, *dev, bd)
+    _check(y, xb, p, dtype, o.to_dtype_f32(bias, dtype))
+    assert torch.equal(y, _linear("awq_linear", xd, *dev, bd))
+    new, old = names.index("wide2d2m4"), names.index("wided2m4")
+    for split in (1, 3, sp.value, 25):
+        yv = awq_gemv_variant(xd, *dev, new, split, bias=bd)
+        assert torch.equal(yv, awq_gemv_variant(xd, *dev, old, split, bias=bd)), split
+        assert torch.equal(yv, awq_gemv_variant(xd, *dev, new, split, bias=bd)), split
+        if split == sp.value:
+            assert torch.equal(yv, y)
 
 
 def test_gemv_reference_test_shape():
