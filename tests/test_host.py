@@ -168,7 +168,7 @@ def test_dispatch_plans_are_consistent():
                     assert M <= 16
                 if name.startswith("wide"):
                     cols = 256 if name.startswith("wide2") else 512      # columns per workgroup
-                    assert N % cols == 0 and K * N >= (45000000 if M > 32 else 48000000)
+                    assert N % cols == 0 and K * N >= (40000000 if M > 48 else 45000000 if M > 32 else 48000000)
                     one = name.endswith(("m1", "m1t"))
                     assert one == (M <= 16) and name.endswith("m4") == (M > 32)
                     cps = -(-chunks // s)
@@ -183,7 +183,7 @@ def test_dispatch_plans_are_consistent():
                     if cols == 256 and M <= 32:
                         assert (5120 if one else 4096) <= N < 28672
                     if name == "wide2d2m4":                               # plan B from 92 % of the CUs, else about 500
-                        assert N >= 3584 and ((236 <= wgs <= 256 and cps <= 12) or wgs > 256 or 512 // (N // 256) >= chunks // 4)
+                        assert N >= 3584 and ((216 <= wgs <= 256 and cps <= 12) or wgs > 256 or 512 // (N // 256) >= chunks // 4)
                 if not staged_ok:
                     assert not name.startswith(("dma", "wide"))
                 if g == 128:   # awq_gemv_workspace_bytes takes no group size: it must cover this plan
@@ -243,7 +243,9 @@ def test_dispatch_plans_are_consistent():
     assert rc == 0 and gemv_names[v] == "wide2d2m4" and s == 4
     rc, v, s = _plan(L.awq_gemv_plan, 64, 51200, 5120, 128)      # any N
     assert rc == 0 and gemv_names[v] == "wide2d2m4" and s == 2
-    assert gemv_names[_plan(L.awq_gemv_plan, 64, 8192, 5120, 128)[1]] == "dma1x4"      # below 45 M weights: row blocks
+    assert gemv_names[_plan(L.awq_gemv_plan, 48, 5120, 8192, 128)[1]] == "dma1x4"      # below 45 M weights: row blocks
+    rc, v, s = _plan(L.awq_gemv_plan, 64, 5120, 8192, 128)       # from 40 M at 49..64 rows (four row blocks otherwise)
+    assert rc == 0 and gemv_names[v] == "wide2d2m4" and s == 11
     assert gemv_names[_plan(L.awq_gemv_plan, 1, 4096, 16384, 128)[1]] == "dma1x8"      # narrow weights: the one-tile kernel
     assert gemv_names[_plan(L.awq_gemv_plan, 8, 12288, 4096, 128)[1]] == "dma1x4"      # and small ones
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
