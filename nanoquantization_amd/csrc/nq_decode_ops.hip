@@ -706,9 +706,15 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 int attn_waves(int G) { return G <= 2 ? 16 : (G <= 4 ? 8 : 4); }
 
+// Context splits of a (sequence, kv head) pair.  From sweeps at 1..128 sequences x 512..8000 tokens (bf16, caches
+// larger than the Infinity Cache): the four- and eight-wave workgroups of 8 and 4 query heads per kv head run best at
+// about 2048 waves on the chip, the 16-wave ones at about 4096, with 128 tokens or more per split -- 64 sequences x
+// 8 kv heads x 2060 tokens at 8 heads per kv head 124 us in two splits + merge, 105 unsplit; 16 sequences 46 us in
+// eight, 36 in four; 2 x 8 x 1000 at 4 heads per kv head 16.1 us in sixteen, 12.9 in eight.
 int pick_splits(int64_t batch, int64_t nkv, int64_t max_context, int G) {
-    int64_t s = cdiv(4096, batch * nkv * attn_waves(G));   // about 4096 waves on the chip
-    const int64_t cap = max_context / 64 > 1 ? max_context / 64 : 1;
+    const int64_t waves = attn_waves(G);
+    int64_t s = cdiv(waves >= 16 ? 4096 : 2048, batch * nkv * waves);
+    const int64_t cap = max_context / 128 > 1 ? max_context / 128 : 1;
     s = s > cap ? cap : s;
     s = s > 16 ? 16 : s;
     return (int)(s < 1 ? 1 : s);
