@@ -606,6 +606,196 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_mfma_kernel(
     }
 }
 
+// Both products on the matrix cores, for 128 head dims and block sizes that are multiples of 32 (written for any
+// supported number of query heads per kv head; the launcher uses it at 8).  The kernel above multiplies the probabilities with V on the vector ALU (G x 8
+// FMAs per token and lane), which with 8 heads per kv head costs as much as fetching the cache: cache-resident it
+// still takes 62 of the 102 us it needs from HBM at 64 sequences x 8 kv heads x 2060 tokens.  Here a wave takes
+// tiles of 32 tokens:
+//   scores   S^T = K q^T as above (two 16-token halves, four MFMAs each): a lane ends up with the scores of head
+//            lane % 16 and tokens 4 * (lane / 16) + r of both halves -- which is where the B operand of the second
+//            product wants the probabilities of that head, so they never leave their registers;
+//   values   out^T[dims, heads] = V^T P^T, one MFMA per 16 head dims and tile.  Its A operand needs, per lane, eight
+//            tokens of ONE head dim, but a V row has the dims side by side: the tile is brought to LDS (load-to-LDS,
+//            16 lanes per row) and read back with the transposing LDS read (ds_read_b64_tr_b16: in each group of 16
+//            lanes, lane 4q + c receives element c of the four 8-byte pieces that lanes q, q + 4, q + 8, q + 12 point
+//            at).  Rows sit 256 bytes apart, i.e. on the same banks; each row is therefore stored rotated by its own
+//            index in units of 32 bytes (the load's lanes simply fetch the rotated piece), and the 16 tokens of one
+//            transposing read fall on all 64 banks twice.
+// The online-softmax state (running maximum, rescale factor) is per head and lives in the lanes of that head, which
+// are also the lanes that hold that head's output column: nothing crosses lanes but the maximum.
+// Rows past the context may hold anything: their scores are replaced before the maximum, their probabilities are
+// zero, and their V rows are fetched from the last valid token of the tile (0 x NaN would be NaN).
+#define NQ_GPTR(p) ((__attribute__((address_space(1))) void*)(p))
+#define NQ_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+typedef short nq_s16x4 __attribute__((ext_vector_type(4)));
+
+template <typename T, int G, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_tr_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, const int32_t* __restrict__ context_lens, uint16_t* __restrict__ out,
+    float* __restrict__ partial, int nkv, int block_size, int max_blocks, int num_blocks, int nsplit, float scale) {
+    constexpr int HD = 128, TT = 32, VBYTES = TT * HD * 2, WBYTES = 2 * VBYTES;   // a wave's K tile and V tile
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8, "query heads per kv head");
+    static_assert(G * (HD + 2) * 4 <= WBYTES, "the per-wave results reuse the wave's tiles");
+    const int sp = blockIdx.x % nsplit;
+    const int kvh = (blockIdx.x / nsplit) % nkv;
+    const int b = blockIdx.x / (nsplit * nkv);
+    const int nh = nkv * G;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lo = lane & 15, hi = lane >> 4;
+
+    int ctx = context_lens[b];
+    ctx = ctx < 0 ? 0 : (ctx > max_blocks * block_size ? max_blocks * block_size : ctx);
+    const int per = ((ctx + nsplit - 1) / nsplit + TT - 1) / TT * TT;
+    const int t0 = sp * per, t1 = min(ctx, t0 + per);
+
+    __shared__ __attribute__((aligned(1024))) unsigned char s_raw[WAVES * WBYTES];
+    unsigned char* kt = s_raw + wave * WBYTES;                       // this wave's K tile [32 tokens][256 B, rotated]
+    unsigned char* vt = kt + VBYTES;                                 // and its V tile
+    float (*s_acc)[G][HD + 2] = reinterpret_cast<float (*)[G][HD + 2]>(s_raw);   // after the loop
+
+    u32x4 bq[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bq[i] = u32x4{0u, 0u, 0u, 0u};
+        if (lo < G)
+            bq[i] = *reinterpret_cast<const u32x4*>(q + ((int64_t)b * nh + kvh * G + lo) * HD + 32 * i + 8 * hi);
+    }
+    const float sc = scale * kLog2e;
+    float m = kNegBig, lpart = 0.f;
+    f32x4 acc[8];
+#pragma unroll
+    for (int cb = 0; cb < 8; ++cb) acc[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // load-to-LDS lane roles: instruction k fills rows 4k .. 4k + 3, 16 lanes a row (a whole 256-byte row per 16
+    // lanes: 16 rows x 64 bytes per instruction, the A-operand layout of the score product, moves half as fast).
+    // V: 16-byte position c' of row r holds the row's piece (window (c' / 2 - r) mod 8, half c' % 2); K: position c'
+    // holds piece (c' - r) mod 16, so that the 16 token rows a b128 read of one piece index touches differ in bank.
+    const int dma_row = lane >> 4, dma_piece = lane & 15;
+    // transposing read: as a source, this lane points at token 4 * hi + lo / 4 (+ 16 for the second half), quad lo % 4
+    const int tr_tok = 4 * hi + (lo >> 2), tr_quad = (lo & 3) * 8;
+
+    const int32_t* table = block_table + (int64_t)b * max_blocks;
+    for (int tb = t0 + wave * TT; tb < t1; tb += WAVES * TT) {
+        int blk = table[tb / block_size];                         // wave-uniform
+        blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);
+        const int64_t base = (((int64_t)blk * nkv + kvh) * block_size + tb % block_size) * HD;
+        const int last = min(TT, t1 - tb) - 1;                    // last valid row of the tile
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {   // rows past the context are fetched as they are: their scores are replaced
+            const int r = 4 * k + dma_row;
+            const uint16_t* src = k_cache + base + (int64_t)r * HD + 8 * ((dma_piece - r) & 15);
+            __builtin_amdgcn_global_load_lds(NQ_GPTR(src), NQ_LPTR(kt + k * 1024), 16, 0, 0);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int r = 4 * k + dma_row;
+            const int w = ((dma_piece >> 1) - r) & 7;
+            const uint16_t* src = v_cache + base + (int64_t)min(r, last) * HD + 16 * w + 8 * (dma_piece & 1);
+            __builtin_amdgcn_global_load_lds(NQ_GPTR(src), NQ_LPTR(vt + k * 1024), 16, 0, 0);
+        }
+        // the K tile has landed: a wave's loads return in order, the eight of the V tile are the newest
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        f32x4 st[2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            st[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const int r = 16 * a + lo;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32x4 ka = *reinterpret_cast<const u32x4*>(kt + r * 256 + ((4 * i + hi + r) & 15) * 16);
+                st[a] = T::mfma16(ka, bq[i], st[a]);
+            }
+        }
+        // st[a][r]: head lo, token tb + 16 a + 4 hi + r
+        float sv[2][4], mx = kNegBig;
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                sv[a][r] = (16 * a + 4 * hi + r <= last) ? st[a][r] * sc : kNegBig;
+                mx = fmaxf(mx, sv[a][r]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mn = fmaxf(m, mx);
+        const float c = exp2f(m - mn);
+        m = mn;
+        float pr[2][4], ps = 0.f;
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                pr[a][r] = (16 * a + 4 * hi + r <= last) ? exp2f(sv[a][r] - mn) : 0.f;
+                ps += pr[a][r];
+            }
+        lpart = lpart * c + ps;
+        const u32x4 pb = u32x4{T::pack2(pr[0][0], pr[0][1]), T::pack2(pr[0][2], pr[0][3]),
+                               T::pack2(pr[1][0], pr[1][1]), T::pack2(pr[1][2], pr[1][3])};
+#pragma unroll
+        for (int cb = 0; cb < 8; ++cb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[cb][r] *= c;
+        // the V tile has landed
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int cb = 0; cb < 8; ++cb) {
+            u32x4 vf;
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const int tok = 16 * a + tr_tok;
+                const nq_s16x4 t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (nq_s16x4 __attribute__((address_space(3)))*)(vt + tok * 256 + (((cb + tok) & 7) << 5) + tr_quad));
+                const u32x2 t2 = __builtin_bit_cast(u32x2, t4);
+                vf[2 * a] = t2[0];
+                vf[2 * a + 1] = t2[1];
+            }
+            acc[cb] = T::mfma16(vf, pb, acc[cb]);   // rows: dims 16 cb + 4 hi + r, column: head lo
+        }
+        // the next tile's loads overwrite both tiles: every read of them has returned
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+
+    lpart += __shfl_xor(lpart, 16);
+    lpart += __shfl_xor(lpart, 32);
+    __syncthreads();   // every wave is done with its tiles: the area now holds the per-wave results
+    if (lo < G) {
+#pragma unroll
+        for (int cb = 0; cb < 8; ++cb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s_acc[wave][lo][16 * cb + 4 * hi + r] = acc[cb][r];
+        if (hi == 0) {
+            s_acc[wave][lo][HD] = m;
+            s_acc[wave][lo][HD + 1] = lpart;
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * HD; idx += 64 * WAVES) {
+        const int g = idx / HD, d = idx % HD;
+        float mn = kNegBig;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) mn = fmaxf(mn, s_acc[w][g][HD]);
+        float lt = 0.f, at = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float c = exp2f(s_acc[w][g][HD] - mn);
+            lt += s_acc[w][g][HD + 1] * c;
+            at += s_acc[w][g][d] * c;
+        }
+        const int64_t head = (int64_t)b * nh + kvh * G + g;
+        if (nsplit == 1) {
+            out[head * HD + d] = T::from_f32(lt > 0.f ? at / lt : 0.f);
+        } else {
+            float* dst = partial + (head * nsplit + sp) * (HD + 2);
+            dst[d] = at;
+            if (d == 0) {
+                dst[HD] = mn;
+                dst[HD + 1] = lt;
+            }
+        }
+    }
+}
+
 // Merge of the context splits: one workgroup of HD threads per (sequence, query head).
 template <typename T, int HD>
 __global__ __launch_bounds__(HD) void paged_attn_merge_kernel(const float* __restrict__ partial,
@@ -704,15 +894,21 @@ int bad(const char* fn, const char* what) {
 }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int attn_waves(int G) { return G <= 2 ? 16 : (G <= 4 ? 8 : 4); }
+// The kernel with both products on the matrix cores takes 128 head dims and block sizes that are multiples of 32; it
+// is used at 8 query heads per kv head, where the vector-ALU value product of the other kernels costs the most
+// (bf16, against them: 128 sequences x 8 kv heads x 1024 tokens 120 -> 102 us, 32 x 8 x 512 23.2 -> 19.9, 1 x 8 x 8000
+// 31.7 -> 24.6, 64 x 8 x 2060 the same 102 us = 5.3 TB/s; at 4 and 2 heads per kv head it measured equal or slower:
+// 16 x 8 x 4000 at 4 heads 52.6 -> 55.0 us, the Qwen3-0.6B decode step 1.615 -> 1.673 ms).
+bool attn_tr(int G, int64_t head_dim, int64_t block_size) { return G == 8 && head_dim == 128 && block_size % 32 == 0; }
+int attn_waves(int G, bool tr) { return tr ? 4 : (G <= 2 ? 16 : (G <= 4 ? 8 : 4)); }
 
 // Context splits of a (sequence, kv head) pair.  From sweeps at 1..128 sequences x 512..8000 tokens (bf16, caches
-// larger than the Infinity Cache): the four- and eight-wave workgroups of 8 and 4 query heads per kv head run best at
-// about 2048 waves on the chip, the 16-wave ones at about 4096, with 128 tokens or more per split -- 64 sequences x
-// 8 kv heads x 2060 tokens at 8 heads per kv head 124 us in two splits + merge, 105 unsplit; 16 sequences 46 us in
-// eight, 36 in four; 2 x 8 x 1000 at 4 heads per kv head 16.1 us in sixteen, 12.9 in eight.
-int pick_splits(int64_t batch, int64_t nkv, int64_t max_context, int G) {
-    const int64_t waves = attn_waves(G);
+// larger than the Infinity Cache): four- and eight-wave workgroups run best at about 2048 waves on the chip, the
+// 16-wave ones at about 4096, with 128 tokens or more per split -- 64 sequences x 8 kv heads x 2060 tokens at 8 heads
+// per kv head 124 us in two splits + merge, 105 unsplit; 16 sequences 46 us in eight, 36 in four; 2 x 8 x 1000 at 4
+// heads per kv head 16.1 us in sixteen, 12.9 in eight.
+int pick_splits(int64_t batch, int64_t nkv, int64_t max_context, int G, bool tr) {
+    const int64_t waves = attn_waves(G, tr);
     int64_t s = cdiv(waves >= 16 ? 4096 : 2048, batch * nkv * waves);
     const int64_t cap = max_context / 128 > 1 ? max_context / 128 : 1;
     s = s > cap ? cap : s;
@@ -725,6 +921,17 @@ void launch_attn(const void* q, const void* kc, const void* vc, const int32_t* t
                  float* partial, int64_t batch, int nkv, int bs, int max_blocks, int num_blocks, int nsplit,
                  float scale, hipStream_t st) {
     constexpr int WAVES = G <= 2 ? 16 : (G <= 4 ? 8 : 4);
+    if constexpr (HD == 128 && G == 8) {
+        if (attn_tr(G, HD, bs)) {
+            paged_attn_decode_tr_kernel<T, G, 4><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(256), 0, st>>>(
+                (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, table, ctx, (uint16_t*)out, partial, nkv,
+                bs, max_blocks, num_blocks, nsplit, scale);
+            if (nsplit > 1)
+                paged_attn_merge_kernel<T, HD><<<dim3((unsigned)(batch * nkv * G)), dim3(HD), 0, st>>>(
+                    partial, (uint16_t*)out, nsplit);
+            return;
+        }
+    }
     if constexpr (HD == 128 && (G == 4 || G == 8)) {
         if (bs % 16 == 0) {
             paged_attn_decode_mfma_kernel<T, G, WAVES><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(64 * WAVES), 0, st>>>(
@@ -926,7 +1133,10 @@ extern "C" int nq_qk_norm_rope_store(const void* qkv, const void* q_weight, cons
 extern "C" size_t nq_paged_attention_workspace_bytes(int64_t batch, int64_t num_heads, int64_t num_kv_heads,
                                                      int64_t head_dim, int64_t max_context) {
     if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || max_context <= 0) return 0;
-    const int s = pick_splits(batch, num_kv_heads, max_context, (int)(num_heads / num_kv_heads));
+    // the block size decides the kernel and with it the split count: room for either
+    const int G = (int)(num_heads / num_kv_heads);
+    int s = pick_splits(batch, num_kv_heads, max_context, G, false);
+    if (G == 8 && head_dim == 128) s = std::max(s, pick_splits(batch, num_kv_heads, max_context, G, true));
     return s > 1 ? (size_t)(batch * num_heads * s * (head_dim + 2)) * sizeof(float) : 0;
 }
 
@@ -950,8 +1160,9 @@ extern "C" int nq_paged_attention_decode(const void* q, const void* k_cache, con
     const int64_t max_context = block_size * max_blocks_per_seq;
     if (max_context > 0x7fffffff || num_blocks * block_size > 0x7fffffff || batch * num_kv_heads * 16 > 0x7fffffff)
         return bad(fn, "problem too large");
-    const int nsplit = pick_splits(batch, num_kv_heads, max_context, (int)(num_heads / num_kv_heads));
-    const size_t need = nq_paged_attention_workspace_bytes(batch, num_heads, num_kv_heads, head_dim, max_context);
+    const int nsplit = pick_splits(batch, num_kv_heads, max_context, (int)(num_heads / num_kv_heads),
+                                   attn_tr((int)(num_heads / num_kv_heads), head_dim, block_size));
+    const size_t need = nsplit > 1 ? (size_t)(batch * num_heads * nsplit * (head_dim + 2)) * sizeof(float) : 0;
     if (need && (!workspace || workspace_bytes < need || !aligned16(workspace))) {
         set_error("%s: workspace of %zu bytes needed, %zu given", fn, need, workspace ? workspace_bytes : (size_t)0);
         return AWQ_ERR_WORKSPACE;
