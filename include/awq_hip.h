@@ -155,6 +155,17 @@ int awq_gemv_qkv_rope_store(const void* x, const int32_t* qweight, const void* q
 int awq_gemv_add_residual(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
                           void* residual, float* ssq, int64_t M, int64_t N, int64_t K, int64_t group_size,
                           int dtype, void* workspace, size_t workspace_bytes, void* stream);
+/* awq_gemv_add_rmsnorm: the residual add and the RMSNorm that follow o_proj and down_proj in
+ * Qwen3QuantizedBlock.forward (nanoquantization/models/qwen3_quantized.py:194-215; RMSNorm.add_rms_norm,
+ * nanoquantization/layers/norm.py:34-50) inside the GEMV's second pass: residual [M, N] = dtype(residual +
+ * dtype(x @ W)) in place and normed [M, N] = dtype(dtype(residual * rsqrt(mean(residual^2) + norm_eps)) * norm_weight),
+ * the bits of awq_gemv followed by nq_add_rmsnorm.  Only for problems whose plan (awq_gemv_plan) is a shared-chunk
+ * variant (name "wide...") without the in-kernel tail (no trailing 't') and with split_k > 1, and N <= 8192; others
+ * are refused with AWQ_ERR_UNSUPPORTED and take the two calls.  Workspace as for awq_gemv(M, N, K). */
+int awq_gemv_add_rmsnorm(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                         void* residual, const void* norm_weight, float norm_eps, void* normed, int64_t M, int64_t N,
+                         int64_t K, int64_t group_size, int dtype, void* workspace, size_t workspace_bytes,
+                         void* stream);
 int awq_gemv_rmsnorm(const void* x, const float* ssq, const void* norm_weight, float norm_eps,
                      const int32_t* qweight, const void* qscales, const int32_t* qzeros, void* y, int64_t M,
                      int64_t N, int64_t K, int64_t group_size, int gated, int dtype, void* workspace,

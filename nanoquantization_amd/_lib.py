@@ -43,6 +43,7 @@ SYMBOLS = {
     "awq_linear_swiglu_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "awq_gemv_qkv_rope_store": (_int, [_vp] * 12 + [_i64] * 9 + [ctypes.c_float, _int, _vp, _sz, _vp]),
     "awq_gemv_add_residual": (_int, [_vp] * 6 + [_i64] * 4 + [_int, _vp, _sz, _vp]),
+    "awq_gemv_add_rmsnorm": (_int, [_vp] * 6 + [ctypes.c_float, _vp] + [_i64] * 4 + [_int, _vp, _sz, _vp]),
     "awq_gemv_rmsnorm": (_int, [_vp, _vp, _vp, ctypes.c_float] + [_vp] * 4 + [_i64] * 4 + [_int, _int, _vp, _sz, _vp]),
     "awq_gemv_rmsnorm_qkv_rope_store": (_int, [_vp, _vp, _vp, ctypes.c_float] + [_vp] * 11 + [_i64] * 9 +
                                         [ctypes.c_float, _int, _vp, _sz, _vp]),

@@ -40,6 +40,7 @@
 // through LDS in a fixed order; workgroups of different K-splits publish fp32
 // partials and the last one to arrive (an arrival counter per tile) adds them
 // in split order, so results are bit-stable run to run.
+#include <cstring>
 #include <type_traits>
 
 #include <mutex>
@@ -438,10 +439,18 @@ struct EpiArgs {
 
 // Host side: the optional parts of a launch of the staged kernel (at most one epilogue; the prologue combines
 // with none or with the q|k|v epilogue).
+// The second pass of a K-split shared-chunk GEMV as residual add + RMSNorm: y of the GEMV is the residual stream
+// (updated in place), `normed` receives RMSNorm(residual) * weight.
+struct AddNorm {
+    const uint16_t* weight;
+    uint16_t* normed;
+    float eps;
+};
 struct GemvFusion {
     const QkvEpilogue* qe = nullptr;
     const NormPrologue* np = nullptr;
     const ResidEpilogue* re = nullptr;
+    const AddNorm* an = nullptr;
     bool any() const { return qe || np || re; }
 };
 
@@ -1510,6 +1519,78 @@ __global__ __launch_bounds__(256) void gemv_wide_reduce_kernel(const float* __re
     *reinterpret_cast<u32x4*>(y + (size_t)m * N + n0) = o;
 }
 
+// The second pass and the residual add + RMSNorm that follows an o_proj or down_proj in one: a workgroup per row
+// (N <= 8192: a thread per word), residual[m, :] = T(residual + T(sum of the splits)) in place, normed[m, :] =
+// T(T(residual * rsqrt(mean square + eps)) * weight).  The splits are added as in gemv_wide_reduce_kernel, the
+// sum of squares per 128-column tile and the tiles in index order as in the stand-alone norm kernel: the same bits as
+// the two launches, one of which (with the gap before it) is saved -- at 64 rows x 5120 columns 6.5 + 4.4 us.
+template <typename T>
+__global__ __launch_bounds__(1024) void gemv_wide_reduce_add_rmsnorm_kernel(const float* __restrict__ partials,
+                                                                           uint16_t* __restrict__ residual,
+                                                                           const uint16_t* __restrict__ weight,
+                                                                           uint16_t* __restrict__ normed, int M, int N,
+                                                                           int splits, float eps) {
+    __shared__ float s_tile[64];
+    const int words = N >> 3, tiles = (N + 127) >> 7;
+    const int m = blockIdx.x, wc = threadIdx.x;
+    const bool own = wc < words;
+    const size_t n0 = (size_t)wc * 8;
+    const size_t plane = (size_t)M * N;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    u32x4 wraw = u32x4{0u, 0u, 0u, 0u};
+    if (own) {
+        const u32x4 xraw = *reinterpret_cast<const u32x4*>(residual + (size_t)m * N + n0);
+        wraw = *reinterpret_cast<const u32x4*>(weight + n0);
+        const float* p = partials + (size_t)m * N + n0;
+        f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+            f32x4 a[8], b[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const size_t off = (size_t)min(s0 + u, splits - 1) * plane;
+                a[u] = *reinterpret_cast<const f32x4*>(p + off);
+                b[u] = *reinterpret_cast<const f32x4*>(p + off + 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < splits) {
+                    lo += a[u];
+                    hi += b[u];
+                }
+        }
+        const float sum[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int c = 2 * i + h;
+                const float x = T::to_f32((uint16_t)(h ? (xraw[i] >> 16) : (xraw[i] & 0xFFFFu)));
+                const float d = T::to_f32(T::from_f32(as_f32_result(sum[c])));        // the GEMV's output, rounded
+                v[c] = T::to_f32(T::from_f32(as_f32_result(x + d)));                  // the residual add, rounded
+            }
+            o[i] = (uint32_t)T::from_f32(v[2 * i]) | ((uint32_t)T::from_f32(v[2 * i + 1]) << 16);
+        }
+        *reinterpret_cast<u32x4*>(residual + (size_t)m * N + n0) = o;
+    }
+    const float ts = tile_ssq(v);   // every lane takes part; threads past the row add zeros
+    if ((threadIdx.x & 15) == 0 && (int)(threadIdx.x >> 4) < 64) s_tile[threadIdx.x >> 4] = ts;
+    __syncthreads();
+    float tot = 0.f;
+    for (int t = 0; t < tiles; ++t) tot += s_tile[t];
+    const float r = rsqrtf(tot / (float)N + eps);
+    if (own) {
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float w0 = T::to_f32((uint16_t)(wraw[i] & 0xFFFFu)), w1 = T::to_f32((uint16_t)(wraw[i] >> 16));
+            o[i] = (uint32_t)T::from_f32(mul_round<T>(v[2 * i], r) * w0) |
+                   ((uint32_t)T::from_f32(mul_round<T>(v[2 * i + 1], r) * w1) << 16);
+        }
+        *reinterpret_cast<u32x4*>(normed + (size_t)m * N + n0) = o;
+    }
+}
+
 // ---- host side -------------------------------------------------------------
 struct GemvVariant {
     const char* name;
@@ -1699,7 +1780,8 @@ constexpr int kWideTailRows = 4;   // the default dispatch takes the tail up to 
 template <typename T, int DEPTH, int MT, bool TAIL = false, int WN = 4>
 static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
                                    const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
-                                   int g, void* workspace, int split_k, hipStream_t stream, int act) {
+                                   int g, void* workspace, int split_k, hipStream_t stream, int act,
+                                   const AddNorm* an = nullptr) {
     const int groups = N / (128 * WN);
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
@@ -1710,6 +1792,7 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
     constexpr size_t lds = (size_t)DEPTH * wide_buf_bytes(MT, WN);
     static_assert(lds <= 160 * 1024 - 1024, "staging buffers exceed the LDS");
     static_assert(!TAIL || lds >= 128 * WN * 128, "the tail stages 128 bytes per thread");
+    if (an && (splits == 1 || TAIL)) return hipErrorInvalidValue;   // the second pass is what adds and normalises
     auto kern = gemv_wide_kernel<T, DEPTH, MT, TAIL, WN>;
     static bool raised = false;  // once per process and instantiation
     if (!raised) {
@@ -1726,6 +1809,11 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
                        M, N, K, g / 128, cps, splits, act);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || splits == 1 || TAIL) return e;
+    if (an) {   // (checked by the caller: splits > 1, no tail, no bias, no gate, N <= 8192)
+        hipLaunchKernelGGL(gemv_wide_reduce_add_rmsnorm_kernel<T>, dim3((unsigned)M), dim3(1024), 0, stream, partials,
+                           reinterpret_cast<uint16_t*>(y), an->weight, an->normed, M, N, splits, an->eps);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(gemv_wide_reduce_kernel<T>, dim3((unsigned)cdiv((int64_t)M * (N / 8), 256)), dim3(256), 0, stream, partials,
                        reinterpret_cast<const uint16_t*>(bias), reinterpret_cast<uint16_t*>(y), M, N, splits, act);
     return hipGetLastError();
@@ -2070,6 +2158,15 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
                   "staged kernels only (N %% 128 == 0, group_size %% 128 == 0)", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
+    if (fu.an) {
+        const bool second_pass = variant >= 0 && variant < kNumGemvVariants && kGemvVariants[variant].wide &&
+                                 kGemvVariants[variant].name[strlen(kGemvVariants[variant].name) - 1] != 't';
+        if (!second_pass || split_k < 2 || bias || act || fu.any() || N > 8192 || N % 8 != 0) {
+            set_error("%s: the residual add + RMSNorm second pass needs a K-split shared-chunk plan (see awq_gemv_plan), "
+                      "no bias and N <= 8192", fn);
+            return AWQ_ERR_UNSUPPORTED;
+        }
+    }
     if (M > kGemvMaxRows) {
         set_error("%s: M=%lld is outside the decode regime (1..%d); use awq_gemm", fn, (long long)M, kGemvMaxRows);
         return AWQ_ERR_UNSUPPORTED;
@@ -2120,21 +2217,21 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     const bool f16 = dtype == AWQ_F16;
     switch (variant) {
         case kWideM4:
-            e = f16 ? launch_gemv_wide<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
-                    : launch_gemv_wide<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            e = f16 ? launch_gemv_wide<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
+                    : launch_gemv_wide<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
             break;
         case kWideM1:
-            e = f16 ? launch_gemv_wide<F16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
-                    : launch_gemv_wide<BF16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            e = f16 ? launch_gemv_wide<F16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
+                    : launch_gemv_wide<BF16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
             break;
         case kWideM1T:
-            e = f16 ? launch_gemv_wide<F16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
-                    : launch_gemv_wide<BF16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            e = f16 ? launch_gemv_wide<F16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
+                    : launch_gemv_wide<BF16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
             break;
 #define AWQ_WIDE2_CASE(ID, DD, TT)                                                                                      \
         case ID:                                                                                                        \
-            e = f16 ? launch_gemv_wide<F16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act) \
-                    : launch_gemv_wide<BF16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act); \
+            e = f16 ? launch_gemv_wide<F16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an) \
+                    : launch_gemv_wide<BF16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an); \
             break;
         AWQ_WIDE2_CASE(kWide2D2M1, 2, false)
         AWQ_WIDE2_CASE(kWide2D2M1T, 2, true)
@@ -2143,24 +2240,24 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
 #undef AWQ_WIDE2_CASE
 #define AWQ_WIDE2M_CASE(ID, DD, MM)                                                                                     \
         case ID:                                                                                                        \
-            e = f16 ? launch_gemv_wide<F16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act) \
-                    : launch_gemv_wide<BF16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act); \
+            e = f16 ? launch_gemv_wide<F16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an) \
+                    : launch_gemv_wide<BF16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an); \
             break;
         AWQ_WIDE2M_CASE(kWide2D2M2, 2, 2)
         AWQ_WIDE2M_CASE(kWide2D3M2, 3, 2)
         AWQ_WIDE2M_CASE(kWide2D2M4, 2, 4)
 #undef AWQ_WIDE2M_CASE
         case kWideD3M1T:
-            e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
-                    : launch_gemv_wide<BF16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
+                    : launch_gemv_wide<BF16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
             break;
         case kWideD3M1:
-            e = f16 ? launch_gemv_wide<F16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
-                    : launch_gemv_wide<BF16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            e = f16 ? launch_gemv_wide<F16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
+                    : launch_gemv_wide<BF16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
             break;
         case kWideM2:
-            e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act)
-                    : launch_gemv_wide<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act);
+            e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
+                    : launch_gemv_wide<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
             break;
         case kDma1x4:
             e = f16 ? launch_gemv_dma<F16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, pf, fu)
@@ -2377,6 +2474,24 @@ extern "C" int awq_gemv_add_residual(const void* x, const int32_t* qweight, cons
     if (K >= 32 && N >= 8 && group_size > 0) awq::pick_gemv(M, N, K, group_size, &v, &s, false);
     awq::GemvFusion fu;
     fu.re = &re;
+    return awq::gemv_dispatch(fn, x, qweight, qscales, qzeros, nullptr, residual, M, N, K, group_size, dtype,
+                              workspace, workspace_bytes, stream, v, s, 0, fu);
+}
+
+extern "C" int awq_gemv_add_rmsnorm(const void* x, const int32_t* qweight, const void* qscales, const int32_t* qzeros,
+                                    void* residual, const void* norm_weight, float norm_eps, void* normed, int64_t M,
+                                    int64_t N, int64_t K, int64_t group_size, int dtype, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    const char* fn = "awq_gemv_add_rmsnorm";
+    if (!norm_weight || !normed || ((reinterpret_cast<uintptr_t>(norm_weight) | reinterpret_cast<uintptr_t>(normed)) & 15u)) {
+        awq::set_error("%s: norm_weight and normed must be 16-byte aligned device pointers", fn);
+        return awq::fail_drop(AWQ_ERR_INVALID_ARG);
+    }
+    int v = 0, s = 1;
+    if (K >= 32 && N >= 8 && group_size > 0 && M >= 1) awq::pick_gemv(M, N, K, group_size, &v, &s);
+    awq::AddNorm an{reinterpret_cast<const uint16_t*>(norm_weight), reinterpret_cast<uint16_t*>(normed), norm_eps};
+    awq::GemvFusion fu;
+    fu.an = &an;
     return awq::gemv_dispatch(fn, x, qweight, qscales, qzeros, nullptr, residual, M, N, K, group_size, dtype,
                               workspace, workspace_bytes, stream, v, s, 0, fu);
 }

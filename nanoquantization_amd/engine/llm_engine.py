@@ -102,6 +102,13 @@ class LLMEngine:
         hidden = q0.in_features
         self.norm_fused_ok = (fuse_norm and self.qkv_fused_ok and self.swiglu_ok and hidden % 128 == 0
                               and (max_batch <= 16 or 2 * self.inter * hidden < (50 << 20)))
+        # in the plain decode step: the residual add + RMSNorm after o_proj / down_proj inside the GEMV's second pass,
+        # where that GEMV has one at this batch (the large models at 33..64 rows)
+        o0, d0 = layers[0].self_attn.o_proj, layers[0].mlp.down_proj
+        self.o_add_norm = o0.bias is None and ops.gemv_add_rmsnorm_supported(
+            max_batch, o0.out_features, o0.in_features, o0.group_size)
+        self.down_add_norm = d0.bias is None and ops.gemv_add_rmsnorm_supported(
+            max_batch, d0.out_features, d0.in_features, d0.group_size)
         self.use_graph = use_graph
         self._graph = None
         B, dev = max_batch, self.device
@@ -229,11 +236,16 @@ class LLMEngine:
             self._finish_step(ops.add_rmsnorm(x, None, m.norm.weight, m.norm.eps))
             return
         x = m.embed_tokens(self.s_ids)                                   # residual stream [B, hidden]
-        delta = None
+
+        def lin_add_norm(lin, fused, inp, w, e):   # x += lin(inp) in place; returns RMSNorm(x) * w
+            if fused:
+                return ops.awq_gemv_add_rmsnorm(inp, lin.qweight, lin.qscales, lin.qzeros, x, w, e)
+            return ops.add_rmsnorm(x, lin(inp), w, e)
+
+        h = ops.add_rmsnorm(x, None, m.layers[0].input_layernorm.weight, eps)
         for li, layer in enumerate(m.layers):
             attn = layer.self_attn
             gu = self.gate_up_il[li][:2] if self.swiglu_ok else (self.gate_up[li].qweight, self.gate_up[li].qscales)
-            h = ops.add_rmsnorm(x, delta, layer.input_layernorm.weight, eps)
             # every AWQ launch also pulls the next launch's packed weights and scales towards the Infinity Cache
             # (the small zero-point tensor measured as a net loss)
             prefetch_hint(attn.o_proj.qweight, attn.o_proj.qscales)
@@ -248,15 +260,16 @@ class LLMEngine:
                                            self.nh, self.nkv, self.hd, attn.q_norm.eps)
             o = ops.paged_attention_decode(q, self.cache.k[li], self.cache.v[li], self.s_table, ctx, self.scale)
             prefetch_hint(*gu)
-            h = ops.add_rmsnorm(x, attn.o_proj(o), layer.post_attention_layernorm.weight, eps)
+            h = lin_add_norm(attn.o_proj, self.o_add_norm, o, layer.post_attention_layernorm.weight, eps)
             prefetch_hint(layer.mlp.down_proj.qweight, layer.mlp.down_proj.qscales)
             act = (ops.awq_linear_swiglu(h, *self.gate_up_il[li]) if self.swiglu_ok
                    else ops.silu_mul(self.gate_up[li](h)))
             if li + 1 < nl:
                 nq_ = self.qkv[li + 1]
                 prefetch_hint(nq_.qweight, nq_.qscales)
-            delta = layer.mlp.down_proj(act)
-        self._finish_step(ops.add_rmsnorm(x, delta, m.norm.weight, m.norm.eps))
+            nw, ne = (m.layers[li + 1].input_layernorm.weight, eps) if li + 1 < nl else (m.norm.weight, m.norm.eps)
+            h = lin_add_norm(layer.mlp.down_proj, self.down_add_norm, act, nw, ne)
+        self._finish_step(h)
 
     def _finish_step(self, h: torch.Tensor) -> None:
         nxt = ops.argmax_rows(self.model.lm_head(h))

@@ -152,6 +152,39 @@ def awq_gemv_add_residual(x: torch.Tensor, qweight: torch.Tensor, qscales: torch
                                                     _lib.dtype_id(x.dtype), ws, ws_bytes, stream))
 
 
+def gemv_add_rmsnorm_supported(M: int, N: int, K: int, group_size: int) -> bool:
+    """Whether awq_gemv_add_rmsnorm takes this problem: its GEMV plan is a shared-chunk variant whose K splits a
+    second pass adds (that pass is what does the residual add and the norm), and N <= 8192."""
+    import ctypes
+    L = _lib.lib()
+    v, s = ctypes.c_int(-1), ctypes.c_int(-1)
+    if N > 8192 or N % 128 or L.awq_gemv_plan(M, N, K, group_size, ctypes.byref(v), ctypes.byref(s)) != 0:
+        return False
+    name = L.awq_gemv_variant_name(v.value).decode()
+    return name.startswith("wide") and not name.endswith("t") and s.value > 1
+
+
+def awq_gemv_add_rmsnorm(x: torch.Tensor, qweight: torch.Tensor, qscales: torch.Tensor, qzeros: torch.Tensor,
+                         residual: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """residual [M <= 64, N] += x @ W IN PLACE and returns RMSNorm(residual) * norm_weight: a linear, the residual add
+    and the norm that follow it in a Qwen3 block, the last two inside the GEMV's second pass (the bits of the three
+    separate launches).  Only where gemv_add_rmsnorm_supported."""
+    dev = _dev(x, qweight, qscales, qzeros, residual, norm_weight)
+    M, K = x.shape
+    N = qscales.shape[1]
+    g = K // qscales.shape[0]
+    assert qweight.shape == (K, N // 8) and qzeros.shape == (K // g, N // 8) and x.dtype == qscales.dtype
+    assert residual.shape == (M, N) and residual.dtype == x.dtype and residual.is_contiguous()
+    assert norm_weight.shape == (N,) and norm_weight.dtype == x.dtype
+    out = torch.empty_like(residual)
+    with _lib.on_device(dev):
+        ws, ws_bytes, stream = _gemv_ws(dev, M, N, K)
+        _lib.check(_lib.lib().awq_gemv_add_rmsnorm(x.data_ptr(), qweight.data_ptr(), qscales.data_ptr(), qzeros.data_ptr(),
+                                                   residual.data_ptr(), norm_weight.data_ptr(), eps, out.data_ptr(), M, N,
+                                                   K, g, _lib.dtype_id(x.dtype), ws, ws_bytes, stream))
+    return out
+
+
 def awq_gemv_rmsnorm(x: torch.Tensor, ssq: torch.Tensor, norm_weight: torch.Tensor, eps: float, qweight: torch.Tensor,
                      qscales: torch.Tensor, qzeros: torch.Tensor, gated: bool = False) -> torch.Tensor:
     """(RMSNorm(x) * norm_weight) @ W for the residual stream x [M <= 64, K] with its statistics ssq [K / 128, M];

@@ -370,6 +370,36 @@ def test_gemv_add_residual_equals_unfused(dtype, M, K, N):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,N", [(64, 8192, 5120), (64, 25600, 5120), (33, 12288, 4096), (17, 12288, 4096),
+                                   (64, 8192, 8192), (48, 16384, 3584)])
+def test_gemv_add_rmsnorm_equals_unfused(dtype, M, K, N):
+    """The residual add and the RMSNorm after o_proj / down_proj inside the second pass of a K-split shared-chunk
+    GEMV (Qwen3-32B and 8B shapes at 17..64 rows) against the GEMV, then the add + norm kernel: residual stream and
+    normalised output bit for bit, twice in a row; shapes without such a plan are refused."""
+    import nanoquantization_amd as nq
+    from nanoquantization_amd import _lib
+    from nanoquantization_amd.engine import ops
+    g = torch.Generator(device="cuda").manual_seed(M * 11 + K + N)
+    qw, qs, qz = _packed(K, N, dtype, g)
+    x = (torch.randn(M, K, device="cuda", generator=g) * 0.3).to(dtype)
+    res = torch.randn(M, N, device="cuda", generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(N, device="cuda", generator=g)).to(dtype)
+    print(f"gemv_add_rmsnorm M={M} K={K} N={N} {dtype}", flush=True)
+    assert ops.gemv_add_rmsnorm_supported(M, N, K, 128)
+    want_res = res.clone()
+    want = ops.add_rmsnorm(want_res, nq.awq_gemm(x, qw, qs, qz, 8), w, 1e-6)     # updates `want_res` in place
+    for _ in range(2):
+        got_res = res.clone()
+        got = ops.awq_gemv_add_rmsnorm(x, qw, qs, qz, got_res, w, 1e-6)
+        assert torch.equal(got_res, want_res)
+        assert torch.equal(got, want)
+    # one row on the same weight: the in-kernel tail or the one-tile kernel, no second pass to put the norm in
+    assert not ops.gemv_add_rmsnorm_supported(1, N, K, 128)
+    with pytest.raises(_lib.AwqHipError, match="second pass"):
+        ops.awq_gemv_add_rmsnorm(x[:1].contiguous(), qw, qs, qz, res[:1].clone(), w, 1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,N,gated", [(1, 1024, 4096, False), (32, 1024, 6144, True), (16, 2048, 2048, True),
                                          (64, 1024, 4096, False), (7, 5120, 1280, True), (40, 4096, 512, False)])
 def test_gemv_rmsnorm_equals_unfused(dtype, M, K, N, gated):
