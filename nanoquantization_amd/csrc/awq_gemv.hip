@@ -1591,6 +1591,39 @@ __global__ __launch_bounds__(1024) void gemv_wide_reduce_add_rmsnorm_kernel(cons
     }
 }
 
+// The second pass with the q|k|v epilogue of awq_gemv_qkv_rope_store: a thread owns one word of one row as in
+// gemv_wide_reduce_kernel, the 16 threads of a head call qkv_rope_store together (N % 128 == 0: a head never
+// straddles a row, M * N / 8 is a multiple of 16).
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_wide_reduce_qkv_kernel(const float* __restrict__ partials, int M, int N,
+                                                                   int splits, QkvEpilogue qe) {
+    const int words = N >> 3;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= M * words) return;   // whole groups of 16 threads
+    const int m = idx / words, wc = idx - m * words;
+    const size_t n0 = (size_t)wc * 8;
+    const size_t plane = (size_t)M * N;
+    const float* p = partials + (size_t)m * N + n0;
+    f32x4 lo = f32x4{0.f, 0.f, 0.f, 0.f}, hi = lo;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        f32x4 a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const size_t off = (size_t)min(s0 + u, splits - 1) * plane;
+            a[u] = *reinterpret_cast<const f32x4*>(p + off);
+            b[u] = *reinterpret_cast<const f32x4*>(p + off + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (s0 + u < splits) {
+                lo += a[u];
+                hi += b[u];
+            }
+    }
+    const float out[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    qkv_rope_store<T>(out, m, n0, true, qe);
+}
+
 // ---- host side -------------------------------------------------------------
 struct GemvVariant {
     const char* name;
@@ -1781,7 +1814,7 @@ template <typename T, int DEPTH, int MT, bool TAIL = false, int WN = 4>
 static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const void* qscales,
                                    const int32_t* qzeros, const void* bias, void* y, int M, int N, int K,
                                    int g, void* workspace, int split_k, hipStream_t stream, int act,
-                                   const AddNorm* an = nullptr) {
+                                   const AddNorm* an = nullptr, const QkvEpilogue* qe = nullptr) {
     const int groups = N / (128 * WN);
     const int total_chunks = K / 128;
     const int cps = (int)cdiv(total_chunks, split_k);
@@ -1792,7 +1825,7 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
     constexpr size_t lds = (size_t)DEPTH * wide_buf_bytes(MT, WN);
     static_assert(lds <= 160 * 1024 - 1024, "staging buffers exceed the LDS");
     static_assert(!TAIL || lds >= 128 * WN * 128, "the tail stages 128 bytes per thread");
-    if (an && (splits == 1 || TAIL)) return hipErrorInvalidValue;   // the second pass is what adds and normalises
+    if ((an || qe) && (splits == 1 || TAIL)) return hipErrorInvalidValue;   // their work is the second pass's
     auto kern = gemv_wide_kernel<T, DEPTH, MT, TAIL, WN>;
     static bool raised = false;  // once per process and instantiation
     if (!raised) {
@@ -1809,6 +1842,11 @@ static hipError_t launch_gemv_wide(const void* x, const int32_t* qweight, const 
                        M, N, K, g / 128, cps, splits, act);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || splits == 1 || TAIL) return e;
+    if (qe) {
+        hipLaunchKernelGGL(gemv_wide_reduce_qkv_kernel<T>, dim3((unsigned)cdiv((int64_t)M * (N / 8), 256)), dim3(256), 0,
+                           stream, partials, M, N, splits, *qe);
+        return hipGetLastError();
+    }
     if (an) {   // (checked by the caller: splits > 1, no tail, no bias, no gate, N <= 8192)
         hipLaunchKernelGGL(gemv_wide_reduce_add_rmsnorm_kernel<T>, dim3((unsigned)M), dim3(1024), 0, stream, partials,
                            reinterpret_cast<uint16_t*>(y), an->weight, an->normed, M, N, splits, an->eps);
@@ -2152,16 +2190,21 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
         set_error("%s: inconsistent epilogue arguments", fn);
         return AWQ_ERR_INVALID_ARG;
     }
-    if (fu.any() && (variant < kFirstDmaVariant || variant >= kNumGemvVariants || kGemvVariants[variant].wide ||
-                     kGemvVariants[variant].wn != 1)) {
+    // the q|k|v epilogue also runs in the second pass of a K-split shared-chunk plan (no norm prologue there)
+    const bool wide_second_pass = variant >= 0 && variant < kNumGemvVariants && kGemvVariants[variant].wide &&
+                                  kGemvVariants[variant].name[strlen(kGemvVariants[variant].name) - 1] != 't' &&
+                                  split_k >= 2;
+    const bool qkv_second_pass = fu.qe && !fu.np && !fu.re && wide_second_pass && N % 128 == 0;
+    const int wide_act = qkv_second_pass ? 0 : act;   // the main kernel of such a launch only writes partials
+    if (fu.any() && !qkv_second_pass &&
+        (variant < kFirstDmaVariant || variant >= kNumGemvVariants || kGemvVariants[variant].wide ||
+         kGemvVariants[variant].wn != 1)) {
         set_error("%s: the q|k|v / residual epilogues and the RMSNorm prologue run on the one-tile-per-workgroup "
                   "staged kernels only (N %% 128 == 0, group_size %% 128 == 0)", fn);
         return AWQ_ERR_UNSUPPORTED;
     }
     if (fu.an) {
-        const bool second_pass = variant >= 0 && variant < kNumGemvVariants && kGemvVariants[variant].wide &&
-                                 kGemvVariants[variant].name[strlen(kGemvVariants[variant].name) - 1] != 't';
-        if (!second_pass || split_k < 2 || bias || act || fu.any() || N > 8192 || N % 8 != 0) {
+        if (!wide_second_pass || bias || act || fu.any() || N > 8192 || N % 8 != 0) {
             set_error("%s: the residual add + RMSNorm second pass needs a K-split shared-chunk plan (see awq_gemv_plan), "
                       "no bias and N <= 8192", fn);
             return AWQ_ERR_UNSUPPORTED;
@@ -2217,21 +2260,21 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
     const bool f16 = dtype == AWQ_F16;
     switch (variant) {
         case kWideM4:
-            e = f16 ? launch_gemv_wide<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
-                    : launch_gemv_wide<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
+            e = f16 ? launch_gemv_wide<F16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe)
+                    : launch_gemv_wide<BF16, 2, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe);
             break;
         case kWideM1:
-            e = f16 ? launch_gemv_wide<F16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
-                    : launch_gemv_wide<BF16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
+            e = f16 ? launch_gemv_wide<F16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe)
+                    : launch_gemv_wide<BF16, 2, 1>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe);
             break;
         case kWideM1T:
-            e = f16 ? launch_gemv_wide<F16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
-                    : launch_gemv_wide<BF16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
+            e = f16 ? launch_gemv_wide<F16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe)
+                    : launch_gemv_wide<BF16, 2, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe);
             break;
 #define AWQ_WIDE2_CASE(ID, DD, TT)                                                                                      \
         case ID:                                                                                                        \
-            e = f16 ? launch_gemv_wide<F16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an) \
-                    : launch_gemv_wide<BF16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an); \
+            e = f16 ? launch_gemv_wide<F16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe) \
+                    : launch_gemv_wide<BF16, DD, 1, TT, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe); \
             break;
         AWQ_WIDE2_CASE(kWide2D2M1, 2, false)
         AWQ_WIDE2_CASE(kWide2D2M1T, 2, true)
@@ -2240,24 +2283,24 @@ static int gemv_dispatch(const char* fn, const void* x, const int32_t* qweight, 
 #undef AWQ_WIDE2_CASE
 #define AWQ_WIDE2M_CASE(ID, DD, MM)                                                                                     \
         case ID:                                                                                                        \
-            e = f16 ? launch_gemv_wide<F16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an) \
-                    : launch_gemv_wide<BF16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an); \
+            e = f16 ? launch_gemv_wide<F16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe) \
+                    : launch_gemv_wide<BF16, DD, MM, false, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe); \
             break;
         AWQ_WIDE2M_CASE(kWide2D2M2, 2, 2)
         AWQ_WIDE2M_CASE(kWide2D3M2, 3, 2)
         AWQ_WIDE2M_CASE(kWide2D2M4, 2, 4)
 #undef AWQ_WIDE2M_CASE
         case kWideD3M1T:
-            e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
-                    : launch_gemv_wide<BF16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
+            e = f16 ? launch_gemv_wide<F16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe)
+                    : launch_gemv_wide<BF16, 3, 1, true>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe);
             break;
         case kWideD3M1:
-            e = f16 ? launch_gemv_wide<F16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
-                    : launch_gemv_wide<BF16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
+            e = f16 ? launch_gemv_wide<F16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe)
+                    : launch_gemv_wide<BF16, 3, 1, false>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe);
             break;
         case kWideM2:
-            e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an)
-                    : launch_gemv_wide<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, fu.an);
+            e = f16 ? launch_gemv_wide<F16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe)
+                    : launch_gemv_wide<BF16, 2, 2>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, wide_act, fu.an, fu.qe);
             break;
         case kDma1x4:
             e = f16 ? launch_gemv_dma<F16, 4>(x, qweight, qscales, qzeros, bias, y, Mi, Ni, Ki, gi, workspace, split_k, s, act, pf, fu)
@@ -2402,7 +2445,18 @@ static int qkv_rope_store_entry(const char* fn, const void* x, const NormPrologu
     qe.num_slots = num_slots;
     qe.eps = eps;
     int v = 0, s = 1;
-    if (K >= 32 && N >= 8 && group_size > 0) pick_gemv(M, N, K, group_size, &v, &s, false);
+    if (K >= 32 && N >= 8 && group_size > 0) {
+        // From 17 rows on, where the plain GEMV of this weight is a K-split shared-chunk launch, the epilogue runs in
+        // its second pass (Qwen3-32B q|k|v, 5120 x 10240, at 64 rows: 32.4 us in four blocks of 16 rows on the
+        // one-tile kernel); with the norm prologue and below, the one-tile kernels.
+        bool second_pass = false;
+        if (!np && M > 16) {
+            pick_gemv(M, N, K, group_size, &v, &s, true);
+            const char* name = kGemvVariants[v].name;
+            second_pass = kGemvVariants[v].wide && name[strlen(name) - 1] != 't' && s >= 2;
+        }
+        if (!second_pass) pick_gemv(M, N, K, group_size, &v, &s, false);
+    }
     GemvFusion fu;
     fu.qe = &qe;
     fu.np = np;

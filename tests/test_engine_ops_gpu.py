@@ -93,11 +93,13 @@ def test_qk_norm_rope_store(dtype, nh, nkv, hd):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,nh,nkv", [(1, 1024, 16, 8), (32, 1024, 16, 8), (64, 1024, 16, 8), (5, 3072, 4, 2),
-                                        (40, 5120, 64, 8), (16, 2048, 8, 8)])
+                                        (40, 5120, 64, 8), (16, 2048, 8, 8), (64, 5120, 64, 8), (24, 5120, 64, 8),
+                                        (16, 5120, 64, 8), (33, 4096, 32, 8)])
 def test_gemv_qkv_rope_store_equals_unfused(dtype, M, K, nh, nkv):
-    """Projection + q/k norm + rotary + cache write in one launch against the GEMV followed by the stand-alone
-    kernel: bit for bit (same summation order and rounding points), except where the plain projection runs another
-    kernel with another summation order."""
+    """Projection + q/k norm + rotary + cache write in one launch (the epilogue of the one-tile kernel or, from 17
+    rows on the largest weights, of the shared-chunk kernel's second pass) against the GEMV followed by the
+    stand-alone kernel: bit for bit (same summation order and rounding points), except where the plain projection
+    runs another kernel with another summation order (up to 16 rows on the largest weights)."""
     import nanoquantization_amd as nq
     from nanoquantization_amd.engine import ops
     from nanoquantization_amd.layers.rope import RoPE
@@ -123,8 +125,15 @@ def test_gemv_qkv_rope_store_equals_unfused(dtype, M, K, nh, nkv):
     kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
     q2 = ops.qk_norm_rope_store(nq.awq_gemm(x, qw, qs, qz, 8), nqw, nkw, rope.cos_sin_cache, pos, slots, kc2, vc2,
                                 nh, nkv, hd, 1e-6)
-    if M > 32 and K * N >= 50 << 20:
-        # the plain projection runs the shared-chunk kernel here: another sum order
+    import ctypes
+    from nanoquantization_amd import _lib
+    L = _lib.lib()
+    pv, ps = ctypes.c_int(), ctypes.c_int()
+    assert L.awq_gemv_plan(M, N, K, 128, ctypes.byref(pv), ctypes.byref(ps)) == 0
+    plan = L.awq_gemv_variant_name(pv.value).decode()
+    if plan.startswith("wide") and (M <= 16 or plan.endswith("t") or ps.value < 2):
+        # the plain projection runs a shared-chunk kernel whose form the fused entry point does not take: another sum order
+        assert (M, K) == (16, 5120)
         _close(vc, vc2.float(), dtype, what="v cache")
         _close(q, q2.float(), dtype, what="q")
         _close(kc, kc2.float(), dtype, what="k cache")
