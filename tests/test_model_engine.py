@@ -318,6 +318,28 @@ def test_engine_qwen3_32b_widths_batch_64_context_2048():
 
 
 @pytest.mark.gpu
+def test_engine_qwen3_8b_widths_batch_64():
+    """Two blocks at the Qwen3-8B widths (hidden 4096, 32 query / 8 kv heads, intermediate 12288) with 64 rows: here
+    only down_proj (12288 x 4096) and gate|up have a K-split shared-chunk plan, so the decode step mixes the routes --
+    q|k|v on the one-tile kernel with its own epilogue, o_proj followed by the stand-alone add + norm kernel,
+    down_proj with the add + norm in its second pass, attention at 4 query heads per kv head."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+    print("engine: Qwen3-8B widths, 2 layers, batch 64", flush=True)
+    cfg = dict(QWEN3_32B, hidden_size=4096, intermediate_size=12288, total_num_heads=32, total_num_kv_heads=8,
+               num_hidden_layers=2, max_position_embeddings=1024, vocab_size=32000)
+    model = random_awq_qwen3(cfg, seed=41, std=0.02)
+    torch.manual_seed(42)
+    plen, new = 200, 4
+    prompts = torch.randint(0, cfg["vocab_size"], (64, plen)).tolist()
+    eng = LLMEngine(model, max_batch=64, max_seq_len=plen + 56, block_size=64, use_graph=True)
+    assert eng.down_add_norm and not eng.o_add_norm and not eng.norm_fused_ok
+    got = eng.generate(prompts, new)
+    assert len(got) == 64 and all(len(g) == new for g in got)
+    _teacher_forced_check(model, prompts, got, rows=[0, 21, 63])
+
+
+@pytest.mark.gpu
 def test_engine_mixed_decode_and_long_prefill_qwen3_32b_widths():
     """The mixed run of the largest configuration in miniature: two blocks at the Qwen3-32B widths, one serve() call in
     which eight rows decode at a context of 1,024 and more while a longer request (1,536 tokens) waits, is admitted
