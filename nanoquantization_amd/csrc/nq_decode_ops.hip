@@ -606,8 +606,10 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_mfma_kernel(
     }
 }
 
-// Both products on the matrix cores, for 128 head dims and block sizes that are multiples of 32 (written for any
-// supported number of query heads per kv head; the launcher uses it at 8).  The kernel above multiplies the probabilities with V on the vector ALU (G x 8
+// Both products on the matrix cores, for 128 head dims and block sizes that are multiples of 32.  The query heads of
+// a kv head are columns of a 16-column MFMA tile, so any count up to 16 fits: G > 0 fixes it at compile time (the
+// launcher uses 8), G = 0 takes it from `heads_per_kv` -- the route of the head ratios the other kernels have no
+// instantiation for (Qwen3-14B: 40 query heads on 8 kv heads).  The kernel above multiplies the probabilities with V on the vector ALU (G x 8
 // FMAs per token and lane), which with 8 heads per kv head costs as much as fetching the cache: cache-resident it
 // still takes 62 of the 102 us it needs from HBM at 64 sequences x 8 kv heads x 2060 tokens.  Here a wave takes
 // tiles of 32 tokens:
@@ -633,14 +635,17 @@ template <typename T, int G, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_tr_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, const int32_t* __restrict__ context_lens, uint16_t* __restrict__ out,
-    float* __restrict__ partial, int nkv, int block_size, int max_blocks, int num_blocks, int nsplit, float scale) {
+    float* __restrict__ partial, int nkv, int block_size, int max_blocks, int num_blocks, int nsplit, float scale,
+    int heads_per_kv) {
     constexpr int HD = 128, TT = 32, VBYTES = TT * HD * 2, WBYTES = 2 * VBYTES;   // a wave's K tile and V tile
-    static_assert(G == 1 || G == 2 || G == 4 || G == 8, "query heads per kv head");
-    static_assert(G * (HD + 2) * 4 <= WBYTES, "the per-wave results reuse the wave's tiles");
+    constexpr int GA = G ? G : 16;                                                // rows of the per-wave result
+    static_assert(G >= 0 && G <= 16, "query heads per kv head");
+    static_assert(GA * (HD + 2) * 4 <= WBYTES, "the per-wave results reuse the wave's tiles");
+    const int Gv = G ? G : heads_per_kv;
     const int sp = blockIdx.x % nsplit;
     const int kvh = (blockIdx.x / nsplit) % nkv;
     const int b = blockIdx.x / (nsplit * nkv);
-    const int nh = nkv * G;
+    const int nh = nkv * Gv;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lo = lane & 15, hi = lane >> 4;
 
@@ -652,14 +657,14 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_tr_kernel(
     __shared__ __attribute__((aligned(1024))) unsigned char s_raw[WAVES * WBYTES];
     unsigned char* kt = s_raw + wave * WBYTES;                       // this wave's K tile [32 tokens][256 B, rotated]
     unsigned char* vt = kt + VBYTES;                                 // and its V tile
-    float (*s_acc)[G][HD + 2] = reinterpret_cast<float (*)[G][HD + 2]>(s_raw);   // after the loop
+    float (*s_acc)[GA][HD + 2] = reinterpret_cast<float (*)[GA][HD + 2]>(s_raw);   // after the loop
 
     u32x4 bq[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         bq[i] = u32x4{0u, 0u, 0u, 0u};
-        if (lo < G)
-            bq[i] = *reinterpret_cast<const u32x4*>(q + ((int64_t)b * nh + kvh * G + lo) * HD + 32 * i + 8 * hi);
+        if (lo < Gv)
+            bq[i] = *reinterpret_cast<const u32x4*>(q + ((int64_t)b * nh + kvh * Gv + lo) * HD + 32 * i + 8 * hi);
     }
     const float sc = scale * kLog2e;
     float m = kNegBig, lpart = 0.f;
@@ -759,7 +764,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_tr_kernel(
     lpart += __shfl_xor(lpart, 16);
     lpart += __shfl_xor(lpart, 32);
     __syncthreads();   // every wave is done with its tiles: the area now holds the per-wave results
-    if (lo < G) {
+    if (lo < Gv) {
 #pragma unroll
         for (int cb = 0; cb < 8; ++cb)
 #pragma unroll
@@ -770,7 +775,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_tr_kernel(
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < G * HD; idx += 64 * WAVES) {
+    for (int idx = threadIdx.x; idx < Gv * HD; idx += 64 * WAVES) {
         const int g = idx / HD, d = idx % HD;
         float mn = kNegBig;
 #pragma unroll
@@ -782,7 +787,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_tr_kernel(
             lt += s_acc[w][g][HD + 1] * c;
             at += s_acc[w][g][d] * c;
         }
-        const int64_t head = (int64_t)b * nh + kvh * G + g;
+        const int64_t head = (int64_t)b * nh + kvh * Gv + g;
         if (nsplit == 1) {
             out[head * HD + d] = T::from_f32(lt > 0.f ? at / lt : 0.f);
         } else {
@@ -899,7 +904,10 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // (bf16, against them: 128 sequences x 8 kv heads x 1024 tokens 120 -> 102 us, 32 x 8 x 512 23.2 -> 19.9, 1 x 8 x 8000
 // 31.7 -> 24.6, 64 x 8 x 2060 the same 102 us = 5.3 TB/s; at 4 and 2 heads per kv head it measured equal or slower:
 // 16 x 8 x 4000 at 4 heads 52.6 -> 55.0 us, the Qwen3-0.6B decode step 1.615 -> 1.673 ms).
-bool attn_tr(int G, int64_t head_dim, int64_t block_size) { return G == 8 && head_dim == 128 && block_size % 32 == 0; }
+// Head ratios other than 1, 2, 4 and 8 (up to 16) have no other kernel and take it as well.
+bool attn_tr(int G, int64_t head_dim, int64_t block_size) {
+    return (G == 8 || (G != 1 && G != 2 && G != 4 && G >= 1 && G <= 16)) && head_dim == 128 && block_size % 32 == 0;
+}
 int attn_waves(int G, bool tr) { return tr ? 4 : (G <= 2 ? 16 : (G <= 4 ? 8 : 4)); }
 
 // Context splits of a (sequence, kv head) pair.  From sweeps at 1..128 sequences x 512..8000 tokens (bf16, caches
@@ -925,7 +933,7 @@ void launch_attn(const void* q, const void* kc, const void* vc, const int32_t* t
         if (attn_tr(G, HD, bs)) {
             paged_attn_decode_tr_kernel<T, G, 4><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(256), 0, st>>>(
                 (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, table, ctx, (uint16_t*)out, partial, nkv,
-                bs, max_blocks, num_blocks, nsplit, scale);
+                bs, max_blocks, num_blocks, nsplit, scale, G);
             if (nsplit > 1)
                 paged_attn_merge_kernel<T, HD><<<dim3((unsigned)(batch * nkv * G)), dim3(HD), 0, st>>>(
                     partial, (uint16_t*)out, nsplit);
@@ -964,7 +972,19 @@ int launch_attn_g(int G, const void* q, const void* kc, const void* vc, const in
         NQ_CASE(1) NQ_CASE(2) NQ_CASE(4) NQ_CASE(8)
 #undef NQ_CASE
     }
-    set_error("nq_paged_attention_decode: query heads per kv head must be 1, 2, 4 or 8, got %d", G);
+    if constexpr (HD == 128) {
+        if (attn_tr(G, HD, bs)) {   // any other ratio up to 16: the matrix-core kernel with the count at run time
+            paged_attn_decode_tr_kernel<T, 0, 4><<<dim3((unsigned)(batch * nkv * nsplit)), dim3(256), 0, st>>>(
+                (const uint16_t*)q, (const uint16_t*)kc, (const uint16_t*)vc, table, ctx, (uint16_t*)out, partial, nkv,
+                bs, max_blocks, num_blocks, nsplit, scale, G);
+            if (nsplit > 1)
+                paged_attn_merge_kernel<T, HD><<<dim3((unsigned)(batch * nkv * G)), dim3(HD), 0, st>>>(
+                    partial, (uint16_t*)out, nsplit);
+            return AWQ_OK;
+        }
+    }
+    set_error("nq_paged_attention_decode: query heads per kv head must be 1, 2, 4 or 8 (or, with head_dim 128 and a "
+              "block size that is a multiple of 32, any count up to 16), got %d", G);
     return AWQ_ERR_UNSUPPORTED;
 }
 
@@ -1136,7 +1156,7 @@ extern "C" size_t nq_paged_attention_workspace_bytes(int64_t batch, int64_t num_
     // the block size decides the kernel and with it the split count: room for either
     const int G = (int)(num_heads / num_kv_heads);
     int s = pick_splits(batch, num_kv_heads, max_context, G, false);
-    if (G == 8 && head_dim == 128) s = std::max(s, pick_splits(batch, num_kv_heads, max_context, G, true));
+    if (attn_tr(G, head_dim, 32)) s = std::max(s, pick_splits(batch, num_kv_heads, max_context, G, true));
     return s > 1 ? (size_t)(batch * num_heads * s * (head_dim + 2)) * sizeof(float) : 0;
 }
 

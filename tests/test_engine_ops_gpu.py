@@ -172,6 +172,9 @@ def _attn_ref(q, kc, vc, table, ctx, scale):
     (4, 64, 8, 128, 64, 40),      # 8 per kv head, long context, context splits
     (9, 16, 2, 128, 16, 11),      # 8 per kv head, one tile per block
     (3, 8, 1, 128, 24, 5),        # 8 per kv head, block size not a multiple of the tile: the general kernel
+    (6, 40, 8, 128, 64, 5),       # 5 per kv head (Qwen3-14B): the matrix-core kernel with the ratio at run time
+    (3, 12, 4, 128, 32, 7),       # 3 per kv head
+    (2, 16, 1, 128, 64, 4),       # 16 per kv head
 ])
 def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
     from nanoquantization_amd.engine import ops

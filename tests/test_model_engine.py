@@ -318,6 +318,26 @@ def test_engine_qwen3_32b_widths_batch_64_context_2048():
 
 
 @pytest.mark.gpu
+def test_engine_qwen3_14b_widths_five_heads_per_kv_head():
+    """Two blocks at the Qwen3-14B widths (hidden 5120, 40 query / 8 kv heads, intermediate 17408): five query heads
+    per kv head, a ratio only the matrix-core attention kernel takes (the count at run time), at 16 and at 64 rows."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+    print("engine: Qwen3-14B widths, 2 layers", flush=True)
+    cfg = dict(QWEN3_32B, total_num_heads=40, intermediate_size=17408, num_hidden_layers=2,
+               max_position_embeddings=1024, vocab_size=32000)
+    model = random_awq_qwen3(cfg, seed=51, std=0.02)
+    torch.manual_seed(52)
+    plen, new = 150, 4
+    for B in (16, 64):
+        prompts = torch.randint(0, cfg["vocab_size"], (B, plen)).tolist()
+        eng = LLMEngine(model, max_batch=B, max_seq_len=plen + 42, block_size=64, use_graph=True)
+        got = eng.generate(prompts, new)
+        assert len(got) == B and all(len(g) == new for g in got)
+        _teacher_forced_check(model, prompts, got, rows=[0, B // 3, B - 1])
+
+
+@pytest.mark.gpu
 def test_engine_qwen3_8b_widths_batch_64():
     """Two blocks at the Qwen3-8B widths (hidden 4096, 32 query / 8 kv heads, intermediate 12288) with 64 rows: here
     only down_proj (12288 x 4096) and gate|up have a K-split shared-chunk plan, so the decode step mixes the routes --
