@@ -1993,9 +1993,10 @@ static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, 
 // 46.6).
 // 33..64 rows: the same with four m-tiles, 244 registers a wave, so two workgroups a CU and one wave of each per SIMD;
 // the kernel then takes a chunk step by step.  From 45 M weights (40 M above 48 rows, where the row blocks are four:
-// 8192 x 5120 at 64 rows 23.5 -> 22.3 us, at 48 rows 19.2 against 21.7) and 3584 columns on, any N; plan B with up to
-// 12 chunks a split (with 16, 4096 x 28672 runs 38.6 us in 224 workgroups and 36.9 in 448 of 8 chunks; 25600 x 5120
-// at 40 rows 37.6 us in 12 splits of 17 chunks, 33.7 in 25 of 8).  Against the
+// 8192 x 5120 at 64 rows 23.5 -> 22.3 us, at 48 rows 19.2 against 21.7), 3584 columns and K = 3584 on (2560 x 19456 at
+// 40 rows 23.4 us against 19.1 in row blocks), any N; plan B with up to 11 chunks a split (with 16, 4096 x 28672
+// runs 38.6 us in 224 workgroups and 36.9 in 448 of 8 chunks; 25600 x 5120 at 40 rows 37.6 us in 12 splits of 17
+// chunks, 33.7 in 25 of 8; 17408 x 5120 at 40 rows 29.8 us in 12 splits of 12, 27.7 in 23 of 6).  Against the
 // 512-column form or the one-tile kernel's row blocks at 64 rows: 8192 x 8192 30.4 -> 26.1 us, 5120 x 10240 27.8 ->
 // 23.7, 13824 x 5120 31.4 -> 27.2, 18944 x 3584 31.6 -> 27.7, 8192 x 10240 33.8 -> 29.9, 4096 x 12288 25.9 -> 23.5,
 // 5120 x 17408 34.1 -> 32.5, 4096 x 28672 39.6 -> 36.9, 5120 x 25600 40.8 -> 39.1, 5120 x 51200 70.7 -> 65.6; at 40
@@ -2004,12 +2005,14 @@ static int64_t pick_one_m_tile(int64_t M, int64_t N, int64_t K, int64_t chunks, 
 static int64_t pick_shared_256(int64_t M, int64_t N, int64_t K, int64_t chunks, int* variant) {
     if (M > 64 || N % 256 != 0 || chunks < 8) return 0;
     const bool four = M > 32;   // m-tiles: four, else two
-    if (four ? (N < 3584 || K * N < (M > 48 ? 40000000ll : 45000000ll)) : (N < 4096 || N >= 28672 || K * N < 48000000ll)) return 0;
+    if (four ? (N < 3584 || chunks < 28 || K * N < (M > 48 ? 40000000ll : 45000000ll))
+             : (N < 4096 || N >= 28672 || K * N < 48000000ll))
+        return 0;
     auto normalised = [&](int64_t c) { return cdiv(chunks, cdiv(chunks, c)); };
     const int64_t groups = N / 256;
     int64_t sb = 256 / groups;
     if (sb > chunks / 4) sb = chunks / 4;
-    if (sb >= 2 && normalised(sb) * groups >= (four ? 216 : 218) && (!four || cdiv(chunks, sb) <= 12)) {
+    if (sb >= 2 && normalised(sb) * groups >= (four ? 216 : 218) && (!four || cdiv(chunks, sb) <= 11)) {
         sb = normalised(sb);
         *variant = four ? kWide2D2M4 : (cdiv(chunks, sb) >= 6 ? kWide2D3M2 : kWide2D2M2);
         return sb;
@@ -2115,10 +2118,11 @@ static void pick_gemv(int64_t M, int64_t N, int64_t K, int64_t g, int* variant, 
             // adds its tail (2048 x 2048 at 128 rows: 8.6 us unsplit, 9.4 in two)
             const int64_t cap = M > 64 && wgs >= 64 ? 1 : (chunks / 4 > 1 ? chunks / 4 : 1);
             // From 17 rows on, weights under 32 Mi elements (16 MB packed: the linears of Qwen3-1.7B / 4B) are not
-            // streaming-bound, and with 150 workgroups or more any split only adds its tail -- 2560 x 9728 at 64 rows
+            // streaming-bound, and with 144 workgroups or more any split only adds its tail -- 2560 x 9728 at 64 rows
             // 27.2 us in five splits, 16.8 unsplit (304 workgroups); at 32 rows 16.2 -> 13.1; 2048 x 6144 at 64 rows
-            // 12.3 -> 9.7; likewise four row blocks of 128 tiles or more: 2560 x 19456 at 64 rows 33.4 -> 23.4.
-            const bool unsplit = row_blocks >= 2 && wgs >= 150 &&
+            // 12.3 -> 9.7, at 48 rows (144 workgroups) 11.9 -> 10.2; likewise four row blocks of 128 tiles or more:
+            // 2560 x 19456 at 64 rows 33.4 -> 23.4.
+            const bool unsplit = row_blocks >= 2 && wgs >= 144 &&
                                  (K * N < (32ll << 20) || (row_blocks >= 4 && wgs >= 512));
             int64_t s0 = wgs < 200 ? cdiv(200, wgs) : 1;
             if (s0 > cap) s0 = cap;

@@ -183,7 +183,8 @@ def test_dispatch_plans_are_consistent():
                     if cols == 256 and M <= 32:
                         assert (5120 if one else 4096) <= N < 28672
                     if name == "wide2d2m4":                               # plan B from 92 % of the CUs, else about 500
-                        assert N >= 3584 and ((216 <= wgs <= 256 and cps <= 12) or wgs > 256 or 512 // (N // 256) >= chunks // 4)
+                        assert N >= 3584 and chunks >= 28
+                        assert (216 <= wgs <= 256 and cps <= 11) or wgs > 256 or 512 // (N // 256) >= chunks // 4
                 if not staged_ok:
                     assert not name.startswith(("dma", "wide"))
                 if g == 128:   # awq_gemv_workspace_bytes takes no group size: it must cover this plan
