@@ -83,3 +83,28 @@ def test_forward_empty_and_boundary_row_counts(bias):
         ref = o.linear_fp32(to_bits(x), qw, qz, qs, "bf16", b)
         err = o.max_rel_err(m(x).float().cpu().numpy(), ref)
         assert err <= 6e-3, (M, err)
+
+
+@pytest.mark.parametrize("K,N,g", [(1024, 151936, 128), (65536, 1024, 128), (128, 8, 128), (64, 8, 64), (32, 4096, 32),
+                                   (256, 262144, 128)])
+def test_linear_extreme_widths_default_dispatch(K, N, g):
+    """Widths at the ends of what the entry point takes -- a vocabulary-sized N (a quantised lm_head), one packed word
+    of N, one group of K, a K of 512 chunks -- at row counts on both sides of every regime switch, through the default
+    dispatch.  Reference: x @ awq_dequantize(...) in fp32 on the device (the dequantise kernel is bit-exact against the
+    oracle, tests/test_dequant_gpu.py; the CPU oracle would need minutes at these sizes).  Bound: the 1e-2 of the
+    task, and the rounding-only bound the other GEMV tests use."""
+    from nanoquantization_amd.layers.gemm import _linear
+    torch.manual_seed(K + N)
+    for tdt, tight in ((torch.float16, 1.5e-3), (torch.bfloat16, 6e-3)):
+        qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32, device="cuda")
+        qz = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // g, N // 8), dtype=torch.int32, device="cuda")
+        qs = (torch.rand(K // g, N, device="cuda") * 0.02 + 0.001).to(tdt)
+        W = nq.awq_dequantize(qw, qs, qz).float()
+        for M in (1, 5, 16, 17, 64, 65, 129):
+            print(f"extreme widths K={K} N={N} g={g} {tdt} M={M}", flush=True)
+            x = (torch.randn(M, K, device="cuda") * 0.5).to(tdt)
+            y = _linear("awq_linear", x, qw, qs, qz, None)
+            ref = x.float() @ W
+            err = ((y.float() - ref).abs().max() / ref.abs().max()).item()
+            assert y.shape == (M, N) and y.dtype == tdt and err <= tight, (M, err)
+        del W
