@@ -247,6 +247,12 @@ def test_dispatch_plans_are_consistent():
     assert gemv_names[_plan(L.awq_gemv_plan, 48, 5120, 8192, 128)[1]] == "dma1x4"      # below 45 M weights: row blocks
     rc, v, s = _plan(L.awq_gemv_plan, 64, 5120, 8192, 128)       # from 40 M at 49..64 rows (four row blocks otherwise)
     assert rc == 0 and gemv_names[v] == "wide2d2m4" and s == 11
+    rc, v, s = _plan(L.awq_gemv_plan, 48, 19456, 2560, 128)      # 20 chunks of K: four row blocks, and unsplit at 456 workgroups
+    assert rc == 0 and gemv_names[v] == "dma1x4" and s == 1
+    rc, v, s = _plan(L.awq_gemv_plan, 48, 6144, 2048, 128)       # a small weight in 144 workgroups: unsplit as well
+    assert rc == 0 and gemv_names[v] == "dma1x4" and s == 1
+    rc, v, s = _plan(L.awq_gemv_plan, 40, 5120, 17408, 128)      # 12 chunks a split would fill the CUs: 23 splits of 6 instead
+    assert rc == 0 and gemv_names[v] == "wide2d2m4" and s == 23
     assert gemv_names[_plan(L.awq_gemv_plan, 1, 4096, 16384, 128)[1]] == "dma1x8"      # narrow weights: the one-tile kernel
     assert gemv_names[_plan(L.awq_gemv_plan, 8, 12288, 4096, 128)[1]] == "dma1x4"      # and small ones
     # narrow-tile GEMM (65..128 rows): the split fills whole rounds of the 512 resident workgroups (two per CU), so
