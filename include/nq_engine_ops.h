@@ -64,7 +64,7 @@ size_t nq_paged_attention_workspace_bytes(int64_t batch, int64_t num_heads, int6
  * of block block_table[b, t / block_size] in k_cache / v_cache
  * [num_blocks, num_kv_heads, block_size, head_dim]; query head h reads kv head
  * h / (num_heads / num_kv_heads).  q, out: [batch, num_heads, head_dim].  head_dim 64 or 128,
- * num_heads / num_kv_heads in {1, 2, 4, 8} -- with head_dim 128 and block_size % 32 == 0 any ratio up to 16 (Qwen3-14B
+ * num_heads / num_kv_heads in {1, 2, 4, 8} -- with head_dim 128 and block_size % 16 == 0 any ratio up to 16 (Qwen3-14B
  * has 5); block indices are clamped to the cache.
  * F.scaled_dot_product_attention(..., enable_gqa) of Qwen3QuantizedAttention.forward,
  * nanoquantization/models/qwen3_quantized.py:94-99, restricted to the last query position. */

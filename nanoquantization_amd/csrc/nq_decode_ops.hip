@@ -606,7 +606,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_mfma_kernel(
     }
 }
 
-// Both products on the matrix cores, for 128 head dims and block sizes that are multiples of 32.  The query heads of
+// Both products on the matrix cores, for 128 head dims and block sizes that are multiples of 16.  The query heads of
 // a kv head are columns of a 16-column MFMA tile, so any count up to 16 fits: G > 0 fixes it at compile time (the
 // launcher uses 8), G = 0 takes it from `heads_per_kv` -- the route of the head ratios the other kernels have no
 // instantiation for (Qwen3-14B: 40 query heads on 8 kv heads).  The kernel above multiplies the probabilities with V on the vector ALU (G x 8
@@ -686,17 +686,29 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attn_decode_tr_kernel(
         blk = blk < 0 ? 0 : (blk >= num_blocks ? num_blocks - 1 : blk);
         const int64_t base = (((int64_t)blk * nkv + kvh) * block_size + tb % block_size) * HD;
         const int last = min(TT, t1 - tb) - 1;                    // last valid row of the tile
+        // rows 16..31: in the same cache block 16 rows on, or (block sizes that are odd multiples of 16) at the start
+        // of the next one; where the context ends before them, the first 16 rows stand in (their scores are replaced)
+        int64_t base16 = base + 16 * HD;
+        if (tb % block_size + 16 >= block_size) {                 // wave-uniform
+            base16 = base;
+            if (tb + 16 < t1) {
+                int blk1 = table[(tb + 16) / block_size];
+                blk1 = blk1 < 0 ? 0 : (blk1 >= num_blocks ? num_blocks - 1 : blk1);
+                base16 = ((int64_t)blk1 * nkv + kvh) * block_size * HD;
+            }
+        }
 #pragma unroll
         for (int k = 0; k < 8; ++k) {   // rows past the context are fetched as they are: their scores are replaced
             const int r = 4 * k + dma_row;
-            const uint16_t* src = k_cache + base + (int64_t)r * HD + 8 * ((dma_piece - r) & 15);
+            const uint16_t* src = k_cache + (k < 4 ? base : base16) + (int64_t)(r & 15) * HD + 8 * ((dma_piece - r) & 15);
             __builtin_amdgcn_global_load_lds(NQ_GPTR(src), NQ_LPTR(kt + k * 1024), 16, 0, 0);
         }
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const int r = 4 * k + dma_row;
             const int w = ((dma_piece >> 1) - r) & 7;
-            const uint16_t* src = v_cache + base + (int64_t)min(r, last) * HD + 16 * w + 8 * (dma_piece & 1);
+            const int rr = min(r, last);
+            const uint16_t* src = v_cache + (rr < 16 ? base : base16) + (int64_t)(rr & 15) * HD + 16 * w + 8 * (dma_piece & 1);
             __builtin_amdgcn_global_load_lds(NQ_GPTR(src), NQ_LPTR(vt + k * 1024), 16, 0, 0);
         }
         // the K tile has landed: a wave's loads return in order, the eight of the V tile are the newest
@@ -899,14 +911,14 @@ int bad(const char* fn, const char* what) {
 }
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// The kernel with both products on the matrix cores takes 128 head dims and block sizes that are multiples of 32; it
+// The kernel with both products on the matrix cores takes 128 head dims and block sizes that are multiples of 16; it
 // is used at 8 query heads per kv head, where the vector-ALU value product of the other kernels costs the most
 // (bf16, against them: 128 sequences x 8 kv heads x 1024 tokens 120 -> 102 us, 32 x 8 x 512 23.2 -> 19.9, 1 x 8 x 8000
 // 31.7 -> 24.6, 64 x 8 x 2060 the same 102 us = 5.3 TB/s; at 4 and 2 heads per kv head it measured equal or slower:
 // 16 x 8 x 4000 at 4 heads 52.6 -> 55.0 us, the Qwen3-0.6B decode step 1.615 -> 1.673 ms).
 // Head ratios other than 1, 2, 4 and 8 (up to 16) have no other kernel and take it as well.
 bool attn_tr(int G, int64_t head_dim, int64_t block_size) {
-    return (G == 8 || (G != 1 && G != 2 && G != 4 && G >= 1 && G <= 16)) && head_dim == 128 && block_size % 32 == 0;
+    return (G == 8 || (G != 1 && G != 2 && G != 4 && G >= 1 && G <= 16)) && head_dim == 128 && block_size % 16 == 0;
 }
 int attn_waves(int G, bool tr) { return tr ? 4 : (G <= 2 ? 16 : (G <= 4 ? 8 : 4)); }
 
@@ -984,7 +996,7 @@ int launch_attn_g(int G, const void* q, const void* kc, const void* vc, const in
         }
     }
     set_error("nq_paged_attention_decode: query heads per kv head must be 1, 2, 4 or 8 (or, with head_dim 128 and a "
-              "block size that is a multiple of 32, any count up to 16), got %d", G);
+              "block size that is a multiple of 16, any count up to 16), got %d", G);
     return AWQ_ERR_UNSUPPORTED;
 }
 

@@ -175,6 +175,9 @@ def _attn_ref(q, kc, vc, table, ctx, scale):
     (6, 40, 8, 128, 64, 5),       # 5 per kv head (Qwen3-14B): the matrix-core kernel with the ratio at run time
     (3, 12, 4, 128, 32, 7),       # 3 per kv head
     (2, 16, 1, 128, 64, 4),       # 16 per kv head
+    (5, 20, 4, 128, 16, 9),       # 5 per kv head, 16-token blocks: every tile of 32 tokens spans two blocks
+    (4, 24, 4, 128, 48, 6),       # 6 per kv head, 48-token blocks: every third tile does
+    (7, 64, 8, 128, 80, 5),       # 8 per kv head, 80-token blocks
 ])
 def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
     from nanoquantization_amd.engine import ops
@@ -195,12 +198,12 @@ def test_paged_attention_decode(dtype, B, nh, nkv, hd, bs, max_blocks):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv", [(16, 8), (64, 8), (16, 4)])
-def test_paged_attention_ignores_rows_past_the_context(dtype, nh, nkv):
+@pytest.mark.parametrize("nh,nkv,bs", [(16, 8, 32), (64, 8, 32), (16, 4, 32), (40, 8, 32), (64, 8, 16), (40, 8, 48)])
+def test_paged_attention_ignores_rows_past_the_context(dtype, nh, nkv, bs):
     """Cache rows past a sequence's context (and unused blocks) hold whatever was there before: NaNs planted there
     must not reach the output."""
     from nanoquantization_amd.engine import ops
-    B, hd, bs, max_blocks = 6, 128, 32, 5
+    B, hd, max_blocks = 6, 128, -(-160 // bs)
     g = torch.Generator().manual_seed(nh)
     nb = B * max_blocks + 2
     table = torch.randperm(nb, generator=g)[: B * max_blocks].view(B, max_blocks).to(torch.int32)
@@ -223,7 +226,7 @@ def test_paged_attention_ignores_rows_past_the_context(dtype, nh, nkv):
 def test_paged_attention_rejects_unsupported():
     from nanoquantization_amd import _lib
     from nanoquantization_amd.engine import ops
-    kc = torch.zeros(4, 1, 16, 128, dtype=torch.bfloat16, device="cuda")
+    kc = torch.zeros(4, 1, 24, 128, dtype=torch.bfloat16, device="cuda")   # 3 per kv head needs 16 | block size
     q = torch.zeros(1, 3, 128, dtype=torch.bfloat16, device="cuda")
     tb = torch.zeros(1, 2, dtype=torch.int32, device="cuda")
     cx = torch.ones(1, dtype=torch.int32, device="cuda")
