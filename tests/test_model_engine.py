@@ -320,7 +320,8 @@ def test_engine_qwen3_32b_widths_batch_64_context_2048():
 @pytest.mark.gpu
 def test_engine_qwen3_14b_widths_five_heads_per_kv_head():
     """Two blocks at the Qwen3-14B widths (hidden 5120, 40 query / 8 kv heads, intermediate 17408): five query heads
-    per kv head, a ratio only the matrix-core attention kernel takes (the count at run time), at 16 and at 64 rows."""
+    per kv head, a ratio only the matrix-core attention kernel takes (the count at run time), at 16 and at 64 rows --
+    the 16 rows on 16-token cache blocks, where every 32-token tile of the kernel spans two table entries."""
     from nanoquantization_amd.engine import LLMEngine
     from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
     print("engine: Qwen3-14B widths, 2 layers", flush=True)
@@ -329,9 +330,9 @@ def test_engine_qwen3_14b_widths_five_heads_per_kv_head():
     model = random_awq_qwen3(cfg, seed=51, std=0.02)
     torch.manual_seed(52)
     plen, new = 150, 4
-    for B in (16, 64):
+    for B, bs in ((16, 16), (64, 64)):
         prompts = torch.randint(0, cfg["vocab_size"], (B, plen)).tolist()
-        eng = LLMEngine(model, max_batch=B, max_seq_len=plen + 42, block_size=64, use_graph=True)
+        eng = LLMEngine(model, max_batch=B, max_seq_len=plen + 42, block_size=bs, use_graph=True)
         got = eng.generate(prompts, new)
         assert len(got) == B and all(len(g) == new for g in got)
         _teacher_forced_check(model, prompts, got, rows=[0, B // 3, B - 1])
