@@ -348,3 +348,13 @@ def test_superseded_workspaces_stay_alive():
     assert _lib.workspace(dev, key_stream, 0) is None
     del _lib._workspaces[(0, key_stream)]
     _lib._retired_workspaces.pop()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits non-zero before touching a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=300)
+    assert p.returncode != 0 and "one GPU" in p.stderr and p.stdout.strip() == ""
