@@ -298,6 +298,26 @@ def test_engine_full_qwen3_0p6b_architecture_batch_32():
 
 
 @pytest.mark.gpu
+def test_engine_full_qwen3_0p6b_architecture_full_length():
+    """The same architecture at the full length of the small end-to-end configuration: 32 sequences, 512-token
+    prompts, 256 new tokens each (contexts of 512..767 tokens, 8..12 cache blocks per sequence, 256 replays of the
+    captured decode step), against the full-recompute forward on a sample of the sequences."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_0P6B, random_awq_qwen3
+    print("engine: Qwen3-0.6B architecture, 28 layers, batch 32, 512 + 256 tokens", flush=True)
+    cfg = dict(QWEN3_0P6B, max_position_embeddings=1024)
+    model = random_awq_qwen3(cfg, seed=25, std=0.02)
+    torch.manual_seed(26)
+    plen, new = 512, 256
+    prompts = torch.randint(0, cfg["vocab_size"], (32, plen)).tolist()
+    eng = LLMEngine(model, max_batch=32, max_seq_len=plen + new, block_size=64, use_graph=True)
+    got = eng.generate(prompts, new)
+    assert len(got) == 32 and all(len(g) == new for g in got)
+    clear = _teacher_forced_check(model, prompts, got, rows=[0, 17, 31])
+    assert clear > 0.2, clear   # a good share of the steps has a clear winner: the exact comparison is not vacuous
+
+
+@pytest.mark.gpu
 def test_engine_qwen3_32b_widths_batch_64_context_2048():
     """Two blocks at the Qwen3-32B widths with 64 sequences of 2,048 cached tokens each: the decode shapes of the
     largest configuration (64-row GEMVs on the shared-chunk kernel, paged attention over 32 blocks per sequence with 8
