@@ -318,6 +318,30 @@ def test_engine_full_qwen3_0p6b_architecture_full_length():
 
 
 @pytest.mark.gpu
+@pytest.mark.timeout(600)
+def test_engine_full_qwen3_32b_architecture_batch_64_context_2048():
+    """The largest configuration at full depth: all 64 blocks of the Qwen3-32B architecture (16 GB of packed weights),
+    64 sequences of 2,048 prompt tokens (one 131,072-token prefill pass through the fused GEMM), then captured decode
+    steps at 64 rows over 2,048..2,050 cached tokens per sequence, against the full-recompute forward on two of the
+    sequences."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+    print("engine: Qwen3-32B architecture, 64 layers, batch 64, context 2048", flush=True)
+    cfg = dict(QWEN3_32B, max_position_embeddings=4096)
+    model = random_awq_qwen3(cfg, seed=27, std=0.02)
+    torch.manual_seed(28)
+    plen, new = 2048, 3
+    prompts = torch.randint(0, cfg["vocab_size"], (64, plen)).tolist()
+    eng = LLMEngine(model, max_batch=64, max_seq_len=plen + 64, block_size=64, use_graph=True)
+    assert eng.o_add_norm and eng.down_add_norm
+    got = eng.generate(prompts, new)
+    assert len(got) == 64 and all(len(g) == new for g in got)
+    _teacher_forced_check(model, prompts, got, rows=[0, 63])
+    del eng, model
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.gpu
 def test_engine_qwen3_32b_widths_batch_64_context_2048():
     """Two blocks at the Qwen3-32B widths with 64 sequences of 2,048 cached tokens each: the decode shapes of the
     largest configuration (64-row GEMVs on the shared-chunk kernel, paged attention over 32 blocks per sequence with 8
