@@ -256,10 +256,13 @@ def test_engine_norm_fused_decode_equals_separate_kernels():
     assert outs[0] == outs[1]
 
 
-def _teacher_forced_check(model, prompts, got, rows=None):
+def _teacher_forced_check(model, prompts, got, rows=None, gap_tol=2e-2):
     """The engine's own continuation pushed through the full-recompute forward (the reference semantics: no cache):
     every chosen token is that forward's argmax up to the 16-bit noise of a near-tie, and exactly it wherever the
-    logits are not near-tied.  `rows` limits the recompute to some sequences."""
+    logits are not near-tied.  `rows` limits the recompute to some sequences.  `gap_tol` (a fraction of the largest
+    logit) is the near-tie noise allowed; it grows with depth -- measured on these random-weight stacks at the
+    Qwen3-32B widths over 256 decoded tokens: at most 0.010 with 2 blocks, 0.015 with 8, 0.026 with 32, 0.066 with
+    64, while a token from a wrong cache row or position lands about 1.0 away."""
     rows = list(range(len(prompts))) if rows is None else rows
     plen = len(prompts[0])
     seqs = torch.tensor([prompts[r] + got[r] for r in rows], device="cuda")
@@ -269,9 +272,9 @@ def _teacher_forced_check(model, prompts, got, rows=None):
     chosen = torch.tensor([got[r] for r in rows], device="cuda")
     gap = logits.max(-1).values - logits.gather(-1, chosen.unsqueeze(-1)).squeeze(-1)
     scale = logits.abs().max().item()
-    assert gap.max().item() <= 2e-2 * scale, (gap.max().item(), scale)
+    assert gap.max().item() <= gap_tol * scale, (gap.max().item(), scale)
     top2 = logits.topk(2, dim=-1).values
-    clear = (top2[..., 0] - top2[..., 1]) > 4e-2 * scale
+    clear = (top2[..., 0] - top2[..., 1]) > 2 * gap_tol * scale
     assert torch.equal(chosen[clear], logits.argmax(-1)[clear])
     return clear.float().mean().item()
 
@@ -336,7 +339,7 @@ def test_engine_full_qwen3_32b_architecture_batch_64_context_2048():
     assert eng.o_add_norm and eng.down_add_norm
     got = eng.generate(prompts, new)
     assert len(got) == 64 and all(len(g) == new for g in got)
-    _teacher_forced_check(model, prompts, got, rows=[0, 63])
+    _teacher_forced_check(model, prompts, got, rows=[0, 21, 42, 63], gap_tol=0.12)   # 64 blocks deep
     del eng, model
     torch.cuda.empty_cache()
 
@@ -430,6 +433,36 @@ def test_engine_mixed_decode_and_long_prefill_qwen3_32b_widths():
     for (prompt, _), cont in zip(reqs, got):
         _teacher_forced_check(model, [prompt], [cont])
     assert eng.serve(reqs, batch_prefill=True, max_prefill_tokens=4 * P) == got
+
+
+@pytest.mark.gpu
+@pytest.mark.timeout(900)
+def test_engine_mixed_run_full_qwen3_32b_architecture():
+    """The mixed run of the largest configuration at full size: all 64 blocks of the Qwen3-32B architecture, one
+    serve() call with 64 requests of 2,048 prompt tokens and a 4,096-token request that is admitted when the first
+    row frees and prefilled between two decode steps of the other 63 rows.  Three of the continuations (a short
+    request, a long-running one and the 4,096-token one) are checked against the full-recompute forward."""
+    from nanoquantization_amd.engine import LLMEngine
+    from nanoquantization_amd.models.random_init import QWEN3_32B, random_awq_qwen3
+    print("engine: mixed decode + 4096-token prefill, Qwen3-32B architecture, 64 layers, batch 64", flush=True)
+    cfg = dict(QWEN3_32B, max_position_embeddings=8192)
+    model = random_awq_qwen3(cfg, seed=33, std=0.02)
+    rg = torch.Generator().manual_seed(34)
+    B, P, LONG = 64, 2048, 4096
+    prompts = torch.randint(0, cfg["vocab_size"], (B, P), generator=rg).tolist()
+    long_prompt = torch.randint(0, cfg["vocab_size"], (LONG,), generator=rg).tolist()
+    reqs = [(p, 3 if i == 0 else 8) for i, p in enumerate(prompts)] + [(long_prompt, 4)]
+    eng = LLMEngine(model, max_batch=B, max_seq_len=LONG + 64, block_size=64, use_graph=True)
+    st = {}
+    got = eng.serve(reqs, stats=st, batch_prefill=True, max_prefill_tokens=4 * P)
+    assert [len(g) for g in got] == [m for _, m in reqs]
+    long_pf = [p for p in st["prefill_log"] if p[0] == LONG]
+    assert len(long_pf) == 1 and long_pf[0][1] == 1, st["prefill_log"]
+    assert 1 <= long_pf[0][2] < st["decode_steps"], "the long prefill must sit between decode steps of the other rows"
+    for i in (0, 37, B):
+        _teacher_forced_check(model, [reqs[i][0]], [got[i]], gap_tol=0.12)   # 64 blocks deep
+    del eng, model
+    torch.cuda.empty_cache()
 
 
 @pytest.mark.gpu
