@@ -90,9 +90,13 @@ __device__ __forceinline__ void publish_f32(float* p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // 16-byte form of publish_f32.  The store is invisible to the compiler's wait-count
-// bookkeeping, which is why arrive_last waits for vmcnt = 0 explicitly.
+// bookkeeping, which is why arrive_last waits for vmcnt = 0 explicitly.  It is invisible to the compiler's
+// hazard pass as well: a store of more than 8 bytes reads its data registers up to two wait states after it
+// issues (gfx940 and later), and to the compiler those registers are free the moment the statement ends -- it
+// has put the next address computation into them one instruction later, and the store then wrote that value
+// now and then.  Hence the two wait states inside the statement.
 __device__ __forceinline__ void publish_f32x4(float* p, f32x4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ float fetch_f32(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -56,3 +56,12 @@ def test_staged_gemv_issues_each_load_once(tmp_path):
         else:
             per_site = 11 if re.search(r"ELb[01]ELi4E", name) else 12
         assert loads == 3 * per_site, (name, loads)
+    # The 16-byte publish store is issued as assembly (publish_f32x4), out of sight of the compiler's hazard pass: a
+    # store of more than 8 bytes reads its data registers up to two wait states after it issues (gfx940 and later),
+    # and the compiler, to which those registers are free at once, has put the next address computation into them one
+    # instruction later -- the store then published that value now and then.  Every such store carries its own two
+    # wait states.
+    stores = [m.end() for m in re.finditer(r"global_store_dwordx4 [^\n]* sc1\n", asm)]
+    assert len(stores) >= 50, len(stores)
+    for pos in stores:
+        assert re.match(r"\s*s_nop 1\b", asm[pos:pos + 40]), asm[pos - 80:pos + 80]
