@@ -65,3 +65,30 @@ def test_staged_gemv_issues_each_load_once(tmp_path):
     assert len(stores) >= 50, len(stores)
     for pos in stores:
         assert re.match(r"\s*s_nop 1\b", asm[pos:pos + 40]), asm[pos - 80:pos + 80]
+    # The 16-byte fetches of the exchange are assembly too (fetch_f32x4_nowait) and arrive behind the compiler's back:
+    # until the s_waitcnt vmcnt(0) that the code issues by hand, nothing may touch their destination registers -- a
+    # copy or a select placed there by the compiler would read what the registers held before.  (A linear scan of the
+    # listing: the fetch sites are straight-line code up to their wait.)
+    def vregs(text):
+        regs = set()
+        for m in re.finditer(r"\bv\[(\d+):(\d+)\]", text):
+            regs |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+        regs |= {int(m.group(1)) for m in re.finditer(r"\bv(\d+)\b", text)}
+        return regs
+    pending, fetches = set(), 0
+    for line in asm.split("\n"):
+        line = line.strip()
+        if not line or line[0] in ";." or line.endswith(":"):
+            continue
+        if line.startswith("s_waitcnt") and "vmcnt(0)" in line:
+            pending = set()
+            continue
+        m = re.match(r"global_load_dwordx4 (v\[\d+:\d+\]), (v\[\d+:\d+\]), off sc1", line)
+        if m:
+            assert not (vregs(m.group(2)) & pending), line
+            pending |= vregs(m.group(1))
+            fetches += 1
+            continue
+        if pending and line.split()[0].startswith(("v_", "ds_", "global_", "buffer_")):
+            assert not (vregs(line.split(None, 1)[1] if " " in line else "") & pending), line
+    assert fetches >= 500, fetches
