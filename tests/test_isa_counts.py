@@ -92,3 +92,30 @@ def test_staged_gemv_issues_each_load_once(tmp_path):
         if pending and line.split()[0].startswith(("v_", "ds_", "global_", "buffer_")):
             assert not (vregs(line.split(None, 1)[1] if " " in line else "") & pending), line
     assert fetches >= 500, fetches
+
+
+@pytest.mark.skipif(shutil.which(nq_build.HIPCC) is None and not os.path.exists(nq_build.HIPCC), reason="hipcc not found")
+def test_matrix_core_attention_counts_its_tile_loads(tmp_path):
+    """paged_attn_decode_tr_kernel brings a K tile and a V tile with eight load-to-LDS instructions each and reads the
+    K tile after s_waitcnt vmcnt(8): the eight loads of the V tile may still be on their way, nothing else.  Every
+    instantiation must issue exactly those sixteen loads, in one run with no other vector-memory instruction among them,
+    and wait by that count right behind them."""
+    src = os.path.join(nq_build.CSRC, "nq_decode_ops.hip")
+    out = tmp_path / "nq_decode_ops.s"
+    flags = [f for f in nq_build.FLAGS if f not in ("-shared", "-fPIC")]
+    cmd = [nq_build.HIPCC, *flags, *nq_build.EXTRA.get("nq_decode_ops.hip", []), "--cuda-device-only", "-S", src, "-o", str(out)]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-2000:]
+    asm = out.read_text()
+    names = re.findall(r"^(_ZN3awq\S*paged_attn_decode_tr_kernel[^:\s]*):", asm, re.M)
+    assert len(names) == 4, names             # 2 types x (8 heads per kv head at compile time, the count at run time)
+    for name in names:
+        begin = asm.index("\n" + name + ":")
+        body = asm[begin:asm.index(".Lfunc_end", begin)]
+        ins = [l.strip() for l in body.split("\n")]
+        ins = [l for l in ins if l and l[0] not in ";." and not l.endswith(":")]
+        dma = [k for k, l in enumerate(ins) if "global_load_lds_dwordx4" in l]
+        assert len(dma) == 16, (name, len(dma))
+        assert ins[dma[-1] + 1].startswith("s_waitcnt vmcnt(8)"), (name, ins[dma[-1] + 1])
+        between = [l for l in ins[dma[0]:dma[-1]] if l.split()[0].startswith(("global_", "buffer_", "flat_"))]
+        assert len(between) == 15, (name, between)
